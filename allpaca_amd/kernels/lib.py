@@ -1,0 +1,84 @@
+"""Loads the kernel libraries with ctypes and declares their entry points.
+
+Every entry point is `extern "C" int apc_*(..., hipStream_t)`; it returns 0, a
+hipError_t (> 0) or one of our own codes (< 0).  There is no fallback: if a
+library cannot be built or loaded the caller gets `KernelLibraryError`."""
+from __future__ import annotations
+
+import ctypes
+from typing import Dict
+
+from . import build as _build
+
+P, I, F, Z = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
+
+
+class KernelLibraryError(RuntimeError):
+    pass
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+# name -> argument types (the trailing stream included)
+SIGNATURES: Dict[str, Dict[str, list]] = {
+    "plain": {
+        "apc_embed_rows": [P, I, P, P, I, I, I, I, P],
+        "apc_gather_rows": [P, I, I, P, P, I, I, I, P],
+        "apc_rmsnorm_rows": [P, I, I, P, P, F, P, I, I, I, I, P],
+        "apc_add_into": [P, I, P, I, I, I, I, P],
+        "apc_silu_mul": [P, I, I, P, I, I, I, I, P],
+        "apc_rope_kv_write": [P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, I, P, I, I, P],
+        "apc_cast": [P, I, P, I, Z, P],
+        "apc_gemm_plain": [P, I, I, P, I, I, P, I, I, I, I, I, I, P],
+        "apc_paged_attention_plain": [P, I, I, I, P, I, I, I, I, I, I, P, I, I, P, I, P, P, I, F, P],
+        "apc_argmax_rows": [P, I, I, I, P, P],
+        "apc_sample_rows": [P, I, I, I, P, P, P, P, P, P],
+    },
+    "tuned": {
+        "apc_gemm_bf16": [P, I, P, I, P, I, I, I, I, I, I, P],
+        "apc_gemm_swiglu_bf16": [P, I, P, P, I, P, I, I, I, I, P],
+        "apc_skinny_gemm_bf16": [P, I, P, I, P, I, I, I, I, I, I, P],
+        "apc_skinny_swiglu_bf16": [P, I, P, P, I, P, I, I, I, I, P],
+        "apc_attention_prefill_bf16": [P, I, I, P, I, I, I, I, P, I, P, I, P, P, P, I, I, F, P],
+        "apc_attention_decode_bf16": [P, I, I, P, I, I, I, I, I, P, I, P, I, P, P, I, F, P, P, I, P],
+        "apc_attention_decode_workspace": [I, I, I, I],
+    },
+}
+
+_loaded: Dict[str, ctypes.CDLL] = {}
+
+ERRORS = {-1: "bad argument (shape or stride the kernel does not accept)", -2: "size not supported by this kernel"}
+
+
+def load(name: str) -> ctypes.CDLL:
+    """The library `name`, built first if it is missing or stale."""
+    lib = _loaded.get(name)
+    if lib is not None:
+        return lib
+    try:
+        path = _build.build(name)
+    except _build.KernelBuildError as e:
+        raise KernelLibraryError(f"kernel library '{name}' is not available: {e}") from None
+    try:
+        lib = ctypes.CDLL(path)
+    except OSError as e:
+        raise KernelLibraryError(f"cannot load {path}: {e}") from None
+    for fn, args in SIGNATURES[name].items():
+        try:
+            f = getattr(lib, fn)
+        except AttributeError:
+            raise KernelLibraryError(f"{path} lacks entry point {fn}") from None
+        f.argtypes = args
+        f.restype = I
+    _loaded[name] = lib
+    return lib
+
+
+def check(code: int, what: str) -> None:
+    if code == 0:
+        return
+    if code < 0:
+        raise KernelError(f"{what}: {ERRORS.get(code, f'error {code}')}")
+    raise KernelError(f"{what}: HIP error {code}")

@@ -1,0 +1,9 @@
+from .base import (ARRANGEMENTS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITION_ENCODINGS, FeedForward,
+                   FixedState, Mixer, Norm, PagedKV, Part, PositionEncoding, Runtime, build_part)
+from .spec import BlockSpec, ModelSpec, ParamSpec, PartSpec, PlanEntry
+from . import attention, block, embedding, mlp, norm, rope  # noqa: F401  (registers the built-in parts)
+from .block import Block
+
+__all__ = ["ARRANGEMENTS", "EMBEDDINGS", "FEED_FORWARDS", "HEADS", "MIXERS", "NORMS", "POSITION_ENCODINGS",
+           "FeedForward", "FixedState", "Mixer", "Norm", "PagedKV", "Part", "PositionEncoding", "Runtime",
+           "build_part", "BlockSpec", "ModelSpec", "ParamSpec", "PartSpec", "PlanEntry", "Block"]

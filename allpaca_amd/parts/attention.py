@@ -1,0 +1,77 @@
+"""Grouped-query attention over the paged cache.
+
+Per row: q = h Wq^T, k = h Wk^T, v = h Wv^T (no bias); q and k are turned by the
+position encoding before k is cached; query head j reads kv head j // (H/Hk);
+score = (q.k)/sqrt(d) on the finished dot product; keys at positions <= the
+row's own (of the last `window` positions if a window is set); softmax in
+32-bit; out = sum p V; residual += out Wo^T
+(crates/allpaca-core/src/model.rs:8528-8684, crates/allpaca-cpu/src/kernels.rs:293-356)."""
+from __future__ import annotations
+
+from typing import Dict, Mapping, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedKV, Runtime, build_part, to_device
+from .spec import ParamSpec, PartSpec
+
+
+@MIXERS.register("attention")
+class Attention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 position: Optional[PartSpec] = None, window: Optional[int] = None, scale: Optional[float] = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        self.D, self.H, self.Hk, self.d = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
+        self.window = int(window) if window else None
+        self.scale = float(scale) if scale is not None else None
+        self.position = build_part(POSITION_ENCODINGS, position) if position is not None else None
+        self.q_off, self.k_off, self.v_off = 0, self.H * self.d, (self.H + self.Hk) * self.d
+        self.qkv_width = (self.H + 2 * self.Hk) * self.d
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {
+            "q_proj.weight": ParamSpec((self.H * self.d, self.D)),
+            "k_proj.weight": ParamSpec((self.Hk * self.d, self.D)),
+            "v_proj.weight": ParamSpec((self.Hk * self.d, self.D)),
+            "o_proj.weight": ParamSpec((self.D, self.H * self.d)),
+        }
+
+    def cache_need(self):
+        return PagedKV(self.Hk, self.d, self.window)
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
+        self.rt = rt
+        parts = [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
+        dt = parts[0].dtype if all(p.dtype == parts[0].dtype for p in parts) else torch.float32
+        # one [(H + 2 Hk) d, D] matrix: a single product gives q, k and v of a row
+        self.w_qkv = torch.cat([to_device(p, rt, dt) for p in parts], dim=0).contiguous()
+        self.w_o = to_device(tensors["o_proj.weight"], rt)
+        if self.position is not None:
+            self.position.bind({}, rt)
+
+    def forward_add(self, h: torch.Tensor, step, cache, residual: torch.Tensor) -> None:
+        T = h.shape[0]
+        qkv = torch.empty((T, self.qkv_width), dtype=self.rt.dtype, device=h.device)
+        ops.linear(h, self.w_qkv, qkv)
+        rot, table = (0, None)
+        if self.position is not None:
+            fused = self.position.fused()
+            if fused is None:
+                self.position.apply(qkv, self.q_off, self.k_off, self.H, self.Hk, self.d, step.positions)
+            else:
+                rot, table = fused
+        kv = cache.kv if cache.writes else None
+        if kv is not None or rot:
+            ops.rope_kv_write(qkv, self.q_off, self.k_off, self.v_off, self.H, self.Hk, self.d, rot, table,
+                              step.positions, step.row_seg, cache.block_table, kv, cache.page_tokens)
+        attn = torch.empty((T, self.H * self.d), dtype=self.rt.dtype, device=h.device)
+        ops.paged_attention(qkv, self.q_off, attn, self.H, self.Hk, self.d, cache.kv, cache.page_tokens,
+                            cache.block_table, step, window=self.window or 0, scale=self.scale)
+        ops.linear(attn, self.w_o, residual, accumulate=True)
+
+    def forward(self, h, step, cache):
+        out = torch.zeros((h.shape[0], self.D), dtype=torch.float32, device=h.device)
+        self.forward_add(h, step, cache, out)
+        return out

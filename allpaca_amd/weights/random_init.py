@@ -1,0 +1,67 @@
+"""Seeded random weights for any described model, and a writer that turns a
+configuration and a seed into a model folder (config.json, model.safetensors).
+
+The reference's synthetic model draws uniform values from one generator in a
+fixed order (crates/allpaca-core/src/model.rs:5061-5125, 13369-13387); here each
+tensor has a generator of its own keyed by (seed, tensor name), so a tensor does
+not depend on which others exist or in which order they are made.  Matrices are
+N(0, std); norm weights are 1 + N(0, norm_std)."""
+from __future__ import annotations
+
+import hashlib
+import json
+import os
+from typing import Any, Dict, Mapping, Optional
+
+import torch
+
+from ..parts.spec import ParamSpec
+from .safetensors_io import write_safetensors
+
+
+def _tensor_seed(seed: int, name: str) -> int:
+    h = hashlib.sha256(f"{int(seed)}:{name}".encode()).digest()
+    return int.from_bytes(h[:8], "little") & 0x7FFFFFFFFFFFFFFF
+
+
+def random_tensors(specs: Mapping[str, ParamSpec], seed: int, dtype: torch.dtype, std: float = 0.02,
+                   norm_std: float = 0.0, device: str | torch.device = "cpu") -> Dict[str, torch.Tensor]:
+    """name -> tensor.  "compute" tensors get `dtype`; norm weights float32; integer tables zeros."""
+    out: Dict[str, torch.Tensor] = {}
+    dev = torch.device(device)
+    for name, ps in specs.items():
+        g = torch.Generator(device=dev)
+        g.manual_seed(_tensor_seed(seed, name))
+        if ps.store == "int32":
+            out[name] = torch.zeros(ps.shape, dtype=torch.int32, device=dev)
+        elif ps.store == "float32":
+            t = torch.ones(ps.shape, dtype=torch.float32, device=dev)
+            if norm_std:
+                t += norm_std * torch.randn(ps.shape, generator=g, dtype=torch.float32, device=dev)
+            out[name] = t
+        else:
+            t = torch.randn(ps.shape, generator=g, dtype=torch.float32, device=dev) * std
+            out[name] = t.to(dtype)
+    return out
+
+
+def write_model_folder(path: str, config_json: Mapping[str, Any], seed: int, dtype: torch.dtype = torch.float32,
+                       std: float = 0.02, norm_std: float = 0.0,
+                       overrides: Optional[Mapping[str, torch.Tensor]] = None) -> Dict[str, torch.Tensor]:
+    """Writes `path/config.json` and `path/model.safetensors` for the architecture that
+    `config_json` names.  `overrides` replaces tensors by name (tests plant values with it)."""
+    from ..models import DecoderModel, describe_model
+    _, cfg, spec = describe_model(config_json)
+    model = DecoderModel(spec)
+    tensors = random_tensors(model.param_specs(), seed, dtype, std, norm_std)
+    for name, t in (overrides or {}).items():
+        if name not in tensors:
+            raise KeyError(f"override {name!r} is not a tensor of this model")
+        if tuple(t.shape) != tuple(tensors[name].shape):
+            raise ValueError(f"override {name!r} has shape {tuple(t.shape)}, needs {tuple(tensors[name].shape)}")
+        tensors[name] = t.to(tensors[name].dtype)
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(dict(config_json), f, indent=1)
+    write_safetensors(os.path.join(path, "model.safetensors"), tensors, {"format": "pt", "seed": str(seed)})
+    return tensors

@@ -1,0 +1,188 @@
+"""The engine against the plain implementation, in float32 and in bfloat16, under
+every cutting of the work: each request alone and whole; most of it in one step
+and the last 32 tokens one by one; portions of changing size down to two tokens;
+mixed batches of up to four live requests with so few pages that they are used
+again; long decoding; the first tokens of a sequence."""
+import numpy as np
+import pytest
+import torch
+
+import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+TORCH = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def make_runner(folder, dtype, page_tokens=16, num_pages=64, max_requests=8, max_positions=None):
+    from allpaca_amd.engine.runner import ModelRunner
+    from allpaca_amd.models import load_model
+    cfg, model = load_model(folder, TORCH[dtype], "cuda:0", max_positions=max_positions)
+    return cfg, ModelRunner(model, page_tokens, num_pages, max_requests)
+
+
+def run_cut(runner, seq, tokens, cuts):
+    """Feeds `tokens` of one request in portions `cuts`, asking for every row's logits."""
+    from allpaca_amd.engine.batch import Entry
+    runner.admit(seq)
+    out, at = [], 0
+    for n in cuts:
+        lg = runner.step([Entry(seq, tokens[at:at + n], list(range(n)))])
+        out.append(lg.float().cpu().numpy())
+        at += n
+    runner.release(seq)
+    assert at == len(tokens)
+    return np.concatenate(out, axis=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("sharp", [False, True])
+def test_whole_tail_and_portions(name, dtype, sharp):
+    folder = H.model_folder(name, dtype, sharp)
+    cfg, runner = make_runner(folder, dtype)
+    lens = {"A": [1, 7, 16, 33, 100], "B": [2, 33, 150], "C": [5, 64, 129]}[name]
+    for i, n in enumerate(lens):
+        toks = H.random_tokens(cfg.vocab_size, n, seed=10 * i + 1)
+        want = H.oracle_logits(folder, toks)
+        whole = run_cut(runner, "w", toks, H.cut_whole(n))
+        H.assert_close(whole, want, dtype, f"{name} whole n={n}")
+        tail = run_cut(runner, "t", toks, H.cut_tail_decoded(n))
+        H.assert_close(tail, want, dtype, f"{name} tail-decoded n={n}")
+        for s in range(2):
+            cuts = H.cut_changing(n, seed=s)
+            got = run_cut(runner, "c", toks, cuts)
+            H.assert_close(got, want, dtype, f"{name} portions {cuts}")
+        if dtype == "float32":
+            # rows do not depend on the cutting at all: the products and the attention of a row
+            # add in an order that its position alone fixes
+            assert np.array_equal(whole, tail), f"{name} n={n}: whole and tail-decoded logits differ in bits"
+    runner.cache.check()
+    assert runner.cache.free_pages(0) == 64
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens_and_page_sizes(name, dtype):
+    """The first tokens of a sequence (positions 0, 1, 2), and the same logits for any page size."""
+    folder = H.model_folder(name, dtype, True)
+    toks = None
+    for page_tokens in (1, 2, 16, 64):
+        cfg, runner = make_runner(folder, dtype, page_tokens=page_tokens, num_pages=80)
+        toks = toks or H.random_tokens(cfg.vocab_size, 40, seed=3)
+        want = H.oracle_logits(folder, toks)
+        got = run_cut(runner, "p", toks, [1, 1, 1, 2, 35])
+        H.assert_close(got, want, dtype, f"{name} page_tokens={page_tokens}")
+
+
+def mixed_schedule(lengths, seed, live_max=4):
+    """Steps of a mixed batch: requests start at different times, advance by portions of changing
+    size or single tokens, some pause for a step, and end; at most `live_max` are live."""
+    rng = np.random.default_rng(seed)
+    todo = list(range(len(lengths)))
+    done_at = {i: 0 for i in todo}
+    live, steps = [], []
+    while todo or live:
+        while todo and len(live) < live_max and (not live or rng.random() < 0.6):
+            live.append(todo.pop(0))
+        entries, ends = [], []
+        for i in list(live):
+            left = lengths[i] - done_at[i]
+            if len(live) > 1 and rng.random() < 0.15:
+                continue  # left out of this step, goes on later
+            mode = rng.random()
+            n = 1 if mode < 0.45 else int(rng.choice([2, 2, 3, 5, 8, 13, 21, 40]))
+            n = min(n, left)
+            entries.append((i, done_at[i], n))
+            done_at[i] += n
+            if done_at[i] == lengths[i]:
+                ends.append(i)
+                live.remove(i)
+        if entries:
+            steps.append((entries, ends))
+    return steps
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_batches_with_page_reuse(name, dtype):
+    from allpaca_amd.engine.batch import Entry
+    folder = H.model_folder(name, dtype, True)
+    lengths = {"A": [33, 100, 16, 7, 64, 1, 90, 50], "B": [150, 2, 77, 40, 120, 33, 9], "C": [129, 64, 5, 200, 31, 90]}[name]
+    # pages for four live requests of the longest kind only: finished requests' pages must be used again
+    page_tokens = 16
+    worst = sorted(lengths)[-4:]
+    num_pages = sum(-(-n // page_tokens) for n in worst)
+    cfg, runner = make_runner(folder, dtype, page_tokens=page_tokens, num_pages=num_pages)
+    toks = [H.random_tokens(cfg.vocab_size, n, seed=100 + i) for i, n in enumerate(lengths)]
+    got = {i: [] for i in range(len(lengths))}
+    for entries, ends in mixed_schedule(lengths, seed=7):
+        batch = []
+        for i, at, n in entries:
+            if i not in runner.cache:
+                runner.admit(i)
+            batch.append(Entry(i, toks[i][at:at + n], list(range(n))))
+        lg = runner.step(batch).float().cpu().numpy()
+        row = 0
+        for i, at, n in entries:
+            got[i].append(lg[row:row + n])
+            row += n
+        for i in ends:
+            runner.release(i)
+        runner.cache.check()
+    assert runner.cache.paged_groups[0].pool.allocations > num_pages, "the schedule did not reuse pages"
+    for i, n in enumerate(lengths):
+        H.assert_close(np.concatenate(got[i]), H.oracle_logits(folder, toks[i]), dtype, f"{name} mixed request {i}")
+    assert runner.cache.free_pages(0) == num_pages
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding(dtype):
+    """A short prompt and 200 tokens decoded one by one, across many page edges."""
+    folder = H.model_folder("B", dtype, True)
+    cfg, runner = make_runner(folder, dtype, page_tokens=16, num_pages=20)
+    toks = H.random_tokens(cfg.vocab_size, 230, seed=5)
+    got = run_cut(runner, "d", toks, [30] + [1] * 200)
+    H.assert_close(got, H.oracle_logits(folder, toks), dtype, "long decoding")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_far_key_is_found(dtype):
+    """One early token is made to match the last query exactly with a large score in every head of layer 0;
+    the result must follow that token's value whatever stands between."""
+    import plain_llama as P
+    from allpaca_amd.weights import write_model_folder
+    import os
+    cfg = dict(H.TINY_B, num_hidden_layers=1, rope_scaling=None)
+    D, Hh, Hk, d = 192, 6, 2, 32
+    wq = torch.zeros(Hh * d, D)
+    wk = torch.zeros(Hk * d, D)
+    # keys answer to coordinate 0 of the normed input and queries to coordinate 1, both through the slowest
+    # rotation pair (index d/2 - 1 turns by < 1e-3 rad over 300 positions).  Token 7 alone carries coordinate 0
+    # and token 9 alone carries coordinate 1: a row holding token 9 scores ~2000 on rows holding token 7 and
+    # exactly 0 on every other row, itself included.
+    for h in range(Hh):
+        wq[h * d + d // 2 - 1, 1] = 8.0
+    for h in range(Hk):
+        wk[h * d + d // 2 - 1, 0] = 8.0
+    emb = torch.randn(1000, D, generator=torch.Generator().manual_seed(0)) * 0.02
+    emb[:, 0] = 0.0
+    emb[:, 1] = 0.0
+    emb[7, 0] = 3.0      # the marked token
+    emb[9, 1] = 3.0      # the asking token
+    path = os.path.join(H.tmp_root(), f"farkey_{dtype}")
+    write_model_folder(path, cfg, 3, TORCH[dtype], overrides={
+        "model.layers.0.self_attn.q_proj.weight": wq, "model.layers.0.self_attn.k_proj.weight": wk,
+        "model.embed_tokens.weight": emb})
+    toks = [t if t not in (7, 9) else 8 for t in H.random_tokens(1000, 250, seed=1)]
+    toks[19] = 7
+    toks[-1] = 9
+    _, runner = make_runner(path, dtype)
+    want = H.oracle_logits(path, toks)
+    for cuts in ([250], [249, 1], [17, 3, 100, 2, 127, 1]):
+        got = run_cut(runner, "f", toks, cuts)
+        H.assert_close(got, want, dtype, f"far key, cuts {cuts}")
+    without = list(toks)
+    without[19] = 8  # no marked token: the logits at the end are far from the ones found above
+    assert np.abs(H.oracle_logits(path, without)[-1] - want[-1]).max() > 0.1
