@@ -191,11 +191,26 @@ def llama_dims(cfg: dict):
     return H, Hk, d
 
 
-def llama_forward(cfg: dict, w: dict, tokens, positions=None, return_hidden: bool = False):
+def round_bf16(x):
+    """Round to the nearest bfloat16 (ties to even), returned as float64: what storing an
+    activation in bfloat16 does to it."""
+    f = np.asarray(x, np.float32)
+    u = f.view(np.uint32)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & np.uint32(0xFFFF0000)
+    return u.view(np.float32).astype(F64)
+
+
+def llama_forward(cfg: dict, w: dict, tokens, positions=None, return_hidden: bool = False, store=None):
     """Logits [T, V] of one whole sequence (crates/allpaca-core/src/model.rs:8301-8792
     in the order of the host forward): embed; per layer  h = norm(x); q,k,v;
     rope(q,k); causal attention; x += o Wo^T; h = norm(x); x += swiglu(h);
-    final norm; head (tied: the embedding matrix, model.rs:8005-8009)."""
+    final norm; head (tied: the embedding matrix, model.rs:8005-8009).
+
+    `store` (e.g. `round_bf16`) is applied to every activation that a reduced-precision
+    run keeps between two matrix products (normed input, q/k/v before and after
+    rotation, attention output, SwiGLU output), never to the residual stream or the
+    logits: it shows what such storage alone costs, with exact arithmetic otherwise."""
+    st = store if store is not None else (lambda z: z)
     H, Hk, d = llama_dims(cfg)
     eps = cfg.get("rms_norm_eps", 1e-5)
     theta = cfg.get("rope_theta", 10000.0)
@@ -205,16 +220,20 @@ def llama_forward(cfg: dict, w: dict, tokens, positions=None, return_hidden: boo
     x = embedding(w["model.embed_tokens.weight"], tokens)
     for l in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{l}."
-        h = rms_norm(x, w[p + "input_layernorm.weight"], eps)
-        q = linear(h, w[p + "self_attn.q_proj.weight"]).reshape(T, H, d)
-        k = linear(h, w[p + "self_attn.k_proj.weight"]).reshape(T, Hk, d)
-        v = linear(h, w[p + "self_attn.v_proj.weight"]).reshape(T, Hk, d)
-        q, k = rope_neox(q, pos, inv_freq), rope_neox(k, pos, inv_freq)
-        o = attention(q, k, v, H, Hk, causal=True).reshape(T, H * d)
+        h = st(rms_norm(x, w[p + "input_layernorm.weight"], eps))
+        q = st(linear(h, w[p + "self_attn.q_proj.weight"])).reshape(T, H, d)
+        k = st(linear(h, w[p + "self_attn.k_proj.weight"])).reshape(T, Hk, d)
+        v = st(linear(h, w[p + "self_attn.v_proj.weight"])).reshape(T, Hk, d)
+        q, k = st(rope_neox(q, pos, inv_freq)), st(rope_neox(k, pos, inv_freq))
+        o = st(attention(q, k, v, H, Hk, causal=True).reshape(T, H * d))
         x = x + linear(o, w[p + "self_attn.o_proj.weight"])
-        h = rms_norm(x, w[p + "post_attention_layernorm.weight"], eps)
-        x = x + swiglu(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
-    hN = rms_norm(x, w["model.norm.weight"], eps)
+        h = st(rms_norm(x, w[p + "post_attention_layernorm.weight"], eps))
+        if store is None:
+            x = x + swiglu(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+        else:
+            a = st(silu(linear(h, w[p + "mlp.gate_proj.weight"])) * linear(h, w[p + "mlp.up_proj.weight"]))
+            x = x + linear(a, w[p + "mlp.down_proj.weight"])
+    hN = st(rms_norm(x, w["model.norm.weight"], eps))
     head = w["lm_head.weight"] if "lm_head.weight" in w else w["model.embed_tokens.weight"]
     logits = linear(hN, head)
     return (logits, hN) if return_hidden else logits

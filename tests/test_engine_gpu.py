@@ -45,15 +45,14 @@ def test_whole_tail_and_portions(name, dtype, sharp):
     lens = {"A": [1, 7, 16, 33, 100], "B": [2, 33, 150], "C": [5, 64, 129]}[name]
     for i, n in enumerate(lens):
         toks = H.random_tokens(cfg.vocab_size, n, seed=10 * i + 1)
-        want = H.oracle_logits(folder, toks)
         whole = run_cut(runner, "w", toks, H.cut_whole(n))
-        H.assert_close(whole, want, dtype, f"{name} whole n={n}")
+        H.check_logits(whole, folder, toks, dtype, f"{name} whole n={n}")
         tail = run_cut(runner, "t", toks, H.cut_tail_decoded(n))
-        H.assert_close(tail, want, dtype, f"{name} tail-decoded n={n}")
+        H.check_logits(tail, folder, toks, dtype, f"{name} tail-decoded n={n}")
         for s in range(2):
             cuts = H.cut_changing(n, seed=s)
             got = run_cut(runner, "c", toks, cuts)
-            H.assert_close(got, want, dtype, f"{name} portions {cuts}")
+            H.check_logits(got, folder, toks, dtype, f"{name} portions {cuts}")
         if dtype == "float32":
             # rows do not depend on the cutting at all: the products and the attention of a row
             # add in an order that its position alone fixes
@@ -71,9 +70,8 @@ def test_first_tokens_and_page_sizes(name, dtype):
     for page_tokens in (1, 2, 16, 64):
         cfg, runner = make_runner(folder, dtype, page_tokens=page_tokens, num_pages=80)
         toks = toks or H.random_tokens(cfg.vocab_size, 40, seed=3)
-        want = H.oracle_logits(folder, toks)
         got = run_cut(runner, "p", toks, [1, 1, 1, 2, 35])
-        H.assert_close(got, want, dtype, f"{name} page_tokens={page_tokens}")
+        H.check_logits(got, folder, toks, dtype, f"{name} page_tokens={page_tokens}")
 
 
 def mixed_schedule(lengths, seed, live_max=4):
@@ -133,7 +131,7 @@ def test_mixed_batches_with_page_reuse(name, dtype):
         runner.cache.check()
     assert runner.cache.paged_groups[0].pool.allocations > num_pages, "the schedule did not reuse pages"
     for i, n in enumerate(lengths):
-        H.assert_close(np.concatenate(got[i]), H.oracle_logits(folder, toks[i]), dtype, f"{name} mixed request {i}")
+        H.check_logits(np.concatenate(got[i]), folder, toks[i], dtype, f"{name} mixed request {i}")
     assert runner.cache.free_pages(0) == num_pages
 
 
@@ -144,7 +142,7 @@ def test_long_decoding(dtype):
     cfg, runner = make_runner(folder, dtype, page_tokens=16, num_pages=20)
     toks = H.random_tokens(cfg.vocab_size, 230, seed=5)
     got = run_cut(runner, "d", toks, [30] + [1] * 200)
-    H.assert_close(got, H.oracle_logits(folder, toks), dtype, "long decoding")
+    H.check_logits(got, folder, toks, dtype, "long decoding")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -182,7 +180,7 @@ def test_a_far_key_is_found(dtype):
     want = H.oracle_logits(path, toks)
     for cuts in ([250], [249, 1], [17, 3, 100, 2, 127, 1]):
         got = run_cut(runner, "f", toks, cuts)
-        H.assert_close(got, want, dtype, f"far key, cuts {cuts}")
+        H.check_logits(got, path, toks, dtype, f"far key, cuts {cuts}")
     without = list(toks)
     without[19] = 8  # no marked token: the logits at the end are far from the ones found above
     assert np.abs(H.oracle_logits(path, without)[-1] - want[-1]).max() > 0.1
