@@ -25,3 +25,14 @@ def read_config_json(model_dir: str) -> dict:
 
 
 __all__ = ["ConfigError", "EngineConfig", "Llama3RopeScaling", "LlamaConfig", "read_config_json"]
+
+
+def preset(name: str) -> dict:
+    """A config.json of a known model shape, kept as data under `config/presets/`."""
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "presets")
+    path = os.path.join(here, name + ".json")
+    if not os.path.isfile(path):
+        known = sorted(f[:-5] for f in os.listdir(here) if f.endswith(".json"))
+        raise ConfigError(f"no preset {name!r}; known: {', '.join(known)}")
+    with open(path) as f:
+        return json.load(f)

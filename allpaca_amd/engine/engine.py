@@ -1,0 +1,138 @@
+"""The engine: requests in, tokens out.  It owns the model, the step function,
+the scheduler and the sampler, and offers the reference's calls
+(`generate`, `generate_stream`, `begin_request`, `step`/`poll`:
+crates/allpaca-core/src/engine.rs:2895, 3002, 3167, 3650, 3661)."""
+from __future__ import annotations
+
+import os
+import tempfile
+from typing import Dict, Iterator, List, Mapping, Optional, Sequence
+
+import torch
+
+from ..config import EngineConfig
+from ..models import load_model
+from ..sampling.params import FinishReason, GenerationOutput, GenerationParams, TokenEvent
+from ..sampling.sampler import Sampler
+from .batch import Entry
+from .runner import ModelRunner
+from .scheduler import FINISHED, Request, Scheduler
+
+_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+class Engine:
+    def __init__(self, model: str, config: Optional[EngineConfig] = None, **options):
+        """`model`: a folder with config.json and model.safetensors.  Options are those of `EngineConfig`."""
+        cfg = config or EngineConfig()
+        for k, v in options.items():
+            if not hasattr(cfg, k):
+                raise TypeError(f"unknown engine option {k!r}")
+            setattr(cfg, k, v)
+        cfg.validate()
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU is visible; the engine has no CPU path")
+        self.config = cfg
+        dtype = _DTYPES[cfg.dtype]
+        num_pages = cfg.num_pages or -(-cfg.max_tokens // cfg.page_tokens)
+        self.model_config, self.model = load_model(model, dtype, cfg.device,
+                                                   max_positions=num_pages * cfg.page_tokens)
+        self.runner = ModelRunner(self.model, cfg.page_tokens, num_pages, cfg.max_active_requests)
+        self.scheduler = Scheduler(self.runner.cache, cfg.max_active_requests, cfg.max_batch_tokens, cfg.chunk_tokens)
+        self.sampler = Sampler(self.runner.rt.device, cfg.seed)
+        self.requests: Dict[int, Request] = {}
+        self._next_id = 0
+        self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0}
+
+    @classmethod
+    def synthetic(cls, config_json: Mapping, seed: int = 0, config: Optional[EngineConfig] = None, **options) -> "Engine":
+        """An engine on random weights: the model folder is written to a temporary place first
+        (the reference's `--synthetic`, crates/allpaca-core/src/engine.rs:1577-1586)."""
+        from ..weights import write_model_folder
+        dtype = _DTYPES[(config.dtype if config else options.get("dtype", EngineConfig().dtype))]
+        folder = tempfile.mkdtemp(prefix="allpaca_amd_synthetic_")
+        write_model_folder(folder, config_json, seed, dtype)
+        return cls(folder, config, **options)
+
+    # ---- requests ------------------------------------------------------------
+    def add_request(self, prompt_token_ids: Sequence[int], params: Optional[GenerationParams] = None) -> int:
+        params = params or GenerationParams()
+        prompt = [int(t) for t in prompt_token_ids]
+        for t in prompt:
+            if not (0 <= t < self.runner.vocab_size):
+                raise ValueError(f"token {t} is outside the vocabulary of {self.runner.vocab_size}")
+        if len(prompt) + params.max_tokens > self.runner.rt.max_positions:
+            raise ValueError(f"{len(prompt)} prompt + {params.max_tokens} new tokens exceed the "
+                             f"{self.runner.rt.max_positions} positions this engine was set up for")
+        rid = self._next_id
+        self._next_id += 1
+        req = Request(rid, prompt, params)
+        self.scheduler.add(req)
+        self.requests[rid] = req
+        return rid
+
+    begin_request = add_request
+
+    def abort(self, request_id: int) -> None:
+        req = self.requests.pop(request_id, None)
+        if req is not None and req.status != FINISHED:
+            self.scheduler.abort(req)
+
+    def has_unfinished(self) -> bool:
+        return self.scheduler.has_work()
+
+    # ---- one tick ---------------------------------------------------------------
+    def step(self) -> List[TokenEvent]:
+        """One batch through the model: every decoding request advances by a token, prompts by a portion."""
+        plan = self.scheduler.plan()
+        self.stats["preemptions"] += len(plan.preempted)
+        for req in plan.admitted:
+            self.runner.storage.zero_slot(self.runner.cache.slot_of(req.id))
+        if not plan.scheduled:
+            return []
+        entries = []
+        for s in plan.scheduled:
+            toks = s.request.tokens[s.start:s.start + s.count]
+            entries.append(Entry(s.request.id, toks, [s.count - 1] if s.samples else []))
+        logits = self.runner.step(entries)
+        sampled = [s for s in plan.scheduled if s.samples]
+        for s in plan.scheduled:
+            self.scheduler.advance(s)
+            self.stats["decode_tokens" if s.request.output and s.count == 1 else "prefill_tokens"] += s.count
+        self.stats["steps"] += 1
+        events: List[TokenEvent] = []
+        if sampled:
+            tokens = self.sampler.sample(logits, [s.request.params for s in sampled],
+                                         [len(s.request.output) for s in sampled])
+            for s, tok in zip(sampled, tokens):
+                reason = self.scheduler.append_token(s.request, tok)
+                events.append(TokenEvent(s.request.id, int(tok), reason, len(s.request.prompt)))
+                if reason is not None:
+                    self.scheduler.finish(s.request, reason)
+        return events
+
+    poll = step
+
+    # ---- whole generations ---------------------------------------------------------
+    def generate_stream(self, prompt_token_ids: Sequence[int],
+                        params: Optional[GenerationParams] = None) -> Iterator[TokenEvent]:
+        rid = self.add_request(prompt_token_ids, params)
+        while self.requests[rid].status != FINISHED:
+            for ev in self.step():
+                if ev.request_id == rid:
+                    yield ev
+        self.requests.pop(rid, None)
+
+    def generate(self, prompts: Sequence[Sequence[int]], params=None) -> List[GenerationOutput]:
+        """Runs all prompts to the end under continuous batching; `params` is one `GenerationParams`
+        for all or one per prompt."""
+        if params is None or isinstance(params, GenerationParams):
+            params = [params] * len(prompts)
+        ids = [self.add_request(p, q) for p, q in zip(prompts, params)]
+        while any(self.requests[i].status != FINISHED for i in ids):
+            self.step()
+        out = []
+        for i in ids:
+            r = self.requests.pop(i)
+            out.append(GenerationOutput(list(r.output), len(r.prompt), len(r.output), r.finish_reason))
+        return out

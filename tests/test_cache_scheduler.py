@@ -1,0 +1,288 @@
+"""The cache manager's bookkeeping and the scheduler's decisions (no GPU)."""
+import numpy as np
+import pytest
+
+from allpaca_amd.cache import FREED, CacheError, CacheManager, OutOfPages, OutOfSlots, PagePool
+from allpaca_amd.engine.scheduler import Request, RequestTooLarge, Scheduler
+from allpaca_amd.parts import FixedState, PagedKV
+from allpaca_amd.sampling import FinishReason, GenerationParams
+
+FULL = PagedKV(2, 32)
+WIN = PagedKV(2, 32, window=10)
+
+
+def test_pool_hands_out_each_page_once_and_reuses():
+    pool = PagePool(3)
+    a, b, c = pool.alloc(), pool.alloc(), pool.alloc()
+    assert sorted([a, b, c]) == [0, 1, 2] and pool.free_count == 0
+    with pytest.raises(OutOfPages):
+        pool.alloc()
+    pool.free(b)
+    with pytest.raises(CacheError, match="twice"):
+        pool.free(b)
+    with pytest.raises(CacheError, match="outside"):
+        pool.free(7)
+    assert pool.alloc() == b and pool.allocations == 4  # last freed, first reused
+
+
+def test_pages_are_taken_on_demand_and_given_back():
+    cm = CacheManager([FULL, FULL, FULL], page_tokens=4, num_pages=6, max_requests=2)
+    assert len(cm.paged_groups) == 1 and cm.paged_groups[0].entries == [0, 1, 2]  # one group, one table per request
+    cm.admit("a")
+    assert cm.pages_needed("a", 5) == [2]
+    cm.reserve("a", 5)
+    cm.commit("a", 5)
+    assert cm.length("a") == 5 and len(cm.block_table("a", 0)) == 2 and cm.free_pages() == 4
+    cm.reserve("a", 3)      # positions 5..7 fit the second page
+    assert cm.free_pages() == 4
+    cm.commit("a", 3)
+    cm.reserve("a", 1)      # position 8 opens a third page
+    assert cm.free_pages() == 3
+    with pytest.raises(CacheError, match="beyond"):
+        cm.commit("a", 6)
+    cm.admit("b")
+    with pytest.raises(OutOfPages):
+        cm.reserve("b", 13)  # four pages wanted, three free: nothing is taken
+    assert cm.free_pages() == 3 and cm.block_table("b", 0) == []
+    with pytest.raises(OutOfSlots):
+        cm.admit("c")
+    with pytest.raises(CacheError, match="already live"):
+        cm.admit("a")
+    cm.release("a")
+    cm.check()
+    assert cm.free_pages() == 6
+    cm.release("b")
+    assert cm.slots.free_count == 2
+
+
+def test_groups_by_need_have_pools_of_their_own_and_windows_give_pages_back():
+    needs = [FULL, WIN, FULL, None, FixedState((4, 8)), WIN]
+    cm = CacheManager(needs, page_tokens=4, num_pages=[8, 5], max_requests=3)
+    assert [g.entries for g in cm.paged_groups] == [[0, 2], [1, 5]]
+    assert [g.entries for g in cm.state_groups] == [[4]]
+    assert cm.location[5] == ("paged", 1, 1) and cm.location[4] == ("state", 0, 0) and 3 not in cm.location
+    cm.admit("a")
+    for n in (6, 1, 1, 9, 3):
+        cm.reserve("a", n)
+        cm.commit("a", n)
+        cm.check()
+    L = cm.length("a")
+    assert L == 20
+    full, win = cm.block_table("a", 0), cm.block_table("a", 1)
+    assert len(full) == 5 and FREED not in full
+    # the next row is at position 20 and reads keys 11..20: pages 0 and 1 (positions 0..7) are passed
+    assert win[:2] == [FREED, FREED] and FREED not in win[2:]
+    assert cm.free_pages(0) == 3 and cm.free_pages(1) == 5 - 3
+    cm.release("a")
+    cm.check()
+    assert cm.free_pages(0) == 8 and cm.free_pages(1) == 5
+
+
+def test_truncate():
+    cm = CacheManager([FULL], page_tokens=4, num_pages=6, max_requests=1)
+    cm.admit("a")
+    cm.reserve("a", 14)
+    cm.commit("a", 14)
+    cm.truncate("a", 5)
+    assert cm.length("a") == 5 and len(cm.block_table("a", 0)) == 2 and cm.free_pages() == 4
+    cm.check()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_orders_lose_no_page(seed):
+    """Admissions, steps of random sizes, releases and truncations in random order: after every operation
+    no page is lost, held twice or free while held; at the end everything is back."""
+    rng = np.random.default_rng(seed)
+    cm = CacheManager([FULL, WIN, FixedState((3,))], page_tokens=int(rng.choice([1, 2, 16])), num_pages=[40, 24],
+                      max_requests=5)
+    live, next_id = [], 0
+    for _ in range(600):
+        op = rng.random()
+        if op < 0.15 and len(live) < 5:
+            cm.admit(next_id)
+            live.append(next_id)
+            next_id += 1
+        elif op < 0.8 and live:
+            s = live[int(rng.integers(len(live)))]
+            n = int(rng.choice([1, 1, 1, 2, 3, 7, 20]))
+            if cm.can_reserve(s, n):
+                cm.reserve(s, n)
+                cm.commit(s, n)
+            else:
+                with pytest.raises(OutOfPages):
+                    cm.reserve(s, n)
+        elif op < 0.9 and live:
+            s = live.pop(int(rng.integers(len(live))))
+            cm.release(s)
+            with pytest.raises(KeyError):
+                cm.release(s)       # a second release finds no such request
+        elif live:
+            s = live[int(rng.integers(len(live)))]
+            L = cm.length(s)
+            if L and cm.paged_groups[1].need.window is not None:
+                try:
+                    cm.truncate(s, int(rng.integers(max(0, L - 3), L + 1)))
+                except CacheError:
+                    pass
+        cm.check()
+    for s in live:
+        cm.release(s)
+    cm.check()
+    assert cm.free_pages(0) == 40 and cm.free_pages(1) == 24 and cm.slots.free_count == 5
+    assert cm.paged_groups[0].pool.allocations > 40  # pages went round more than once
+
+
+# ---------------------------------------------------------------------------- scheduler
+def sched(num_pages=16, page_tokens=4, max_active=4, budget=16, chunk=8):
+    cm = CacheManager([FULL], page_tokens, num_pages, max_requests=max_active)
+    return cm, Scheduler(cm, max_active, budget, chunk)
+
+
+def req(i, n_prompt, max_tokens=4, **kw):
+    return Request(i, list(range(1, n_prompt + 1)), GenerationParams(max_tokens=max_tokens, temperature=0.0, **kw))
+
+
+def run_step(cm, s, token_of=lambda r: 100 + len(r.output)):
+    """Plays the engine's part: reserve + commit pages, advance, append a token where one is sampled."""
+    plan = s.plan()
+    for e in plan.scheduled:
+        cm.reserve(e.request.id, e.count)
+    for e in plan.scheduled:
+        cm.commit(e.request.id, e.count)
+        s.advance(e)
+        if e.samples:
+            reason = s.append_token(e.request, token_of(e.request))
+            if reason:
+                s.finish(e.request, reason)
+    cm.check()
+    return plan
+
+
+def test_prompts_are_cut_under_the_budget_and_decodes_come_first():
+    cm, s = sched(num_pages=32, budget=16, chunk=8)
+    a, b = req(0, 20), req(1, 5)
+    s.add(a)
+    s.add(b)
+    p = run_step(cm, s)
+    # a gets a chunk of 8, b its 5 tokens: 13 <= 16
+    assert [(e.request.id, e.start, e.count, e.samples) for e in p.scheduled] == [(0, 0, 8, False), (1, 0, 5, True)]
+    p = run_step(cm, s)
+    # b decodes first (1 token), then a's next chunk
+    assert [(e.request.id, e.start, e.count, e.samples) for e in p.scheduled] == [(1, 5, 1, True), (0, 8, 8, False)]
+    p = run_step(cm, s)
+    assert [(e.request.id, e.count, e.samples) for e in p.scheduled] == [(1, 1, True), (0, 4, True)]
+    s.add(req(2, 30))
+    p = run_step(cm, s)
+    # two decodes, then the newcomer gets what is left of the chunk/budget
+    assert [(e.request.id, e.count) for e in p.scheduled] == [(0, 1), (1, 1), (2, 8)]
+    assert p.n_tokens <= 16
+
+
+def test_budget_cuts_a_portion_to_any_size():
+    cm, s = sched(num_pages=64, budget=10, chunk=8, max_active=4)
+    for i in range(3):
+        s.add(req(i, 9))
+    p = run_step(cm, s)
+    assert [(e.request.id, e.count) for e in p.scheduled] == [(0, 8), (1, 2)]
+    p = run_step(cm, s)
+    assert [(e.request.id, e.count, e.samples) for e in p.scheduled] == [(0, 1, True), (1, 7, True), (2, 2, False)]
+
+
+def test_admission_is_fifo_and_capped():
+    cm, s = sched(num_pages=64, max_active=2, budget=64, chunk=64)
+    for i in range(4):
+        s.add(req(i, 3, max_tokens=2))
+    p = run_step(cm, s)
+    assert [e.request.id for e in p.scheduled] == [0, 1] and len(s.waiting) == 2
+    p = run_step(cm, s)   # 0 and 1 produce their second token and finish: their slots free up
+    assert [r.status for r in (p.scheduled[0].request, p.scheduled[1].request)] == ["finished", "finished"]
+    p = run_step(cm, s)
+    assert [e.request.id for e in p.scheduled] == [2, 3]
+
+
+def test_every_request_finishes_with_length_or_stop():
+    cm, s = sched(num_pages=40, max_active=3, budget=12, chunk=5)
+    reqs = [req(i, n, max_tokens=m) for i, (n, m) in enumerate([(7, 3), (1, 5), (19, 2), (4, 6), (11, 1)])]
+    reqs[1].params.stop_token_ids = [102]
+    for r in reqs:
+        s.add(r)
+    for _ in range(200):
+        if not s.has_work():
+            break
+        p = run_step(cm, s)
+        assert p.n_tokens <= 12 and len(s.running) <= 3
+    assert not s.has_work()
+    assert [r.finish_reason for r in reqs] == ["length", "stop", "length", "length", "length"]
+    assert [len(r.output) for r in reqs] == [3, 3, 2, 6, 1]
+    assert cm.free_pages() == 40 and cm.slots.free_count == 3
+
+
+def test_a_waiting_prompt_waits_for_pages():
+    cm, s = sched(num_pages=4, page_tokens=4, max_active=4, budget=64, chunk=64)
+    s.add(req(0, 10, max_tokens=2))     # 3 pages
+    s.add(req(1, 9, max_tokens=2))      # 3 pages: does not fit beside request 0
+    p = run_step(cm, s)
+    # request 1 gets the one page that is left: a portion of 4 tokens
+    assert [(e.request.id, e.count) for e in p.scheduled] == [(0, 10), (1, 4)]
+    p = run_step(cm, s)
+    assert [(e.request.id, e.count) for e in p.scheduled] == [(0, 1)]      # 1 has no page to go on with
+    assert reqs_status(s) == {1: "running"}                                 # 0 produced its two tokens and is gone
+    p = run_step(cm, s)
+    assert [(e.request.id, e.count) for e in p.scheduled] == [(1, 5)]      # 0's pages came back
+
+
+def reqs_status(s):
+    out = {r.id: r.status for r in s.running}
+    out.update({r.id: r.status for r in s.waiting})
+    return out | {}
+
+
+def test_preemption_when_a_decode_needs_a_page():
+    cm, s = sched(num_pages=4, page_tokens=4, max_active=4, budget=64, chunk=64)
+    a, b = req(0, 7, max_tokens=8), req(1, 6, max_tokens=8)
+    s.add(a)
+    s.add(b)
+    run_step(cm, s)                      # both prefilled: 2 pages each, pool empty
+    assert cm.free_pages() == 0
+    p = run_step(cm, s)                  # a: position 7 fits its page; b: position 6 fits
+    assert [e.request.id for e in p.scheduled] == [0, 1] and not p.preempted
+    p = run_step(cm, s)                  # a needs a third page: b, admitted last, gives way
+    assert [r.id for r in p.preempted] == [1] and [e.request.id for e in p.scheduled] == [0]
+    assert b.status == "waiting" and b.computed == 0 and b.preemptions == 1 and len(b.output) == 2
+    assert s.waiting[0] is b
+    out_before = list(b.output)
+    for _ in range(40):
+        if not s.has_work():
+            break
+        run_step(cm, s)
+    assert a.finish_reason == b.finish_reason == "length"
+    # the preempted request recomputed prompt + its two tokens and went on from there
+    assert b.output[:2] == out_before and len(b.output) == 8
+    assert cm.free_pages() == 4
+
+
+def test_the_newest_request_preempts_itself():
+    cm, s = sched(num_pages=4, page_tokens=4, max_active=4, budget=64, chunk=64)
+    a, b = req(0, 4, max_tokens=8), req(1, 11, max_tokens=4)
+    s.add(a)
+    s.add(b)
+    run_step(cm, s)                      # a: 1 page, b: 3 pages
+    p = run_step(cm, s)                  # a (older) takes... no page free: b, the newest, gives way
+    assert [r.id for r in p.preempted] == [1] and [e.request.id for e in p.scheduled] == [0]
+
+
+def test_a_request_larger_than_the_pool_is_refused():
+    cm, s = sched(num_pages=4, page_tokens=4)
+    with pytest.raises(RequestTooLarge, match="whole pool"):
+        s.add(req(0, 14, max_tokens=4))
+    s.add(req(1, 12, max_tokens=4))       # exactly the pool
+    with pytest.raises(ValueError):
+        s.add(Request(2, [], GenerationParams()))
+
+
+def test_params_defaults_follow_the_reference():
+    p = GenerationParams()
+    assert (p.max_tokens, p.temperature, p.top_k, p.top_p, p.seed, p.stop_token_ids) == (32, 0.8, 40, 0.95, None, [])
+    assert GenerationParams(max_tokens=0).max_tokens == 1   # crates/allpaca-core/src/engine.rs:3194
+    assert GenerationParams(temperature=1e-6).greedy and not GenerationParams(temperature=0.1).greedy
+    assert FinishReason.STOP == "stop" and FinishReason.LENGTH == "length"

@@ -1,0 +1,195 @@
+"""Generation through the entry points: greedy and sampled tokens against the plain
+implementation, concurrency against solo runs, preemption, the command line and
+the trace replay program."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import helpers as H
+import plain_llama as P
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def engine_for(folder, dtype="float32", **opts):
+    from allpaca_amd.engine import Engine
+    base = dict(dtype=dtype, max_tokens=1024, max_active_requests=8, use_graphs=False)
+    base.update(opts)
+    return Engine(folder, **base)
+
+
+def params(**kw):
+    from allpaca_amd.sampling import GenerationParams
+    return GenerationParams(**kw)
+
+
+def test_greedy_generation_equals_the_plain_implementation():
+    """Tiny A: prompts of 1, 7, 16 and 33 tokens, 16 greedy tokens each, alone and as chunked mixed batches."""
+    folder = H.model_folder("A", "float32", True)
+    cfg, w = H.oracle(folder)
+    prompts = [H.random_tokens(256, n, seed=n) for n in (1, 7, 16, 33)]
+    want = [P.greedy_generate(cfg, w, p, 16) for p in prompts]
+    eng = engine_for(folder)
+    for p, wnt in zip(prompts, want):
+        out = eng.generate([p], params(max_tokens=16, temperature=0.0))[0]
+        assert out.token_ids == wnt and out.finish_reason == "length" and out.prompt_tokens == len(p)
+    eng = engine_for(folder, chunk_tokens=8, max_batch_tokens=12)
+    outs = eng.generate(prompts, params(max_tokens=16, temperature=0.0))
+    assert [o.token_ids for o in outs] == want
+    assert eng.stats["steps"] < sum(len(p) + 16 for p in prompts)   # prompts ran in portions, not token by token
+
+
+def test_sampled_generation_equals_the_plain_sampler():
+    """Tiny B: six prompts of 2 to 150 tokens, temperature 0.8 (top-k 40, top-p 0.95), 24 tokens each:
+    every token is what the plain sampler draws from the plain logits of the same context with the same
+    uniform number."""
+    from allpaca_amd.sampling.sampler import uniform_for
+    folder = H.model_folder("B", "float32", True)
+    cfg, w = H.oracle(folder)
+    prompts = [H.random_tokens(1000, n, seed=n) for n in (2, 9, 31, 64, 100, 150)]
+    eng = engine_for(folder, chunk_tokens=32, max_batch_tokens=48)
+    pr = [params(max_tokens=24, temperature=0.8, seed=7 + i) for i in range(len(prompts))]
+    outs = eng.generate(prompts, pr)
+    for i, (p, o) in enumerate(zip(prompts, outs)):
+        assert len(o.token_ids) == 24
+        toks = list(p)
+        for j, t in enumerate(o.token_ids):
+            if j % 6 == 0:   # every sixth token is checked against the oracle (each check is a whole forward)
+                lg = P.llama_forward(cfg, w, toks)[-1]
+                assert t == P.sample(lg, 0.8, 40, 0.95, uniform_for(7 + i, j)), f"prompt {i} token {j}"
+            toks.append(t)
+    assert len({tuple(o.token_ids) for o in outs}) == len(outs)
+
+
+def test_same_seed_same_tokens_under_any_batching_and_stop_ids():
+    folder = H.model_folder("B", "float32", True)
+    prompts = [H.random_tokens(1000, n, seed=50 + n) for n in (3, 40, 77, 12, 130)]
+    pr = [params(max_tokens=12, temperature=0.9, top_k=0, top_p=1.0, seed=3),
+          params(max_tokens=12, temperature=0.0),
+          params(max_tokens=12, temperature=0.7, top_k=5, seed=11),
+          params(max_tokens=12, temperature=1.3, top_k=0, top_p=0.6, seed=5),
+          params(max_tokens=12, temperature=0.8)]
+    solo = [engine_for(folder).generate([p], q)[0].token_ids for p, q in zip(prompts, pr)]
+    together = engine_for(folder, chunk_tokens=16, max_batch_tokens=24).generate(prompts, pr)
+    assert [o.token_ids for o in together] == solo        # crates/allpaca-core/tests/hip_runtime.rs:8149-8176 in spirit
+    stop = solo[1][4]
+    first = solo[1].index(stop)
+    out = engine_for(folder).generate([prompts[1]], params(max_tokens=12, temperature=0.0, stop_token_ids=[stop]))[0]
+    assert out.token_ids == solo[1][: first + 1] and out.finish_reason == "stop"   # the stop token is emitted
+
+
+def test_preemption_gives_the_same_tokens():
+    folder = H.model_folder("A", "float32", True)
+    prompts = [H.random_tokens(256, n, seed=70 + n) for n in (30, 25, 28)]
+    pr = params(max_tokens=40, temperature=0.8, seed=1)
+    solo = [engine_for(folder).generate([p], pr)[0].token_ids for p in prompts]
+    # 3 requests grow to ~70 tokens = 5 pages each; 11 pages cannot hold them all: someone must give way
+    eng = engine_for(folder, num_pages=11, max_active_requests=3)
+    outs = eng.generate(prompts, pr)
+    assert eng.stats["preemptions"] > 0
+    assert [o.token_ids for o in outs] == solo
+    assert eng.runner.cache.free_pages(0) == 11
+    eng.runner.cache.check()
+
+
+def test_stream_and_low_level_calls():
+    folder = H.model_folder("A", "float32")
+    eng = engine_for(folder)
+    p = H.random_tokens(256, 9, seed=1)
+    evs = list(eng.generate_stream(p, params(max_tokens=5, temperature=0.0)))
+    assert [e.finish_reason for e in evs] == [None] * 4 + ["length"] and all(e.prompt_tokens == 9 for e in evs)
+    rid = eng.begin_request(p, params(max_tokens=5, temperature=0.0))
+    got = []
+    while eng.has_unfinished():
+        got += [e.token_id for e in eng.poll() if e.request_id == rid]
+    assert got == [e.token_id for e in evs]
+    from allpaca_amd.engine import RequestTooLarge
+    with pytest.raises(ValueError):
+        eng.add_request([256])                       # outside the vocabulary
+    small = engine_for(folder, num_pages=2)
+    with pytest.raises((RequestTooLarge, ValueError)):
+        small.add_request(p, params(max_tokens=60))
+
+
+def test_command_line_generate():
+    folder = H.model_folder("A", "float32", True)
+    cfg, w = H.oracle(folder)
+    p1, p2 = H.random_tokens(256, 5, seed=1), H.random_tokens(256, 11, seed=2)
+    spec = ",".join(map(str, p1)) + ";" + ",".join(map(str, p2))
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "allpaca-amd"), "generate", "--model", folder, "--dtype", "fp32",
+           "--prompt-tokens", spec, "--max-tokens", "6", "--temperature", "0", "--json"]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=280)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [json.loads(ln) for ln in r.stdout.strip().splitlines()]
+    assert [ln["token_ids"] for ln in lines] == [P.greedy_generate(cfg, w, p, 6) for p in (p1, p2)]
+    r = subprocess.run(cmd[:2] + ["generate", "--synthetic", "--cpu-only", "--prompt-tokens", "1"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "no CPU path" in r.stderr or "not available" in r.stderr
+
+
+def replay(folder, dtype, steps, max_tokens, out_dir, page_tokens=16):
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+           "--out", out_dir, "--max-tokens", str(max_tokens), "--page-tokens", str(page_tokens)]
+    text = "".join(json.dumps(s) + "\n" for s in steps)
+    r = subprocess.run(cmd, input=text, capture_output=True, text=True, timeout=280)
+    assert r.returncode == 0, r.stderr[-3000:]
+    assert r.stdout.split() == [w for s in steps for w in ("done", str(s["step"]))]
+    return r
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(dtype, tmp_path):
+    """The replay program, as a user runs it: the same requests whole, with the last 32 tokens decoded one by
+    one, and mixed with other requests so that pages are used again."""
+    folder = H.model_folder("B", dtype, True)
+    V = 1000
+    lens = [70, 150, 33, 100, 64]
+    toks = {f"r{i}": H.random_tokens(V, n, seed=200 + i) for i, n in enumerate(lens)}
+    # whole
+    steps = [dict(step=i, entries=[dict(id=k, tokens=t, want=list(range(len(t))))], end=[k])
+             for i, (k, t) in enumerate(toks.items())]
+    out = str(tmp_path / "whole")
+    replay(folder, dtype, steps, 192, out)
+    for i, (k, t) in enumerate(toks.items()):
+        got = np.fromfile(os.path.join(out, f"{i}.f32"), dtype="<f4").reshape(len(t), V)
+        H.check_logits(got, folder, t, dtype, f"trace whole {k}")
+    # tail decoded: logits wanted only at the last prompt row and at the decoded ones; a step without `want`
+    k, t = "r1", toks["r1"]
+    steps = [dict(step=0, entries=[dict(id=k, tokens=t[:60], want=[])], end=[]),
+             dict(step=1, entries=[dict(id=k, tokens=t[60:118], want=[57])], end=[])]
+    steps += [dict(step=2 + j, entries=[dict(id=k, tokens=[t[118 + j]], want=[0])], end=[k] if j == 31 else [])
+              for j in range(32)]
+    out = str(tmp_path / "tail")
+    replay(folder, dtype, steps, 192, out)
+    assert not os.path.exists(os.path.join(out, "0.f32"))
+    rows = [np.fromfile(os.path.join(out, f"{s}.f32"), dtype="<f4").reshape(1, V) for s in range(1, 34)]
+    want_rows = list(range(117, 150))
+    noise = H.oracle_logits_bf16_storage(folder, t)[want_rows] if dtype == "bfloat16" else None
+    H.assert_close(np.concatenate(rows), H.oracle_logits(folder, t)[want_rows], dtype, "trace tail", noise)
+    # mixed, four live at most, pool of 4 x 64-rounded tokens of the smaller requests: pages are used again
+    import test_engine_gpu as E
+    sched = E.mixed_schedule(lens, seed=3)
+    steps, got = [], {k: [] for k in toks}
+    keys = list(toks)
+    for si, (entries, ends) in enumerate(sched):
+        steps.append(dict(step=si, entries=[dict(id=keys[i], tokens=toks[keys[i]][at:at + n], want=list(range(n)))
+                                            for i, at, n in entries], end=[keys[i] for i in ends]))
+    out = str(tmp_path / "mixed")
+    live_budget = sum(sorted(-(-n // 64) * 64 for n in lens)[-4:])
+    replay(folder, dtype, steps, live_budget, out)
+    for si, (entries, ends) in enumerate(sched):
+        arr = np.fromfile(os.path.join(out, f"{si}.f32"), dtype="<f4").reshape(-1, V)
+        row = 0
+        for i, at, n in entries:
+            got[keys[i]].append(arr[row:row + n])
+            row += n
+        assert row == arr.shape[0]
+    for k, t in toks.items():
+        H.check_logits(np.concatenate(got[k]), folder, t, dtype, f"trace mixed {k}")
