@@ -1,8 +1,10 @@
 """Device memory of the cache: one tensor per paged group and per state group,
 allocated once.  A paged group's tensor is
 [layers of the group, pages + 1, 2 (keys, values), kv_heads, page_tokens, head_dim];
-the extra last page is never handed out (rows that pad a replayed graph write
-there).  A state group's tensor is [layers of the group, slots + 1, *shape]."""
+inside a page, a key's elements lie together ([page_tokens, head_dim]) and a
+value's positions lie together ([head_dim, page_tokens], the same count of
+elements); the extra last page is never handed out (rows that pad a replayed
+graph write there).  A state group's tensor is [layers of the group, slots + 1, *shape]."""
 from __future__ import annotations
 
 from dataclasses import dataclass

@@ -80,4 +80,4 @@ __device__ __forceinline__ float block_max(float v, float* smem) {
   return t;
 }
 
-static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+__host__ __device__ static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }

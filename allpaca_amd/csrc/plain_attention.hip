@@ -10,7 +10,8 @@
 // order of additions for a row is fixed by its position alone, never by what
 // else is in the batch or how the prompt was cut.
 //
-// cache[page][0|1][kv_head][slot][d]; page = block_table[seg][t / P], slot = t % P.
+// keys cache[page][0][kv_head][slot][i], values cache[page][1][kv_head][i][slot];
+// page = block_table[seg][t / P], slot = t % P.
 #include "common.h"
 #include <math.h>
 
@@ -63,11 +64,11 @@ __global__ __launch_bounds__(64) void paged_attention_plain_kernel(
       const float pj = ps[j];
       const int tj = c * WAVE + j;
       const int page = bt[tj / P];
-      const size_t vb = ((((size_t)page * 2 + 1) * Hk + kvh) * P + (tj % P)) * d;
+      const size_t vb = (((size_t)page * 2 + 1) * Hk + kvh) * (size_t)P * d + (tj % P);
 #pragma unroll
       for (int i = 0; i < MAX_D_PER_LANE; ++i) {
         const int e = lane + i * WAVE;
-        if (e < d) o[i] = fmaf(pj, load_f(cache, cache_dtype, vb + e), o[i]);
+        if (e < d) o[i] = fmaf(pj, load_f(cache, cache_dtype, vb + (size_t)e * P), o[i]);
       }
     }
   }

@@ -134,9 +134,12 @@ APC_EXPORT int apc_silu_mul(const void* gu, int in_dtype, int ldg, void* out, in
 //   x_i' = a cos - b sin,  x_{i+rot/2}' = a sin + b cos
 // (crates/allpaca-cpu/src/kernels.rs:676-682).  cos/sin come from a table
 // [max_pos, 2, rot/2] made on the host in 64-bit and rounded once to float32.
-// q is rotated in place.  k (rotated) and v go to
-//   cache[page][0 or 1][kv_head][slot][:]   page = block_table[seg][pos / P], slot = pos % P
-// (reference: page = pos / P, slot = pos % P, crates/allpaca-core/src/model.rs:10439-10443).
+// q is rotated in place.  k (rotated) and v go to the page
+//   page = block_table[seg][pos / P], slot = pos % P
+// (reference: page = pos / P, slot = pos % P, crates/allpaca-core/src/model.rs:10439-10443):
+//   keys    cache[page][0][kv_head][slot][i]      (a key's elements lie together)
+//   values  cache[page][1][kv_head][i][slot]      (an element's slots lie together: the
+//           value product sums over positions, and matrix cores want that axis contiguous)
 // With cache == nullptr only the rotation is done (k in place as well).
 // ---------------------------------------------------------------------------
 __global__ void rope_kv_write_kernel(void* __restrict__ qkv, int dtype, int ld, int q_off, int k_off, int v_off,
@@ -157,11 +160,13 @@ __global__ void rope_kv_write_kernel(void* __restrict__ qkv, int dtype, int ld, 
   size_t dst = 0;
   if (kind != 0 && cache) {
     const int page = block_table[(size_t)row_seg[t] * max_blocks + pos / P];
-    dst = ((((size_t)page * 2 + (kind - 1)) * Hk + head) * P + (pos % P)) * d;
+    const size_t head_base = (((size_t)page * 2 + (kind - 1)) * Hk + head) * (size_t)P * d;
+    dst = kind == 1 ? head_base + (size_t)(pos % P) * d : head_base + (pos % P);
   }
   if (kind == 2) {
     if (!cache) return;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) store_f(cache, cache_dtype, dst + i, load_f(qkv, dtype, src + i));
+    for (int i = threadIdx.x; i < d; i += blockDim.x)
+      store_f(cache, cache_dtype, dst + (size_t)i * P, load_f(qkv, dtype, src + i));
     return;
   }
   const float* cs = cos_sin + (size_t)pos * rot;  // [2][half]

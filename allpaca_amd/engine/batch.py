@@ -45,6 +45,17 @@ class StepInfo:
     max_context: int = 0              # largest (pos0 + rows) of the step
     max_rows: int = 0                 # largest segment
     decode_only: bool = False         # every segment is a single row
+    # how attention kernels divide the rows: single-row segments ("decode rows") and, for longer
+    # segments, tiles of at most TILE_ROWS consecutive rows of one segment
+    decode_rows: Optional[torch.Tensor] = None   # int32 [n_decode_rows] row indices; None when every row is one
+    n_decode_rows: int = 0
+    max_decode_context: int = 0       # largest (position + 1) among the decode rows
+    tile_row0: Optional[torch.Tensor] = None     # int32 [n_tiles]
+    tile_rows: Optional[torch.Tensor] = None     # int32 [n_tiles]
+    n_tiles: int = 0
+
+
+TILE_ROWS = 64
 
 
 def pack_step(entries: Sequence[Entry], pos0: Sequence[int], slots: Sequence[int],
@@ -70,8 +81,16 @@ def pack_step(entries: Sequence[Entry], pos0: Sequence[int], slots: Sequence[int
                 a = np.asarray(t, dtype=np.int32)
                 bt[s, : len(t)] = np.where(a < 0, pad_page[g], a)
         blocks.append(bt)
+    decode_rows = np.asarray([r0 for r0, n in zip(row0, rows) if n == 1], dtype=np.int32)
+    t_row0, t_rows = [], []
+    for r0, n in zip(row0, rows):
+        if n > 1:
+            for a in range(0, n, TILE_ROWS):
+                t_row0.append(r0 + a)
+                t_rows.append(min(TILE_ROWS, n - a))
     parts = [tokens, positions, row_seg, row0, np.asarray(rows, np.int32), np.asarray(pos0, np.int32),
-             np.asarray(slots, np.int32), logit_rows] + [b.reshape(-1) for b in blocks]
+             np.asarray(slots, np.int32), logit_rows, decode_rows, np.asarray(t_row0, np.int32),
+             np.asarray(t_rows, np.int32)] + [b.reshape(-1) for b in blocks]
     flat = np.concatenate(parts) if parts else np.zeros(0, np.int32)
     host = torch.from_numpy(flat).pin_memory() if device.type == "cuda" else torch.from_numpy(flat)
     dev = host.to(device, non_blocking=False)
@@ -80,7 +99,10 @@ def pack_step(entries: Sequence[Entry], pos0: Sequence[int], slots: Sequence[int
     return StepInfo(
         n_rows=T, n_segs=S, tokens=v[0], positions=v[1], row_seg=v[2], seg_row0=v[3], seg_rows=v[4], seg_pos0=v[5],
         state_slots=v[6], logit_rows=v[7] if logit_rows.size else None, n_logit_rows=int(logit_rows.size),
-        block_tables=[v[8 + g].view(S, blocks[g].shape[1]) for g in range(len(blocks))],
+        block_tables=[v[11 + g].view(S, blocks[g].shape[1]) for g in range(len(blocks))],
+        decode_rows=None if decode_rows.size == T else v[8], n_decode_rows=int(decode_rows.size),
+        max_decode_context=max([p + 1 for p, n in zip(pos0, rows) if n == 1] or [0]),
+        tile_row0=v[9], tile_rows=v[10], n_tiles=len(t_row0),
         host_row0=row0.tolist(), host_rows=list(rows), host_pos0=list(pos0), host_slots=list(slots),
         max_context=max([p + n for p, n in zip(pos0, rows)] or [0]), max_rows=max(rows or [0]),
         decode_only=all(n == 1 for n in rows))

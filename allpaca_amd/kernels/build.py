@@ -23,9 +23,9 @@ CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
 
 LIBS: Dict[str, List[str]] = {
     "plain": ["plain_ops.hip", "plain_gemm.hip", "plain_attention.hip", "sampling.hip"],
-    "tuned": ["gemm_bf16.hip", "skinny_gemm_bf16.hip", "attention_bf16.hip", "fused_ops.hip"],
+    "tuned": ["gemm_bf16.hip", "skinny_gemm_bf16.hip", "attention_bf16.hip"],
 }
-HEADERS = ["common.h", "allpaca_kernels.h"]
+HEADERS = ["common.h", "mfma.h"]
 
 ARCH = "gfx950"
 # -packed-fp32-ops is switched off for device code: some packed forms have given wrong results on this hardware.

@@ -37,13 +37,12 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_sample_rows": [P, I, I, I, P, P, P, P, P, P],
     },
     "tuned": {
-        "apc_gemm_bf16": [P, I, P, I, P, I, I, I, I, I, I, P],
+        "apc_gemm_bf16": [P, I, P, I, P, I, I, I, I, I, P],
         "apc_gemm_swiglu_bf16": [P, I, P, P, I, P, I, I, I, I, P],
-        "apc_skinny_gemm_bf16": [P, I, P, I, P, I, I, I, I, I, I, P],
+        "apc_skinny_gemm_bf16": [P, I, P, I, P, I, I, I, I, I, P],
         "apc_skinny_swiglu_bf16": [P, I, P, P, I, P, I, I, I, I, P],
-        "apc_attention_prefill_bf16": [P, I, I, P, I, I, I, I, P, I, P, I, P, P, P, I, I, F, P],
-        "apc_attention_decode_bf16": [P, I, I, P, I, I, I, I, I, P, I, P, I, P, P, I, F, P, P, I, P],
-        "apc_attention_decode_workspace": [I, I, I, I],
+        "apc_attention_prefill_bf16": [P, I, I, P, I, I, I, I, P, I, P, I, P, P, P, P, I, I, F, P],
+        "apc_attention_decode_bf16": [P, I, I, P, I, I, I, I, I, P, I, P, I, P, P, P, I, F, I, I, P, P],
     },
 }
 

@@ -165,7 +165,9 @@ def make_cache(n_seq_tokens, Hk, d, P_, dtype, seed=0, shuffle=True):
             bt[s, b] = page
             lo, hi = b * P_, min(n, (b + 1) * P_)
             cache[page, 0, :, : hi - lo] = k[lo:hi].permute(1, 0, 2)
-            cache[page, 1, :, : hi - lo] = v[lo:hi].permute(1, 0, 2)
+            vt = torch.zeros(Hk, d, P_, dtype=dtype)          # values lie [element][slot] inside a page
+            vt[:, :, : hi - lo] = v[lo:hi].permute(1, 2, 0)
+            cache[page, 1] = vt.reshape(Hk, P_, d)
     return cache.to(DEV), torch.from_numpy(bt).to(DEV), ks, vs
 
 
@@ -266,10 +268,12 @@ def test_rope_kv_write(dtype):
         for t in range(T):
             page, slot = btc[seg_list[t], pos_list[t] // P_], pos_list[t] % P_
             close(f64(cache[page, 0, :, slot]), rk[t], **tol)
-            close(f64(cache[page, 1, :, slot]), v[t], atol=0, rtol=0)
+            close(f64(cache[page, 1].reshape(Hk, d, P_)[:, :, slot]), v[t], atol=0, rtol=0)
             written[page, slot] = True
-        untouched = cache.cpu()[~written.unsqueeze(1).unsqueeze(2).expand(13, 2, Hk, P_)]
-        assert untouched.abs().max().item() == 0.0  # nothing written anywhere else
+        c = cache.cpu()
+        keys_untouched = c[:, 0][~written.unsqueeze(1).expand(13, Hk, P_)]
+        vals_untouched = c[:, 1].reshape(13, Hk, d, P_).permute(0, 1, 3, 2)[~written.unsqueeze(1).expand(13, Hk, P_)]
+        assert keys_untouched.abs().max().item() == 0.0 and vals_untouched.abs().max().item() == 0.0
 
 
 def test_argmax_rows():

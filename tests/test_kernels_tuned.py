@@ -1,0 +1,176 @@
+"""Each bfloat16 MFMA kernel alone against a float64 reference of the same operation on the same
+bfloat16 inputs, at sizes other than the engine's: widths and row counts that are no multiple of a
+tile, every head size in steps of 16, head counts and groups of any kind, windows, page sizes."""
+import math
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+from test_kernels_plain import DEV, f64, gen, make_cache
+
+pytestmark = pytest.mark.gpu
+
+BF = torch.bfloat16
+
+
+def tuned():
+    from allpaca_amd.kernels import tuned as t
+    return t
+
+
+def check(got, want, out_dtype):
+    """Sums are float32 over exact bfloat16 products: the result is within float32 summation error of the
+    float64 value, plus one rounding to bfloat16 if it is stored so."""
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    scale = np.abs(want).max() + 1e-30
+    d = np.abs(got - want)
+    tol = 1e-5 * scale + (2.0 ** -8) * np.abs(want) if out_dtype == BF else 1e-5 * scale + 1e-5 * np.abs(want)
+    assert (d <= tol).all(), f"max diff {d.max():.3e} (scale {scale:.3e}) at {np.unravel_index((d - tol).argmax(), d.shape)}"
+
+
+GEMM_SHAPES = [(1, 5, 16), (3, 100, 136), (8, 4096, 512), (16, 33, 1208), (17, 257, 72), (33, 64, 8), (64, 130, 264),
+               (65, 64, 64), (128, 129, 72), (200, 300, 200), (300, 515, 120), (1000, 40, 1024)]
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_gemm_bf16(M, N, K):
+    t = tuned()
+    a, w = gen(M, K, seed=1, dtype=BF).to(DEV), gen(N, K, seed=2, dtype=BF).to(DEV)
+    want = f64(a) @ f64(w).T
+    for out_dtype in (BF, torch.float32):
+        out = torch.full((M, N), 7.0, dtype=out_dtype, device=DEV)
+        t.gemm_bf16(a, w, out)
+        check(f64(out), want, out_dtype)
+    acc = gen(M, N, seed=3).to(DEV)
+    before = f64(acc)
+    t.gemm_bf16(a, w, acc, accumulate=True)
+    check(f64(acc) - before, want, torch.float32)
+
+
+def test_gemm_bf16_strided_views_and_padding_rows_untouched():
+    t = tuned()
+    big = gen(40, 200, seed=5, dtype=BF).to(DEV)
+    a = big[:, 16:16 + 72]                              # row stride 200, offset 32 bytes
+    w = gen(50, 72, seed=6, dtype=BF).to(DEV)
+    wide = torch.full((40, 64), 3.0, dtype=BF, device=DEV)
+    out = wide[:, 8:58]                                 # out is a view too: columns beside it must stay
+    t.gemm_bf16(a, w, out)
+    check(f64(out), f64(a) @ f64(w).T, BF)
+    assert (wide[:, :8] == 3.0).all() and (wide[:, 58:] == 3.0).all()
+
+
+def test_sizes_the_mfma_kernels_refuse_go_to_the_plain_kernel():
+    t = tuned()
+    a, w = gen(5, 13, seed=1, dtype=BF).to(DEV), gen(7, 13, seed=2, dtype=BF).to(DEV)   # K = 13
+    out = torch.empty(5, 7, dtype=BF, device=DEV)
+    t.gemm_bf16(a, w, out)
+    check(f64(out), f64(a) @ f64(w).T, BF)
+
+
+def test_skinny_rows_together_equal_each_row_alone():
+    """A decoded row is the same alone and in any batch of up to 16 rows, bit for bit."""
+    t = tuned()
+    for N, K in [(4096, 512), (100, 1208), (33, 72)]:
+        a, w = gen(16, K, seed=3, dtype=BF).to(DEV), gen(N, K, seed=4, dtype=BF).to(DEV)
+        tog = torch.empty(16, N, dtype=torch.float32, device=DEV)
+        t.gemm_bf16(a, w, tog)
+        for r in (0, 7, 15):
+            alone = torch.empty(1, N, dtype=torch.float32, device=DEV)
+            t.gemm_bf16(a[r:r + 1], w, alone)
+            assert torch.equal(alone[0], tog[r])
+        some = torch.empty(5, N, dtype=torch.float32, device=DEV)
+        t.gemm_bf16(a[3:8], w, some)
+        assert torch.equal(some, tog[3:8])
+
+
+@pytest.mark.parametrize("M,F,K", [(1, 24, 64), (8, 176, 64), (9, 200, 120), (64, 512, 192), (65, 40, 72),
+                                   (130, 200, 120), (300, 512, 192), (256, 14336 // 8, 512)])
+def test_swiglu_bf16(M, F, K):
+    t = tuned()
+    h = gen(M, K, seed=1, dtype=BF).to(DEV)
+    w = gen(2 * F, K, seed=2, scale=0.3, dtype=BF).to(DEV)
+    out = torch.empty(M, F, dtype=BF, device=DEV)
+    t.swiglu_bf16(h, w, out)
+    g = f64(h) @ f64(w[:F]).T
+    u = f64(h) @ f64(w[F:]).T
+    check(f64(out), P.silu(g) * u, BF)
+
+
+def run_attention(H, Hk, d, P_, lens, rows_per_seg, window=0, seed=0):
+    """Sequences of `lens` keys in the cache; the last `rows_per_seg[s]` positions of sequence s are the step's rows."""
+    from allpaca_amd.engine.batch import Entry, pack_step
+    t = tuned()
+    cache, bt, ks, vs = make_cache(lens, Hk, d, P_, BF, seed=seed)
+    pos0 = [n - r for n, r in zip(lens, rows_per_seg)]
+    entries = [Entry(i, [0] * r, []) for i, r in enumerate(rows_per_seg)]
+    tables = [[list(bt[i, : -(-n // P_)].cpu().numpy()) for i, n in enumerate(lens)]]
+    step = pack_step(entries, pos0, [0] * len(lens), tables, torch.device(DEV), [0])
+    T = sum(rows_per_seg)
+    # queries scaled up: scores of deviation ~2.5, so a few keys carry each row and a wrong or missing one shows
+    q = gen(T, H * d + 16, seed=seed + 7, scale=2.5, dtype=BF).to(DEV)
+    out = torch.zeros(T, H * d, dtype=BF, device=DEV)
+    assert t.attention_bf16(q, 16, out, H, Hk, d, cache, P_, step.block_tables[0], step, window=window)
+    got = f64(out).reshape(T, H, d)
+    q64 = f64(q)[:, 16:].reshape(T, H, d)
+    at = 0
+    for s, r in enumerate(rows_per_seg):
+        want = P.attention(q64[at:at + r], f64(ks[s]), f64(vs[s]), H, Hk, window=window or None)
+        d_ = np.abs(got[at:at + r] - want)
+        # P and the output are rounded to bfloat16: 2^-8 of the largest value that enters a sum
+        tol = 2.0 ** -7 * np.abs(f64(vs[s])).max() * 0.25 + 2.0 ** -8 * np.abs(want)
+        assert (d_ <= tol).all(), (f"segment {s} rows {r}: max diff {d_.max():.3e} at "
+                                   f"{np.unravel_index((d_ - tol).argmax(), d_.shape)}")
+        at += r
+
+
+@pytest.mark.parametrize("d", [16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 256])
+def test_attention_every_head_size(d):
+    run_attention(H=4, Hk=2, d=d, P_=16, lens=[150, 70, 33], rows_per_seg=[150, 1, 5], seed=d)
+
+
+@pytest.mark.parametrize("H,Hk", [(1, 1), (3, 3), (5, 1), (6, 2), (32, 8), (20, 1), (34, 2)])
+def test_attention_heads_and_groups(H, Hk):
+    # 20:1 and 17:1 groups are wider than one 16-row MFMA tile
+    run_attention(H=H, Hk=Hk, d=32, P_=16, lens=[100, 260, 64], rows_per_seg=[1, 1, 64], seed=H)
+
+
+@pytest.mark.parametrize("P_", [8, 16, 24, 32, 64, 128])
+def test_attention_page_sizes(P_):
+    run_attention(H=4, Hk=1, d=64, P_=P_, lens=[300, 129, 64, 1], rows_per_seg=[1, 129, 2, 1], seed=P_)
+
+
+@pytest.mark.parametrize("window", [1, 5, 64, 100, 1000])
+def test_attention_windows(window):
+    run_attention(H=4, Hk=2, d=32, P_=16, lens=[300, 200, 90], rows_per_seg=[1, 200, 17], window=window, seed=window)
+
+
+def test_attention_long_context_decode_and_portion_over_history():
+    # the reference's long rows (crates/allpaca-hip/src/lib.rs:23162-23175: 3000 and 1300 keys) and a portion
+    # of 70 rows over 2,000 keys of history
+    run_attention(H=4, Hk=2, d=128, P_=16, lens=[3000, 1300, 2070], rows_per_seg=[1, 2, 70], seed=1)
+    run_attention(H=8, Hk=8, d=128, P_=16, lens=[5000] + [40] * 7, rows_per_seg=[1] * 8, seed=2)
+
+
+def test_attention_finds_a_far_key_in_every_path():
+    t = tuned()
+    from allpaca_amd.engine.batch import Entry, pack_step
+    H, Hk, d, P_, n = 4, 2, 64, 16, 900
+    for rows in (1, 40):
+        cache, bt, ks, vs = make_cache([n], Hk, d, P_, BF, seed=9)
+        key = 17
+        page, slot = int(bt[0, key // P_]), key % P_
+        cache[page, 0, :, slot] = 0.0
+        cache[page, 0, :, slot, 5] = 30.0
+        q = torch.zeros(rows, H * d, dtype=BF, device=DEV)
+        for h in range(H):
+            q[-1, h * d + 5] = 30.0
+        step = pack_step([Entry(0, [0] * rows, [])], [n - rows], [0],
+                         [[list(bt[0, : -(-n // P_)].cpu().numpy())]], torch.device(DEV), [0])
+        out = torch.zeros(rows, H * d, dtype=BF, device=DEV)
+        assert t.attention_bf16(q, 0, out, H, Hk, d, cache, P_, step.block_tables[0], step)
+        for h in range(H):
+            want = vs[0][key, h // 2].float()
+            assert torch.allclose(out[-1, h * d:(h + 1) * d].float().cpu(), want, atol=2.0 ** -7 * 4)
