@@ -37,7 +37,8 @@ class Engine:
         num_pages = cfg.num_pages or -(-cfg.max_tokens // cfg.page_tokens)
         self.model_config, self.model = load_model(model, dtype, cfg.device,
                                                    max_positions=num_pages * cfg.page_tokens)
-        self.runner = ModelRunner(self.model, cfg.page_tokens, num_pages, cfg.max_active_requests)
+        self.runner = ModelRunner(self.model, cfg.page_tokens, num_pages, cfg.max_active_requests,
+                                  use_graphs=cfg.use_graphs)
         self.scheduler = Scheduler(self.runner.cache, cfg.max_active_requests, cfg.max_batch_tokens, cfg.chunk_tokens)
         self.sampler = Sampler(self.runner.rt.device, cfg.seed)
         self.requests: Dict[int, Request] = {}

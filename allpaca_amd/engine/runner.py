@@ -9,8 +9,9 @@ mixes a prompt portion with decode rows in one of them
 (crates/allpaca-core/src/engine.rs:5451-5607); this is the one generalisation."""
 from __future__ import annotations
 
-from typing import Dict, Hashable, List, Optional, Sequence
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from ..cache import CacheManager, CacheStorage, OutOfPages, PagedView, StateView
@@ -24,7 +25,7 @@ class StepError(ValueError):
 
 class ModelRunner:
     def __init__(self, model: DecoderModel, page_tokens: int, num_pages, max_requests: int,
-                 kv_dtype: Optional[torch.dtype] = None):
+                 kv_dtype: Optional[torch.dtype] = None, use_graphs: bool = False):
         if model.rt is None:
             raise StepError("the model has no weights bound")
         self.model = model
@@ -34,6 +35,10 @@ class ModelRunner:
         self.views = self.storage.views(model.spec.plan)
         self.pad_pages = [self.storage.dummy_page(g) for g in range(len(self.cache.paged_groups))]
         self.vocab_size = model.spec.vocab_size
+        # decode-only steps are replayed as HIP graphs when every mixer of the model allows it
+        self.use_graphs = bool(use_graphs) and all(getattr(b.mixer, "graph_safe", False) for b in model.blocks)
+        self.graphs: Dict[Tuple[int, int], "DecodeGraph"] = {}
+        self.graph_replays = 0
         self.steps = 0
 
     # ---- requests ------------------------------------------------------------
@@ -85,8 +90,11 @@ class ModelRunner:
                 raise OutOfPages(f"the step needs {n} new pages in group {g}, {self.cache.free_pages(g)} are free")
         for e in entries:
             self.cache.reserve(e.seq, len(e.tokens))
-        info = self.pack(entries)
-        logits = self.model.forward(info, self.bind_views(info))
+        if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+            logits = self.graph_step(entries)
+        else:
+            info = self.pack(entries)
+            logits = self.model.forward(info, self.bind_views(info))
         for e in entries:
             self.cache.commit(e.seq, len(e.tokens))
         self.steps += 1
@@ -106,3 +114,103 @@ class ModelRunner:
                 v.slots = info.state_slots
                 v.slots_host = info.host_slots
         return self.views
+
+    # ---- decode-only steps as HIP graphs -----------------------------------------------
+    def graph_step(self, entries: Sequence[Entry]) -> torch.Tensor:
+        """A step in which every request brings one token and wants its logits: the launches of the whole
+        model are replayed from a graph captured for (rows rounded up to a power of two, context rounded
+        up to a power of two); only the batch description is copied in."""
+        n = len(entries)
+        rows = 1 << max(0, (n - 1).bit_length())
+        longest = max(self.cache.length(e.seq) for e in entries) + 1
+        span = max(256, 1 << (longest - 1).bit_length())
+        span = min(span, -(-self.rt.max_positions // self.cache.page_tokens) * self.cache.page_tokens)
+        span = max(span, longest)
+        key = (rows, span)
+        g = self.graphs.get(key)
+        if g is None:
+            g = self.graphs[key] = DecodeGraph(self, rows, span)
+        g.fill(entries)
+        g.replay()
+        self.graph_replays += 1
+        return g.logits[:n]
+
+
+class DecodeGraph:
+    """The launches of one decode step for `rows` single-token requests whose contexts fit `span` positions.
+    Rows beyond the live requests are padding: token 0 at position 0 of the spare page and the spare slot."""
+
+    def __init__(self, runner: ModelRunner, rows: int, span: int):
+        self.runner, self.rows, self.span = runner, rows, span
+        cache = runner.cache
+        self.widths = [-(-span // cache.page_tokens) for _ in cache.paged_groups]
+        # layout of the int32 description: tokens, positions, row_seg, seg_row0, seg_rows, seg_pos0, slots,
+        # logit_rows, then one [rows, width] block table per paged group
+        sizes = [rows] * 8 + [rows * w for w in self.widths]
+        self.cuts = np.cumsum([0] + sizes)
+        dev = runner.rt.device
+        self.host = torch.zeros(int(self.cuts[-1]), dtype=torch.int32).pin_memory()
+        self.np = self.host.numpy()
+        self.dev = torch.zeros(int(self.cuts[-1]), dtype=torch.int32, device=dev)
+        ar = np.arange(rows, dtype=np.int32)
+        self._part(2)[:] = ar          # row_seg
+        self._part(3)[:] = ar          # seg_row0
+        self._part(4)[:] = 1           # seg_rows
+        self._part(7)[:] = ar          # logit_rows
+        v = [self.dev[self.cuts[i]: self.cuts[i + 1]] for i in range(len(sizes))]
+        self.info = StepInfo(
+            n_rows=rows, n_segs=rows, tokens=v[0], positions=v[1], row_seg=v[2], seg_row0=v[3], seg_rows=v[4],
+            seg_pos0=v[5], state_slots=v[6], logit_rows=v[7], n_logit_rows=rows,
+            block_tables=[v[8 + g].view(rows, w) for g, w in enumerate(self.widths)],
+            host_row0=list(range(rows)), host_rows=[1] * rows, host_pos0=[0] * rows, host_slots=[0] * rows,
+            max_context=span, max_rows=1, decode_only=True, decode_rows=None, n_decode_rows=rows,
+            max_decode_context=span, n_tiles=0)
+        self.copied = torch.cuda.Event()
+        self.fill([])
+        views = runner.bind_views(self.info)
+        # one eager run on a side stream (allocations settle), then the capture
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            runner.model.forward(self.info, views)
+        torch.cuda.current_stream(dev).wait_stream(side)
+        torch.cuda.synchronize(dev)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.logits = runner.model.forward(self.info, views)
+        torch.cuda.synchronize(dev)
+
+    def _part(self, i: int) -> np.ndarray:
+        return self.np[self.cuts[i]: self.cuts[i + 1]]
+
+    def fill(self, entries: Sequence[Entry]) -> None:
+        r = self.runner
+        cache = r.cache
+        n = len(entries)
+        self.copied.synchronize()      # the last upload has read the pinned buffer
+        tokens, positions, pos0, slots = self._part(0), self._part(1), self._part(5), self._part(6)
+        tokens[n:] = 0
+        positions[n:] = 0
+        pos0[n:] = 0
+        slots[n:] = cache.max_requests
+        for i, e in enumerate(entries):
+            tokens[i] = e.tokens[0]
+            positions[i] = pos0[i] = cache.length(e.seq)
+            slots[i] = cache.slot_of(e.seq)
+        for g, w in enumerate(self.widths):
+            bt = self._part(8 + g).reshape(self.rows, w)
+            pad = r.pad_pages[g]
+            bt[n:] = pad
+            for i, e in enumerate(entries):
+                t = cache.block_table(e.seq, g)
+                k = len(t)
+                row = bt[i]
+                row[:k] = t
+                row[k:] = pad
+                if cache.paged_groups[g].need.window is not None:
+                    row[:k][row[:k] < 0] = pad
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+
+    def replay(self) -> None:
+        self.graph.replay()

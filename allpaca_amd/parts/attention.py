@@ -19,6 +19,8 @@ from .spec import ParamSpec, PartSpec
 
 @MIXERS.register("attention")
 class Attention(Mixer):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: Optional[PartSpec] = None, window: Optional[int] = None, scale: Optional[float] = None):
         if num_heads % num_kv_heads:

@@ -94,6 +94,11 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    # True if `forward_add` only launches kernels whose arguments stay valid when the step's device
+    # buffers are refilled (nothing read back to the host, no host-side branching on the batch): such a
+    # mixer's decode steps can be replayed as a HIP graph
+    graph_safe = False
+
     def cache_need(self) -> CacheNeed:
         return None
 

@@ -1,0 +1,230 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on Llama-3.1-8B shapes with random weights.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 2048] [--layers L]
+
+A step is one decode step of the whole engine (schedule, batch upload, model, sampling, token ids back).
+Prints one JSON line: `value` = decoded tokens per second at the given batch; `prefill` = a 2,048-token
+prompt in one step; `roofline` = bytes a decode step has to read (every weight once, and the cache of the
+live requests) over its time, against 8 TB/s; `points` = decode at batch 1 and 64.  The way of reporting
+follows the reference's bench tool (bytes per token, effective GB/s, share of the peak:
+tools/bench/src/roofline.rs:35-70).  Peaks: MI355X HBM3E 8 TB/s; dense bf16 MFMA 2.5 PFLOP/s."""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+
+def build_engine(cfg_json, dtype, batch, context, extra_tokens, layers, seed=0, use_graphs=True):
+    """An engine on random weights made directly on the GPU (no model folder is written for 16 GB)."""
+    import torch
+
+    from allpaca_amd.cache import CacheManager  # noqa: F401
+    from allpaca_amd.config import EngineConfig
+    from allpaca_amd.engine.engine import Engine
+    from allpaca_amd.engine.runner import ModelRunner
+    from allpaca_amd.engine.scheduler import Scheduler
+    from allpaca_amd.models import DecoderModel, describe_model
+    from allpaca_amd.parts import Runtime
+    from allpaca_amd.sampling.sampler import Sampler
+    from allpaca_amd.weights import random_tensors
+
+    cfg_json = dict(cfg_json, num_hidden_layers=layers)
+    _, cfg, spec = describe_model(cfg_json)
+    model = DecoderModel(spec)
+    tdt = torch.bfloat16 if dtype == "bf16" else torch.float32
+    page = 16
+    per_seq = -(-(context + extra_tokens) // page) * page
+    ec = EngineConfig(dtype="bfloat16" if dtype == "bf16" else "float32", page_tokens=page,
+                      num_pages=batch * per_seq // page + 8, max_active_requests=max(batch, 1),
+                      max_batch_tokens=2048, chunk_tokens=2048, use_graphs=use_graphs)
+    rt = Runtime(torch.device("cuda:0"), tdt, per_seq)
+    # weights tensor by tensor on the GPU: nothing of 16 GB passes through host memory
+    specs = model.param_specs()
+    tensors = {}
+    for name, ps in specs.items():
+        tensors.update(random_tensors({name: ps}, seed, tdt, 0.02, 0.0, device="cuda:0"))
+    model.bind(tensors, rt)
+    del tensors
+    eng = Engine.__new__(Engine)
+    eng.config, eng.model_config, eng.model = ec, cfg, model
+    eng.runner = ModelRunner(model, ec.page_tokens, ec.num_pages, ec.max_active_requests, use_graphs=use_graphs)
+    eng.scheduler = Scheduler(eng.runner.cache, ec.max_active_requests, ec.max_batch_tokens, ec.chunk_tokens)
+    eng.sampler = Sampler(rt.device, ec.seed)
+    eng.requests, eng._next_id = {}, 0
+    eng.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0}
+    return cfg, eng
+
+
+def weight_bytes(eng):
+    import torch
+    seen, total = set(), 0
+    model = eng.model
+    mats = [model.head.weight]          # the embedding table is read row-wise (a few KB), not counted
+    for b in model.blocks:
+        for part in b.parts.values():
+            for v in vars(part).values():
+                if isinstance(v, torch.Tensor) and v.dim() >= 1:
+                    mats.append(v)
+    for t in mats:
+        if t.data_ptr() not in seen:
+            seen.add(t.data_ptr())
+            total += t.numel() * t.element_size()
+    return total
+
+
+def kv_bytes_per_token(cfg, layers, elem=2):
+    return layers * 2 * cfg.num_key_value_heads * cfg.head_dim * elem
+
+
+def decode_run(eng, cfg, batch, context, steps, warmup):
+    """Fills `batch` requests to `context` tokens, then times `steps` decode steps."""
+    import numpy as np
+    import torch
+
+    from allpaca_amd.sampling import GenerationParams
+    rng = np.random.default_rng(0)
+    # requests that finish their prompt first decode while the others still prefill: leave room for that
+    gp = GenerationParams(max_tokens=warmup + steps + 2 * batch + 8, temperature=0.0)
+    for _ in range(batch):
+        eng.add_request(rng.integers(0, cfg.vocab_size, size=context - 1).tolist(), gp)
+    while any(not r.decoding for r in eng.scheduler.running) or eng.scheduler.waiting:
+        eng.step()
+    for _ in range(warmup):
+        eng.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n = 0
+    for _ in range(steps):
+        n += len(eng.step())
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert n == batch * steps, f"{n} tokens from {steps} steps of batch {batch}"
+    for rid in list(eng.requests):
+        eng.abort(rid)
+    return dt / steps
+
+
+def prefill_run(eng, cfg, tokens, repeats=3):
+    """One prompt of `tokens` tokens in one step (logits of its last row), best of `repeats`."""
+    import numpy as np
+    import torch
+
+    from allpaca_amd.engine.batch import Entry
+    rng = np.random.default_rng(1)
+    best = None
+    for i in range(repeats + 1):
+        toks = rng.integers(0, cfg.vocab_size, size=tokens).tolist()
+        eng.runner.admit(("prefill", i))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.runner.step([Entry(("prefill", i), toks, [tokens - 1])])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        eng.runner.release(("prefill", i))
+        if i > 0:
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def prefill_flops(cfg, layers, T):
+    D, F, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    H, Hk, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    linear = 2 * T * D * ((H + 2 * Hk) * d + H * d) + 2 * T * D * 3 * F
+    attn = 2 * 2 * H * d * (T * (T + 1) // 2)
+    return layers * (linear + attn) + 2 * D * V
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=2048)
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0: all)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--preset", default="llama-3.1-8b")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points and the prefill")
+    ap.add_argument("--no-graphs", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
+        return 2
+
+    import torch
+
+    from allpaca_amd.config import preset
+    from allpaca_amd.kernels import lib as klib
+    cfg_json = preset(args.preset)
+    full_layers = cfg_json["num_hidden_layers"]
+    layers = args.layers or full_layers
+    klib.load("plain")
+    klib.load("tuned")
+
+    points = {}
+    batches = [args.batch] + ([] if args.no_points else [b for b in (1, 64) if b != args.batch])
+    ms = {}
+    prefill = None
+    roof = None
+    for b in batches:
+        extra = args.warmup + args.steps + 2 * b + 16
+        cfg, eng = build_engine(cfg_json, args.dtype, max(b, 1), args.context, extra, layers,
+                                use_graphs=not args.no_graphs)
+        sec = decode_run(eng, cfg, b, args.context, args.steps, args.warmup)
+        ms[b] = sec * 1e3
+        if b == args.batch:
+            wbytes = weight_bytes(eng)
+            ctx_mid = args.context + args.warmup + args.steps // 2
+            total = wbytes + b * ctx_mid * kv_bytes_per_token(cfg, layers, 2 if args.dtype == "bf16" else 4)
+            gbs = total / sec / 1e9
+            roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(gbs / HBM_PEAK_GBS, 4)}
+            if not args.no_points:
+                T = 2048
+                psec = prefill_run(eng, cfg, T)
+                fl = prefill_flops(cfg, layers, T)
+                prefill = {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3),
+                           "frac": round(fl / psec / PEAK_FLOPS[args.dtype], 4)}
+        else:
+            points[f"decode_b{b}"] = round(b / sec, 1)
+        del eng
+        torch.cuda.empty_cache()
+
+    sec = ms[args.batch] / 1e3
+    out = {
+        "metric": "decode tok/s @ batch 8, context 2048 (Llama-3.1-8B shapes)" if (args.batch, args.context) == (8, 2048)
+        else f"decode tok/s @ batch {args.batch}, context {args.context}",
+        "value": round(args.batch / sec, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms[args.batch], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic: random N(0, 0.02) weights, uniform random token ids",
+        "config": {
+            "model": args.preset, "layers": layers, "layers_of_configuration": full_layers,
+            "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+            "rope_theta": cfg.rope_theta, "rope_scaling_factor": cfg.rope_scaling.factor if cfg.rope_scaling else 1.0,
+            "rms_norm_eps": cfg.rms_norm_eps, "tied_head": cfg.tie_word_embeddings, "global_batch": args.batch,
+            "seq_len": args.context, "page_tokens": 16, "parallelism": "single GPU",
+            "graphs": not args.no_graphs,
+        },
+    }
+    if prefill:
+        out["prefill"] = prefill
+    if roof:
+        out["roofline"] = roof
+    if points:
+        out["points"] = points
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

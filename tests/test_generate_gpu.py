@@ -193,3 +193,66 @@ def test_trace_run_program(dtype, tmp_path):
         assert row == arr.shape[0]
     for k, t in toks.items():
         H.check_logits(np.concatenate(got[k]), folder, t, dtype, f"trace mixed {k}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_equal_eager_steps(dtype):
+    """Decode-only steps replayed as HIP graphs give the logits of the same steps run eagerly: several replays of
+    each graph, with eager prefill work, other graphs and synchronisations between them, growing contexts, changing
+    numbers of live requests (so rows are padded) and page edges."""
+    from allpaca_amd.engine.batch import Entry
+    from allpaca_amd.engine.runner import ModelRunner
+    from allpaca_amd.models import load_model
+    folder = H.model_folder("B", dtype, True)
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    cfg, model = load_model(folder, tdt, "cuda:0")
+    runs = {}
+    for graphs in (False, True):
+        runner = ModelRunner(model, 16, 40, 8, use_graphs=graphs)
+        toks = {i: H.random_tokens(1000, 90, seed=300 + i) for i in range(3)}
+        out = []
+        at = {}
+        for i, n0 in ((0, 5), (1, 30)):
+            runner.admit(i)
+            runner.step([Entry(i, toks[i][:n0], [])])
+            at[i] = n0
+        for s in range(40):
+            if s == 7:                                   # a third request joins: eager prefill between replays
+                runner.admit(2)
+                runner.step([Entry(2, toks[2][:17], [])])
+                at[2] = 17
+            if s == 25:                                  # and one leaves: three rows -> two of a four-row graph
+                runner.release(0)
+                del at[0]
+            batch = [Entry(i, [toks[i][p]], [0]) for i, p in sorted(at.items())]
+            lg = runner.step(batch)
+            out.append(lg.float().cpu().numpy())
+            for i in at:
+                at[i] += 1
+        runs[graphs] = out
+        if graphs:
+            assert runner.graph_replays == 40 and len(runner.graphs) >= 2
+    for a, b in zip(runs[False], runs[True]):
+        if dtype == "float32":
+            assert np.array_equal(a, b)
+        else:
+            # same kernels, but the number of key ranges a row is split into follows the graph's size
+            assert np.abs(a - b).max() <= 2.0 ** -7 * np.abs(a).max()
+    # and against the oracle
+    i, upto = 1, 30 + 40
+    toks1 = H.random_tokens(1000, 90, seed=301)
+    got = np.concatenate([r[1 if k < 25 else 0][None] for k, r in enumerate(runs[True])])
+    want_rows = list(range(30, 70))
+    noise = H.oracle_logits_bf16_storage(folder, toks1[:upto])[want_rows] if dtype == "bfloat16" else None
+    H.assert_close(got, H.oracle_logits(folder, toks1[:upto])[want_rows], dtype, "graph decode", noise)
+
+
+def test_generation_with_graphs_equals_the_plain_implementation():
+    folder = H.model_folder("A", "float32", True)
+    cfg, w = H.oracle(folder)
+    prompts = [H.random_tokens(256, n, seed=n) for n in (1, 7, 16, 33)]
+    want = [P.greedy_generate(cfg, w, p, 16) for p in prompts]
+    eng = engine_for(folder, use_graphs=True, chunk_tokens=8, max_batch_tokens=12)
+    outs = eng.generate(prompts, params(max_tokens=16, temperature=0.0))
+    assert [o.token_ids for o in outs] == want
+    assert eng.runner.graph_replays > 0
