@@ -296,37 +296,43 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   }
 }
 
-// merge of the parts of one (row, head), in key order
-__global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict__ parts, int n_parts, int KW, int H,
-                                                        int d, const int* __restrict__ positions,
-                                                        const int* __restrict__ rows, int window,
-                                                        bf16_t* __restrict__ out, int ldo) {
-  const int ri = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+// merge of the parts of one (row, head), in key order: first the weights of all parts (their maxima against
+// the overall maximum), then the weighted sum of their outputs with independent loads
+constexpr int MERGE_NT = 128;
+__global__ __launch_bounds__(MERGE_NT) void attn_merge_kernel(const float* __restrict__ parts, int n_parts, int KW,
+                                                              int H, int d, const int* __restrict__ positions,
+                                                              const int* __restrict__ rows, int window,
+                                                              bf16_t* __restrict__ out, int ldo) {
+  extern __shared__ float wgt[];  // [n_parts] weights, then 1 float: 1 / l
+  const int ri = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int row = rows ? rows[ri] : ri;
   const int pos = positions[row];
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int p_lo = ((first / 32) * 32) / KW, p_hi = pos / KW;  // parts that hold at least one visible key
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
-  for (int p = p_lo; p <= p_hi && p < n_parts; ++p) {
-    const float* src = parts + (((size_t)ri * H + h) * n_parts + p) * (d + 2);
-    const float pm = src[d], pl = src[d + 1];
-    if (pm == -INFINITY) continue;
-    const float m_new = fmaxf(m, pm);
-    const float a = __expf(m - m_new), b = __expf(pm - m_new);
-    l = l * a + pl * b;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int e = lane + i * WAVE;
-      if (e < d) acc[i] = acc[i] * a + src[e] * b;
-    }
-    m = m_new;
+  const int p_lo = ((first / 32) * 32) / KW, p_hi = min(pos / KW, n_parts - 1);  // parts with a visible key
+  const int np = p_hi - p_lo + 1;
+  const float* base = parts + (((size_t)ri * H + h) * n_parts + p_lo) * (d + 2);
+  for (int p = tid; p < np; p += MERGE_NT) wgt[p] = base[(size_t)p * (d + 2) + d];  // the parts' maxima
+  __syncthreads();
+  float m = -INFINITY;
+  for (int p = 0; p < np; ++p) m = fmaxf(m, wgt[p]);
+  __syncthreads();
+  for (int p = tid; p < np; p += MERGE_NT) {
+    const float pm = wgt[p];
+    wgt[p] = pm == -INFINITY ? 0.f : __expf(pm - m);
   }
-  const float inv = 1.0f / l;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int e = lane + i * WAVE;
-    if (e < d) out[(size_t)row * ldo + (size_t)h * d + e] = float_to_bf16(acc[i] * inv);
+  __syncthreads();
+  if (tid == 0) {
+    float l = 0.f;
+    for (int p = 0; p < np; ++p) l += base[(size_t)p * (d + 2) + d + 1] * wgt[p];
+    wgt[np] = 1.0f / l;
+  }
+  __syncthreads();
+  const float inv = wgt[np];
+  for (int e = tid; e < d; e += MERGE_NT) {
+    float acc = 0.f;
+#pragma unroll 8
+    for (int p = 0; p < np; ++p) acc = fmaf(base[(size_t)p * (d + 2) + e], wgt[p], acc);
+    out[(size_t)row * ldo + (size_t)h * d + e] = float_to_bf16(acc * inv);
   }
 }
 
@@ -390,8 +396,8 @@ APC_EXPORT int apc_attention_decode_bf16(const void* q, int ldq, int q_off, void
   else DC_LAUNCH(256);
 #undef DC_LAUNCH
   APC_LAUNCH_CHECK();
-  hipLaunchKernelGGL(attn_merge_kernel, dim3(n_rows, H), dim3(64), 0, stream, workspace, n_parts, keys_per_part, H, d,
-                     positions, rows, window, (bf16_t*)out, ldo);
+  hipLaunchKernelGGL(attn_merge_kernel, dim3(n_rows, H), dim3(MERGE_NT), (n_parts + 1) * sizeof(float), stream,
+                     workspace, n_parts, keys_per_part, H, d, positions, rows, window, (bf16_t*)out, ldo);
   APC_LAUNCH_CHECK();
   return 0;
 }

@@ -72,12 +72,76 @@ __global__ void rmsnorm_rows_kernel(const void* __restrict__ x, int x_dtype, int
   }
 }
 
+// The same for float32 rows whose width is a multiple of 4 and at most NT*4*VPT: every thread keeps its
+// elements in registers between the sum and the scaling, and all its loads are in flight together.
+// Which of the two kernels runs, and so the order of the additions, is fixed by the width and the
+// alignment of the rows alone, never by the batch.
+template <int NT, int VPT>
+__global__ __launch_bounds__(NT) void rmsnorm_rows_f32_kernel(const float* __restrict__ x, int ldx,
+                                                              const int* __restrict__ rows,
+                                                              const float* __restrict__ w, float eps,
+                                                              void* __restrict__ out, int out_dtype, int ldo,
+                                                              int dim) {
+  __shared__ float red[NT / WAVE];
+  const int r = blockIdx.x;
+  const float4* src = reinterpret_cast<const float4*>(x + (size_t)(rows ? rows[r] : r) * ldx);
+  const int n4 = dim / 4;
+  float4 v[VPT];
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = threadIdx.x + j * NT;
+    v[j] = i < n4 ? src[i] : float4{0.f, 0.f, 0.f, 0.f};
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    ss = fmaf(v[j].x, v[j].x, ss);
+    ss = fmaf(v[j].y, v[j].y, ss);
+    ss = fmaf(v[j].z, v[j].z, ss);
+    ss = fmaf(v[j].w, v[j].w, ss);
+  }
+  ss = block_sum<NT>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
+  const float4* w4 = reinterpret_cast<const float4*>(w);
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = threadIdx.x + j * NT;
+    if (i >= n4) continue;
+    const float4 g = w4[i];
+    const float o0 = (v[j].x * inv) * g.x, o1 = (v[j].y * inv) * g.y, o2 = (v[j].z * inv) * g.z,
+                o3 = (v[j].w * inv) * g.w;
+    const size_t at = (size_t)r * ldo + (size_t)i * 4;
+    if (out_dtype == APC_F32) {
+      *reinterpret_cast<float4*>((float*)out + at) = float4{o0, o1, o2, o3};
+    } else {
+      uint2 pk;
+      pk.x = (uint32_t)float_to_bf16(o0) | ((uint32_t)float_to_bf16(o1) << 16);
+      pk.y = (uint32_t)float_to_bf16(o2) | ((uint32_t)float_to_bf16(o3) << 16);
+      *reinterpret_cast<uint2*>((bf16_t*)out + at) = pk;
+    }
+  }
+}
+
 APC_EXPORT int apc_rmsnorm_rows(const void* x, int x_dtype, int ldx, const int* rows, const float* w, float eps,
                                 void* out, int out_dtype, int ldo, int n_rows, int dim, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (dim <= 0 || ldx < dim || ldo < dim) return APC_ERR_BAD_ARG;
-  hipLaunchKernelGGL(rmsnorm_rows_kernel<256>, dim3(n_rows), dim3(256), 0, stream, x, x_dtype, ldx, rows, w, eps, out,
-                     out_dtype, ldo, dim);
+  const bool vec = x_dtype == APC_F32 && dim % 4 == 0 && ldx % 4 == 0 && ldo % 4 == 0 && dim <= 256 * 4 * 8 &&
+                   ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)out % 16) == 0;
+  if (vec) {
+    const int n4 = dim / 4;
+#define RN_LAUNCH(VPT_)                                                                                             \
+  hipLaunchKernelGGL((rmsnorm_rows_f32_kernel<256, VPT_>), dim3(n_rows), dim3(256), 0, stream, (const float*)x, ldx, \
+                     rows, w, eps, out, out_dtype, ldo, dim)
+    if (n4 <= 256) RN_LAUNCH(1);
+    else if (n4 <= 512) RN_LAUNCH(2);
+    else if (n4 <= 1024) RN_LAUNCH(4);
+    else RN_LAUNCH(8);
+#undef RN_LAUNCH
+  } else {
+    hipLaunchKernelGGL(rmsnorm_rows_kernel<256>, dim3(n_rows), dim3(256), 0, stream, x, x_dtype, ldx, rows, w, eps,
+                       out, out_dtype, ldo, dim);
+  }
   APC_LAUNCH_CHECK();
   return 0;
 }

@@ -167,10 +167,71 @@ __global__ __launch_bounds__(SNT) void argmax_rows_kernel(const float* __restric
   }
 }
 
-APC_EXPORT int apc_argmax_rows(const float* logits, int ldl, int n_rows, int V, int* out, hipStream_t stream) {
+// Wide rows are cut into pieces so that more than one block works on a row: a first pass leaves the first
+// maximum of every piece (value, id), a second pass takes the first maximum of those.
+__global__ __launch_bounds__(SNT) void argmax_pieces_kernel(const float* __restrict__ logits, int ldl, int V, int piece,
+                                                            float* __restrict__ pv, int* __restrict__ pi) {
+  __shared__ float bv[SNT / WAVE];
+  __shared__ int bi[SNT / WAVE];
+  const float* row = logits + (size_t)blockIdx.x * ldl;
+  const int lo = blockIdx.y * piece, hi = min(V, lo + piece);
+  float best = -INFINITY;
+  int best_i = 0x7fffffff;
+  for (int i = lo + threadIdx.x; i < hi; i += SNT) {
+    const float v = row[i];
+    if (v > best) { best = v; best_i = i; }
+  }
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, WAVE);
+    const int oi = __shfl_xor(best_i, o, WAVE);
+    if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+  }
+  if (threadIdx.x % WAVE == 0) { bv[threadIdx.x / WAVE] = best; bi[threadIdx.x / WAVE] = best_i; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < SNT / WAVE; ++w)
+      if (bv[w] > best || (bv[w] == best && bi[w] < best_i)) { best = bv[w]; best_i = bi[w]; }
+    pv[(size_t)blockIdx.x * gridDim.y + blockIdx.y] = best;
+    pi[(size_t)blockIdx.x * gridDim.y + blockIdx.y] = best_i;
+  }
+}
+
+__global__ __launch_bounds__(WAVE) void argmax_final_kernel(const float* __restrict__ pv, const int* __restrict__ pi,
+                                                            int pieces, int* __restrict__ out) {
+  float best = -INFINITY;
+  int best_i = 0x7fffffff;
+  for (int p = threadIdx.x; p < pieces; p += WAVE) {
+    const float v = pv[(size_t)blockIdx.x * pieces + p];
+    const int i = pi[(size_t)blockIdx.x * pieces + p];
+    if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
+  }
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, WAVE);
+    const int oi = __shfl_xor(best_i, o, WAVE);
+    if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;
+}
+
+// `scratch`: room for 2 * n_rows * 64 four-byte values, or null for the one-pass kernel
+APC_EXPORT int apc_argmax_rows(const float* logits, int ldl, int n_rows, int V, int* out, void* scratch,
+                               hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (V <= 0 || ldl < V) return APC_ERR_BAD_ARG;
-  hipLaunchKernelGGL(argmax_rows_kernel, dim3(n_rows), dim3(SNT), 0, stream, logits, ldl, V, out);
+  if (!scratch || V < 8192 || n_rows > 65535) {
+    hipLaunchKernelGGL(argmax_rows_kernel, dim3(n_rows), dim3(SNT), 0, stream, logits, ldl, V, out);
+    APC_LAUNCH_CHECK();
+    return 0;
+  }
+  const int pieces = 64;
+  const int piece = ceil_div(V, pieces);
+  float* pv = (float*)scratch;
+  int* pi = (int*)scratch + (size_t)n_rows * pieces;
+  hipLaunchKernelGGL(argmax_pieces_kernel, dim3(n_rows, pieces), dim3(SNT), 0, stream, logits, ldl, V, piece, pv, pi);
+  APC_LAUNCH_CHECK();
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(n_rows), dim3(WAVE), 0, stream, pv, pi, pieces, out);
   APC_LAUNCH_CHECK();
   return 0;
 }

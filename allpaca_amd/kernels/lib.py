@@ -33,7 +33,7 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_cast": [P, I, P, I, Z, P],
         "apc_gemm_plain": [P, I, I, P, I, I, P, I, I, I, I, I, I, P],
         "apc_paged_attention_plain": [P, I, I, I, P, I, I, I, I, I, I, P, I, I, P, I, P, P, I, F, P],
-        "apc_argmax_rows": [P, I, I, I, P, P],
+        "apc_argmax_rows": [P, I, I, I, P, P, P],
         "apc_sample_rows": [P, I, I, I, P, P, P, P, P, P],
     },
     "tuned": {

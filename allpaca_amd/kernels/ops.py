@@ -200,7 +200,9 @@ def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> None:
     R, V = logits.shape
     _need(logits.dtype == torch.float32, "logits are float32")
     L = _lib.load("plain")
-    _lib.check(L.apc_argmax_rows(logits.data_ptr(), ld, R, V, _i32(out, R, "argmax out"), _stream()), "argmax_rows")
+    scratch = torch.empty(2 * R * 64, dtype=torch.int32, device=logits.device) if V >= 8192 else None
+    _lib.check(L.apc_argmax_rows(logits.data_ptr(), ld, R, V, _i32(out, R, "argmax out"),
+                                 scratch.data_ptr() if scratch is not None else 0, _stream()), "argmax_rows")
 
 
 def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
