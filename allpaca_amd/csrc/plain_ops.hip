@@ -26,6 +26,30 @@ APC_EXPORT int apc_embed_rows(const void* table, int table_dtype, const int* tok
   return 0;
 }
 
+// The same from a bfloat16 table kept in the tiled layout of the MFMA kernels (tiles of 16 rows x 32 columns,
+// lane = (k % 32) / 8 * 16 + n % 16 holding the 8 elements k % 8; `chunks` tiles per 16-row band): a tied
+// output head and the embedding then share one buffer.
+__global__ void embed_rows_tiled_kernel(const bf16_t* __restrict__ table, int chunks, const int* __restrict__ tokens,
+                                        void* __restrict__ out, int out_dtype, int dim, int ldo) {
+  const int t = blockIdx.x;
+  const int n = tokens[t];
+  const bf16_t* band = table + (size_t)(n / 16) * chunks * 512 + (n % 16) * 8;
+  for (int k = threadIdx.x; k < dim; k += blockDim.x) {
+    const bf16_t v = band[(size_t)(k / 32) * 512 + ((k % 32) / 8) * 128 + (k % 8)];
+    store_f(out, out_dtype, (size_t)t * ldo + k, bf16_to_float(v));
+  }
+}
+
+APC_EXPORT int apc_embed_rows_tiled(const void* table, int chunks, const int* tokens, void* out, int out_dtype,
+                                    int n_tok, int dim, int ldo, hipStream_t stream) {
+  if (n_tok <= 0) return 0;
+  if (dim <= 0 || ldo < dim || chunks * 32 < dim) return APC_ERR_BAD_ARG;
+  hipLaunchKernelGGL(embed_rows_tiled_kernel, dim3(n_tok), dim3(256), 0, stream, (const bf16_t*)table, chunks, tokens,
+                     out, out_dtype, dim, ldo);
+  APC_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---------------------------------------------------------------------------
 // gather rows: out[r, :] = x[rows[r], :]   (same element type)
 // ---------------------------------------------------------------------------

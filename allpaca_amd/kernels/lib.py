@@ -25,6 +25,7 @@ class KernelError(RuntimeError):
 SIGNATURES: Dict[str, Dict[str, list]] = {
     "plain": {
         "apc_embed_rows": [P, I, P, P, I, I, I, I, P],
+        "apc_embed_rows_tiled": [P, I, P, P, I, I, I, I, P],
         "apc_gather_rows": [P, I, I, P, P, I, I, I, P],
         "apc_rmsnorm_rows": [P, I, I, P, P, F, P, I, I, I, I, P],
         "apc_add_into": [P, I, P, I, I, I, I, P],
@@ -37,10 +38,10 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_sample_rows": [P, I, I, I, P, P, P, P, P, P],
     },
     "tuned": {
-        "apc_gemm_bf16": [P, I, P, I, P, I, I, I, I, I, P],
-        "apc_gemm_swiglu_bf16": [P, I, P, P, I, P, I, I, I, I, P],
-        "apc_skinny_gemm_bf16": [P, I, P, I, P, I, I, I, I, I, P],
-        "apc_skinny_swiglu_bf16": [P, I, P, P, I, P, I, I, I, I, P],
+        "apc_gemm_bf16": [P, I, P, P, I, I, I, I, I, P],
+        "apc_gemm_swiglu_bf16": [P, I, P, P, P, I, I, I, I, P],
+        "apc_skinny_gemm_bf16": [P, I, P, P, I, I, I, I, I, P],
+        "apc_skinny_swiglu_bf16": [P, I, P, P, P, I, I, I, I, P],
         "apc_attention_prefill_bf16": [P, I, I, P, I, I, I, I, P, I, P, I, P, P, P, P, I, I, F, P],
         "apc_attention_decode_bf16": [P, I, I, P, I, I, I, I, I, P, I, P, I, P, P, P, I, F, I, I, P, P],
     },

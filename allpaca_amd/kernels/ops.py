@@ -11,6 +11,7 @@ from typing import Optional
 import torch
 
 from . import lib as _lib
+from .packing import PackedWeight
 
 F32, BF16, I32 = 0, 1, 2
 _CODES = {torch.float32: F32, torch.bfloat16: BF16, torch.int32: I32}
@@ -53,10 +54,18 @@ def _i32(t: Optional[torch.Tensor], n: int, what: str) -> int:
 
 
 # --------------------------------------------------------------------------- plain library
-def embed_rows(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
-    _gpu(table, tokens, out)
+def embed_rows(table, tokens: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t] = table[tokens[t]]; the table is a [vocab, dim] matrix or its tiled form (`PackedWeight`)."""
     T = tokens.numel()
     ldo = _rows(out, "embed out")
+    if isinstance(table, PackedWeight):
+        _gpu(table.data, tokens, out)
+        _need(out.shape == (T, table.K), "embed out must be [tokens, dim]")
+        L = _lib.load("plain")
+        _lib.check(L.apc_embed_rows_tiled(table.data.data_ptr(), table.chunks, _i32(tokens, T, "tokens"),
+                                          out.data_ptr(), _code(out), T, table.K, ldo, _stream()), "embed_rows_tiled")
+        return
+    _gpu(table, tokens, out)
     _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be a contiguous [vocab, dim] matrix")
     _need(out.shape[0] == T and out.shape[1] == table.shape[1], "embed out must be [tokens, dim]")
     L = _lib.load("plain")
@@ -229,20 +238,30 @@ def _tuned_ok(*ts: torch.Tensor) -> bool:
     return (not FORCE_PLAIN) and all(t.dtype == torch.bfloat16 for t in ts)
 
 
-def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
-    """out = a . w^T (or out += ..., out float32).  bfloat16 operands run on the MFMA kernels."""
-    if _tuned_ok(a, w):
+def prepare_matrix(w: torch.Tensor, run_dtype: torch.dtype):
+    """How a weight matrix [out, in] is kept on the GPU: a bfloat16 matrix of a bfloat16 run in the tiled layout
+    of the MFMA kernels (if its width is a multiple of 8), anything else as it is."""
+    from .packing import can_pack, pack_mfma
+    if run_dtype == torch.bfloat16 and not FORCE_PLAIN and w.is_cuda and can_pack(w):
+        return pack_mfma(w)
+    return w.contiguous()
+
+
+def linear(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False) -> None:
+    """out = a . w^T (or out += ..., out float32).  A tiled bfloat16 weight runs on the MFMA kernels."""
+    if isinstance(w, PackedWeight):
         from . import tuned
         tuned.gemm_bf16(a, w, out, accumulate)
     else:
         gemm_plain(a, w, out, accumulate)
 
 
-def swiglu(h: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) -> None:
-    """out[t, f] = silu(h . Wg[f]) * (h . Wu[f]) with w_gate_up = [Wg; Wu] of shape [2F, D]."""
-    if _tuned_ok(h, w_gate_up, out):
+def swiglu(h: torch.Tensor, w_gate_up, out: torch.Tensor) -> None:
+    """out[t, f] = silu(h . Wg[f]) * (h . Wu[f]); w_gate_up is [Wg; Wu] of shape [2F, D], or the pair of
+    their tiled forms."""
+    if isinstance(w_gate_up, tuple):
         from . import tuned
-        tuned.swiglu_bf16(h, w_gate_up, out)
+        tuned.swiglu_bf16(h, w_gate_up[0], w_gate_up[1], out)
         return
     T, F = out.shape
     gu = torch.empty((T, 2 * F), dtype=torch.float32 if h.dtype == torch.float32 else out.dtype, device=h.device)

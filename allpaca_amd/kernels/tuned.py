@@ -1,7 +1,9 @@
-"""Checked wrappers of the bfloat16 MFMA kernels (library `tuned`).  Each checks what the
-kernel assumes; a size a kernel does not take (a width that is no multiple of 8, a page size
-that is no multiple of 8, a head size that is no multiple of 16 or above 256) goes to the
-plain kernel of the same operation instead, never to a wrong result."""
+"""Checked wrappers of the bfloat16 MFMA kernels (library `tuned`).  Each checks what the kernel
+assumes.  Matrix products take weights in the tiled layout (`packing.PackedWeight`), which only
+matrices of a width that is a multiple of 8 get (`ops.prepare_matrix`): other widths stay row-major
+and run on the plain kernel.  Attention returns False for sizes it does not take (a page size that is
+no multiple of 8, a head size that is no multiple of 16 or above 256) and the caller runs the plain
+kernel: never a wrong result."""
 from __future__ import annotations
 
 import math
@@ -11,6 +13,7 @@ import torch
 
 from . import lib as _lib
 from . import ops as _ops
+from .packing import PackedWeight
 
 SKINNY_MAX_ROWS = 64
 
@@ -19,47 +22,47 @@ def _aligned(*ts: torch.Tensor) -> bool:
     return all(t.data_ptr() % 16 == 0 for t in ts)
 
 
-def _mfma_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
-    K = a.shape[1]
-    return (K % 8 == 0 and _ops._rows(a, "a") % 8 == 0 and _ops._rows(w, "w") % 8 == 0 and _aligned(a, w)
-            and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16)
+def _act_ok(a: torch.Tensor) -> bool:
+    return (a.dtype == torch.bfloat16 and a.shape[1] % 8 == 0 and _ops._rows(a, "a") % 8 == 0 and _aligned(a))
 
 
-def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
-    """out = a . w^T (bfloat16 or float32 out), or out += a . w^T (float32 out)."""
-    _ops._gpu(a, w, out)
+def gemm_bf16(a: torch.Tensor, w: PackedWeight, out: torch.Tensor, accumulate: bool = False) -> None:
+    """out = a . w^T (bfloat16 or float32 out), or out += a . w^T (float32 out); w in the tiled layout."""
+    _ops._gpu(a, w.data, out)
     M, K = a.shape
-    N = w.shape[0]
-    _ops._need(w.shape[1] == K, f"gemm: a is [*, {K}] but w is {tuple(w.shape)}")
+    N = w.N
+    _ops._need(w.K == K, f"gemm: a is [*, {K}] but w is {w.shape}")
     _ops._need(out.shape == (M, N), f"gemm: out must be [{M}, {N}], got {tuple(out.shape)}")
     _ops._need(not accumulate or out.dtype == torch.float32, "gemm: accumulation needs a float32 destination")
-    if not _mfma_ok(a, w) or out.dtype not in (torch.bfloat16, torch.float32):
-        return _ops.gemm_plain(a, w, out, accumulate)
-    lda, ldw, ldc = _ops._rows(a, "a"), _ops._rows(w, "w"), _ops._rows(out, "out")
+    _ops._need(out.dtype in (torch.bfloat16, torch.float32), "gemm: out must be bfloat16 or float32")
+    _ops._need(w.data.is_contiguous() and w.data.shape[0] * 16 >= N and w.data.shape[1] * 32 >= K,
+               "gemm: the tiled weight does not cover [N, K]")
+    if not _act_ok(a):
+        raise ValueError("gemm_bf16: activations must be bfloat16 rows of a width and stride that are multiples "
+                         "of 8, 16-byte aligned")
+    lda, ldc = _ops._rows(a, "a"), _ops._rows(out, "out")
     mode = 2 if accumulate else (0 if out.dtype == torch.bfloat16 else 1)
     L = _lib.load("tuned")
     fn = L.apc_skinny_gemm_bf16 if M <= SKINNY_MAX_ROWS else L.apc_gemm_bf16
-    _lib.check(fn(a.data_ptr(), lda, w.data_ptr(), ldw, out.data_ptr(), ldc, M, N, K, mode, _ops._stream()),
+    _lib.check(fn(a.data_ptr(), lda, w.data.data_ptr(), out.data_ptr(), ldc, M, N, K, mode, _ops._stream()),
                "gemm_bf16")
 
 
-def swiglu_bf16(h: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) -> None:
-    """out[t, f] = silu(h . Wg[f]) * (h . Wu[f]), w_gate_up = [Wg; Wu] ([2F, K])."""
-    _ops._gpu(h, w_gate_up, out)
+def swiglu_bf16(h: torch.Tensor, wg: PackedWeight, wu: PackedWeight, out: torch.Tensor) -> None:
+    """out[t, f] = silu(h . Wg[f]) * (h . Wu[f]); Wg, Wu in the tiled layout."""
+    _ops._gpu(h, wg.data, wu.data, out)
     M, K = h.shape
     F = out.shape[1]
-    _ops._need(w_gate_up.shape == (2 * F, K) and w_gate_up.is_contiguous(), "swiglu: weights must be [2F, K]")
-    _ops._need(out.shape[0] == M, "swiglu: out rows differ from h rows")
-    if not _mfma_ok(h, w_gate_up) or out.dtype != torch.bfloat16:
-        gu = torch.empty((M, 2 * F), dtype=out.dtype, device=h.device)
-        _ops.gemm_plain(h, w_gate_up, gu)
-        return _ops.silu_mul(gu, out)
+    _ops._need(wg.shape == (F, K) and wu.shape == (F, K), f"swiglu: weights must both be [{F}, {K}]")
+    _ops._need(out.shape[0] == M and out.dtype == torch.bfloat16, "swiglu: out must be bfloat16 [rows, F]")
+    if not _act_ok(h):
+        raise ValueError("swiglu_bf16: activations must be bfloat16 rows of a width and stride that are multiples "
+                         "of 8, 16-byte aligned")
     lda, ldc = _ops._rows(h, "h"), _ops._rows(out, "out")
-    wg, wu = w_gate_up[:F], w_gate_up[F:]
     L = _lib.load("tuned")
     fn = L.apc_skinny_swiglu_bf16 if M <= SKINNY_MAX_ROWS else L.apc_gemm_swiglu_bf16
-    _lib.check(fn(h.data_ptr(), lda, wg.data_ptr(), wu.data_ptr(), K, out.data_ptr(), ldc, M, F, K, _ops._stream()),
-               "swiglu_bf16")
+    _lib.check(fn(h.data_ptr(), lda, wg.data.data_ptr(), wu.data.data_ptr(), out.data_ptr(), ldc, M, F, K,
+                  _ops._stream()), "swiglu_bf16")
 
 
 def _keys_per_part(n_rows: int, n_kv_heads: int, max_context: int) -> int:

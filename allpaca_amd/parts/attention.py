@@ -48,8 +48,8 @@ class Attention(Mixer):
         parts = [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
         dt = parts[0].dtype if all(p.dtype == parts[0].dtype for p in parts) else torch.float32
         # one [(H + 2 Hk) d, D] matrix: a single product gives q, k and v of a row
-        self.w_qkv = torch.cat([to_device(p, rt, dt) for p in parts], dim=0).contiguous()
-        self.w_o = to_device(tensors["o_proj.weight"], rt)
+        self.w_qkv = ops.prepare_matrix(torch.cat([to_device(p, rt, dt) for p in parts], dim=0), rt.dtype)
+        self.w_o = ops.prepare_matrix(to_device(tensors["o_proj.weight"], rt), rt.dtype)
         if self.position is not None:
             self.position.bind({}, rt)
 

@@ -22,7 +22,7 @@ class TokenEmbedding(Part):
 
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
         self.rt = rt
-        self.weight = to_device(tensors["weight"], rt)
+        self.weight = ops.prepare_matrix(to_device(tensors["weight"], rt), rt.dtype)
 
     def forward(self, tokens: torch.Tensor, out: torch.Tensor) -> None:
         ops.embed_rows(self.weight, tokens, out)
@@ -40,7 +40,7 @@ class LinearHead(Part):
 
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime, shared: Optional[torch.Tensor] = None) -> None:
         self.rt = rt
-        self.weight = shared if self.tied else to_device(tensors["weight"], rt)
+        self.weight = shared if self.tied else ops.prepare_matrix(to_device(tensors["weight"], rt), rt.dtype)
         if self.weight is None:
             raise ValueError("a tied head needs the embedding matrix")
 

@@ -28,9 +28,14 @@ class SwiGLU(FeedForward):
         self.rt = rt
         g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
         dt = g.dtype if g.dtype == u.dtype else torch.float32
-        # [2F, D]: gate rows, then up rows; one pass over h gives both branches
-        self.w_gate_up = torch.cat([to_device(g, rt, dt), to_device(u, rt, dt)], dim=0).contiguous()
-        self.w_down = to_device(tensors["down_proj.weight"], rt)
+        # one pass over h gives both branches: the pair of tiled matrices for the MFMA kernels, else
+        # [2F, D] (gate rows, then up rows)
+        wg, wu = ops.prepare_matrix(to_device(g, rt, dt), rt.dtype), ops.prepare_matrix(to_device(u, rt, dt), rt.dtype)
+        if isinstance(wg, torch.Tensor):
+            self.w_gate_up = torch.cat([wg, wu], dim=0).contiguous()
+        else:
+            self.w_gate_up = (wg, wu)
+        self.w_down = ops.prepare_matrix(to_device(tensors["down_proj.weight"], rt), rt.dtype)
 
     def forward_add(self, h: torch.Tensor, step, residual: torch.Tensor) -> None:
         act = torch.empty((h.shape[0], self.F), dtype=self.rt.dtype, device=h.device)

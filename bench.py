@@ -65,19 +65,31 @@ def build_engine(cfg_json, dtype, batch, context, extra_tokens, layers, seed=0, 
 
 
 def weight_bytes(eng):
+    """Bytes of every matrix and vector a decode step reads once (the embedding table is read row-wise, a few
+    KB, and only counts if the head shares it)."""
     import torch
+
+    from allpaca_amd.kernels.packing import PackedWeight
     seen, total = set(), 0
+
+    def add(v):
+        nonlocal total
+        if isinstance(v, PackedWeight):
+            v = v.data
+        if isinstance(v, (tuple, list)):
+            for x in v:
+                add(x)
+        elif isinstance(v, torch.Tensor) and v.dim() >= 1 and v.data_ptr() not in seen:
+            seen.add(v.data_ptr())
+            total += v.numel() * v.element_size()
+
     model = eng.model
-    mats = [model.head.weight]          # the embedding table is read row-wise (a few KB), not counted
+    add(model.head.weight)
+    add(model.final_norm.weight)
     for b in model.blocks:
         for part in b.parts.values():
             for v in vars(part).values():
-                if isinstance(v, torch.Tensor) and v.dim() >= 1:
-                    mats.append(v)
-    for t in mats:
-        if t.data_ptr() not in seen:
-            seen.add(t.data_ptr())
-            total += t.numel() * t.element_size()
+                add(v)
     return total
 
 

@@ -21,6 +21,23 @@ def tuned():
     return t
 
 
+def pack(w):
+    from allpaca_amd.kernels.packing import pack_mfma
+    return pack_mfma(w)
+
+
+def test_packing_roundtrip_and_lane_order():
+    from allpaca_amd.kernels.packing import pack_mfma, unpack_mfma
+    w = gen(50, 72, seed=1, dtype=BF)
+    p = pack_mfma(w)
+    assert tuple(p.data.shape) == (4, 3, 64, 8) and torch.equal(unpack_mfma(p), w)
+    i, c = 5, 3          # lane c*16 + i of tile (band 1, chunk 2) holds w[16 + i, 64 + 8c : 64 + 8c + 8]
+    assert torch.equal(p.data[1, 2, c * 16 + i], w[16 + i, 64 + c * 8: 72]) if False else True
+    wide = torch.zeros(64, 96, dtype=BF)
+    wide[:50, :72] = w
+    assert torch.equal(p.data[1, 2, c * 16 + i], wide[16 + i, 64 + c * 8: 64 + c * 8 + 8])
+
+
 def check(got, want, out_dtype):
     """Sums are float32 over exact bfloat16 products: the result is within float32 summation error of the
     float64 value, plus one rounding to bfloat16 if it is stored so."""
@@ -40,13 +57,14 @@ def test_gemm_bf16(M, N, K):
     t = tuned()
     a, w = gen(M, K, seed=1, dtype=BF).to(DEV), gen(N, K, seed=2, dtype=BF).to(DEV)
     want = f64(a) @ f64(w).T
+    wp = pack(w)
     for out_dtype in (BF, torch.float32):
         out = torch.full((M, N), 7.0, dtype=out_dtype, device=DEV)
-        t.gemm_bf16(a, w, out)
+        t.gemm_bf16(a, wp, out)
         check(f64(out), want, out_dtype)
     acc = gen(M, N, seed=3).to(DEV)
     before = f64(acc)
-    t.gemm_bf16(a, w, acc, accumulate=True)
+    t.gemm_bf16(a, wp, acc, accumulate=True)
     check(f64(acc) - before, want, torch.float32)
 
 
@@ -57,16 +75,20 @@ def test_gemm_bf16_strided_views_and_padding_rows_untouched():
     w = gen(50, 72, seed=6, dtype=BF).to(DEV)
     wide = torch.full((40, 64), 3.0, dtype=BF, device=DEV)
     out = wide[:, 8:58]                                 # out is a view too: columns beside it must stay
-    t.gemm_bf16(a, w, out)
+    t.gemm_bf16(a, pack(w), out)
     check(f64(out), f64(a) @ f64(w).T, BF)
     assert (wide[:, :8] == 3.0).all() and (wide[:, 58:] == 3.0).all()
 
 
-def test_sizes_the_mfma_kernels_refuse_go_to_the_plain_kernel():
-    t = tuned()
+def test_widths_the_mfma_kernels_do_not_take_stay_row_major_and_run_on_the_plain_kernel():
+    from allpaca_amd.kernels import ops
     a, w = gen(5, 13, seed=1, dtype=BF).to(DEV), gen(7, 13, seed=2, dtype=BF).to(DEV)   # K = 13
+    kept = ops.prepare_matrix(w, BF)
+    assert isinstance(kept, torch.Tensor)                   # no tiled form for this width
+    assert not isinstance(ops.prepare_matrix(gen(7, 16, dtype=BF).to(DEV), BF), torch.Tensor)
+    assert isinstance(ops.prepare_matrix(gen(7, 16).to(DEV), torch.float32), torch.Tensor)
     out = torch.empty(5, 7, dtype=BF, device=DEV)
-    t.gemm_bf16(a, w, out)
+    ops.linear(a, kept, out)
     check(f64(out), f64(a) @ f64(w).T, BF)
 
 
@@ -74,7 +96,7 @@ def test_skinny_rows_together_equal_each_row_alone():
     """A decoded row is the same alone and in any batch of up to 16 rows, bit for bit."""
     t = tuned()
     for N, K in [(4096, 512), (100, 1208), (33, 72)]:
-        a, w = gen(16, K, seed=3, dtype=BF).to(DEV), gen(N, K, seed=4, dtype=BF).to(DEV)
+        a, w = gen(16, K, seed=3, dtype=BF).to(DEV), pack(gen(N, K, seed=4, dtype=BF).to(DEV))
         tog = torch.empty(16, N, dtype=torch.float32, device=DEV)
         t.gemm_bf16(a, w, tog)
         for r in (0, 7, 15):
@@ -86,6 +108,15 @@ def test_skinny_rows_together_equal_each_row_alone():
         assert torch.equal(some, tog[3:8])
 
 
+def test_embedding_from_the_tiled_table():
+    from allpaca_amd.kernels import ops
+    table = gen(515, 120, seed=1, dtype=BF).to(DEV)
+    toks = torch.tensor([0, 514, 17, 16, 15, 17], dtype=torch.int32, device=DEV)
+    out = torch.empty(6, 120, device=DEV)
+    ops.embed_rows(pack(table), toks, out)
+    assert torch.equal(out.cpu(), table.float().cpu()[toks.cpu().long()])
+
+
 @pytest.mark.parametrize("M,F,K", [(1, 24, 64), (8, 176, 64), (9, 200, 120), (64, 512, 192), (65, 40, 72),
                                    (130, 200, 120), (300, 512, 192), (256, 14336 // 8, 512)])
 def test_swiglu_bf16(M, F, K):
@@ -93,7 +124,7 @@ def test_swiglu_bf16(M, F, K):
     h = gen(M, K, seed=1, dtype=BF).to(DEV)
     w = gen(2 * F, K, seed=2, scale=0.3, dtype=BF).to(DEV)
     out = torch.empty(M, F, dtype=BF, device=DEV)
-    t.swiglu_bf16(h, w, out)
+    t.swiglu_bf16(h, pack(w[:F].contiguous()), pack(w[F:].contiguous()), out)
     g = f64(h) @ f64(w[:F]).T
     u = f64(h) @ f64(w[F:]).T
     check(f64(out), P.silu(g) * u, BF)
