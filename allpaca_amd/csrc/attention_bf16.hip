@@ -178,6 +178,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 // ------------------------------------------------------------------------------------------ decode
 // parts[row][head][part][d + 2]: o[0..d), m, l
 template <int DP>
+struct KVRegs {
+  Frag k[2][DP / 32];  // two tiles of 16 keys
+  Frag v[DP / 16];     // 32 positions of 16 value elements per tile
+};
+
+template <int DP>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int ldq, int q_off, int H, int Hk, int d, const bf16_t* __restrict__ cache, int P,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ positions,
@@ -198,6 +204,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int* bt = block_table + (size_t)row_seg[row] * max_blocks;
   const size_t page_stride = (size_t)2 * Hk * P * d;
   const size_t head_off = (size_t)kvh * P * d, v_off = (size_t)Hk * P * d;
+  // the page ids of this wave's range of keys, one per lane, fetched once: the loads of keys and values then
+  // do not wait for a look-up in the block table (a range of KW keys spans at most 64 pages: checked by the host)
+  const int page0 = k_lo / P;
+  const int my_page = bt[min(page0 + lane, pos / P)];
 
   Frag qf[DP / 32];
   {
@@ -217,70 +227,97 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   for (int r = 0; r < 4; ++r) { mrow[r] = -INFINITY; lrow[r] = 0.f; }
   bf16_t* pw = Ps + wave * 16 * (32 + KPAD);
 
-  for (int kb = k_lo; kb < k_hi; kb += 32) {
-    // scores against 32 keys: two tiles of 16, operands straight from the pages
+  // Operands of 32 keys straight from the pages.  Nothing is loaded conditionally: a key beyond the row's own
+  // position is read from that position instead (its score is masked), an element beyond d from element 0 or
+  // d - 1 (the query is zero there; such output columns are not stored), so the loads of the next 32 keys can be
+  // in flight while these are used.
+  auto load_kv = [&](KVRegs<DP>& r, int kb) {
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const int t = min(kb + nt * 16 + li, pos);
+      const int page = __shfl(my_page, t / P - page0, WAVE);
+      const bf16_t* krow = cache + (size_t)page * page_stride + head_off + (size_t)(t % P) * d;
+#pragma unroll
+      for (int ks = 0; ks < DP / 32; ++ks) {
+        const int e = ks * 32 + lc * 8;
+        r.k[nt][ks] = load_frag(krow + (e < d ? e : 0));
+      }
+    }
+    const int tv = min(kb + lc * 8, (pos / 8) * 8);
+    const int vpage = __shfl(my_page, tv / P - page0, WAVE);
+    const bf16_t* vbase = cache + (size_t)vpage * page_stride + v_off + head_off + (tv % P);
+#pragma unroll
+    for (int dt = 0; dt < DP / 16; ++dt) r.v[dt] = load_frag(vbase + (size_t)min(dt * 16 + li, d - 1) * P);
+  };
+
+  auto step = [&](const KVRegs<DP>& r, int kb) {
     floatx4 s[2];
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
       s[nt] = floatx4{0.f, 0.f, 0.f, 0.f};
-      const int t = kb + nt * 16 + li;
-      const bool ok = t <= pos;
-      const bf16_t* krow = cache;
-      if (ok) krow = cache + (size_t)bt[t / P] * page_stride + head_off + (size_t)(t % P) * d;
 #pragma unroll
-      for (int ks = 0; ks < DP / 32; ++ks) {
-        const int e = ks * 32 + lc * 8;
-        const Frag kf = (ok && e < d) ? load_frag(krow + e) : zero_frag();
-        s[nt] = mfma16(qf[ks], kf, s[nt]);
-      }
+      for (int ks = 0; ks < DP / 32; ++ks) s[nt] = mfma16(qf[ks], r.k[nt][ks], s[nt]);
     }
     float alpha[4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
+    for (int rr = 0; rr < 4; ++rr) {
       float mx = -INFINITY;
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) {
         const int t = kb + nt * 16 + li;
-        const float v = (t >= first && t <= pos) ? s[nt][r] * scale : -INFINITY;
-        s[nt][r] = v;
+        const float v = (t >= first && t <= pos) ? s[nt][rr] * scale : -INFINITY;
+        s[nt][rr] = v;
         mx = fmaxf(mx, v);
       }
       mx = group16_max(mx);
-      const float m_new = fmaxf(mrow[r], mx);
+      const float m_new = fmaxf(mrow[rr], mx);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      alpha[r] = __expf(mrow[r] - m_safe);
-      const float p0 = __expf(s[0][r] - m_safe), p1 = __expf(s[1][r] - m_safe);
-      s[0][r] = p0;
-      s[1][r] = p1;
-      lrow[r] = lrow[r] * alpha[r] + group16_sum(p0 + p1);
-      mrow[r] = m_new;
+      alpha[rr] = __expf(mrow[rr] - m_safe);
+      const float p0 = __expf(s[0][rr] - m_safe), p1 = __expf(s[1][rr] - m_safe);
+      s[0][rr] = p0;
+      s[1][rr] = p1;
+      lrow[rr] = lrow[rr] * alpha[rr] + group16_sum(p0 + p1);
+      mrow[rr] = m_new;
     }
 #pragma unroll
     for (int dt = 0; dt < DP / 16; ++dt)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) o[dt][r] *= alpha[r];
+      for (int rr = 0; rr < 4; ++rr) o[dt][rr] *= alpha[rr];
+    // P through this wave's LDS rows into the A operand layout
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) pw[(lc * 4 + r) * (32 + KPAD) + nt * 16 + li] = float_to_bf16(s[nt][r]);
+      for (int rr = 0; rr < 4; ++rr) pw[(lc * 4 + rr) * (32 + KPAD) + nt * 16 + li] = float_to_bf16(s[nt][rr]);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     const Frag pf = *reinterpret_cast<const Frag*>(&pw[li * (32 + KPAD) + lc * 8]);
-    // values: 8 consecutive positions of element dt*16 + li
-    const int tv = kb + lc * 8;
-    const bool vok = tv <= pos;
-    const bf16_t* vbase = cache;
-    if (vok) vbase = cache + (size_t)bt[tv / P] * page_stride + v_off + head_off + (tv % P);
 #pragma unroll
-    for (int dt = 0; dt < DP / 16; ++dt) {
-      const int e = dt * 16 + li;
-      const Frag vf = (vok && e < d) ? load_frag(vbase + (size_t)e * P) : zero_frag();
-      o[dt] = mfma16(pf, vf, o[dt]);
-    }
+    for (int dt = 0; dt < DP / 16; ++dt) o[dt] = mfma16(pf, r.v[dt], o[dt]);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
+  };
+
+  const int nsteps = (k_hi - k_lo + 31) / 32;
+  KVRegs<DP> ra, rb;
+  load_kv(ra, k_lo);
+  int done = 0, kb = k_lo;
+  while (done + 2 < nsteps) {
+    load_kv(rb, kb + 32);
+    step(ra, kb);
+    load_kv(ra, kb + 64);
+    step(rb, kb + 32);
+    kb += 64;
+    done += 2;
   }
+  if (done + 1 < nsteps) {
+    load_kv(rb, kb + 32);
+    step(ra, kb);
+    step(rb, kb + 32);
+  } else {
+    step(ra, kb);
+  }
+
   // this part's result for the heads of the group
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -381,6 +418,7 @@ APC_EXPORT int apc_attention_decode_bf16(const void* q, int ldq, int q_off, void
   if (e) return e;
   if (keys_per_part <= 0 || keys_per_part % 32 || n_parts <= 0 || !workspace || max_blocks <= 0 || window < 0)
     return APC_ERR_BAD_ARG;
+  if (keys_per_part / page_tokens + 2 > 64) return APC_ERR_BAD_ARG;  // a wave keeps one page id per lane
   const int G = H / Hk, gtiles = (G + 15) / 16;
   if (Hk * gtiles > 65535 || (n_parts + 3) / 4 > 65535 || H > 65535) return APC_ERR_BAD_ARG;
   dim3 grid(n_rows, Hk * gtiles, (n_parts + 3) / 4), block(256);

@@ -65,11 +65,16 @@ def swiglu_bf16(h: torch.Tensor, wg: PackedWeight, wu: PackedWeight, out: torch.
                   _ops._stream()), "swiglu_bf16")
 
 
-def _keys_per_part(n_rows: int, n_kv_heads: int, max_context: int) -> int:
-    """Keys one wave covers in the decode kernel: as many as leave about 2,000 waves on the chip."""
-    kw = 32
-    while kw < 1024 and n_rows * n_kv_heads * (-(-max_context // (kw * 2))) >= 2048:
+def _keys_per_part(n_rows: int, n_kv_heads: int, max_context: int, page_tokens: int = 16) -> int:
+    """Keys one wave covers in the decode kernel.  A wave that walks through many keys overlaps its loads
+    with its work, so: the longest range that still leaves about a thousand waves on the chip (four per
+    compute unit), at least 64 keys, and no more pages than a wave keeps ids for (one per lane)."""
+    kw = 64
+    while (kw < 1024 and n_rows * n_kv_heads * (-(-max_context // (kw * 2))) >= 1024
+           and (kw * 2) // page_tokens + 2 <= 64):
         kw *= 2
+    while kw > 32 and kw // page_tokens + 2 > 64:
+        kw //= 2
     return kw
 
 
@@ -105,7 +110,7 @@ def attention_bf16(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int,
     if step.n_decode_rows:
         n = step.n_decode_rows
         span = min(step.max_decode_context, window) if window else step.max_decode_context
-        kw = _keys_per_part(n, n_kv_heads, span)
+        kw = _keys_per_part(n, n_kv_heads, span, page_tokens)
         n_parts = -(-step.max_decode_context // kw)
         ws = torch.empty(n * n_heads * n_parts * (head_dim + 2), dtype=torch.float32, device=q.device)
         rows = step.decode_rows.data_ptr() if step.decode_rows is not None else 0
