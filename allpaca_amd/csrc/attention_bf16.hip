@@ -17,33 +17,60 @@
 #include <math.h>
 
 constexpr int KT = 64;            // keys per tile in the prefill kernel
-constexpr int QT = 64;            // rows per tile in the prefill kernel
+constexpr int QT = 64;            // rows per tile in the prefill kernel (4 waves x 16)
 constexpr int KPAD = 8;
 
-__device__ __forceinline__ float group16_max(float v) {  // over the 16 lanes that share lane/16
-#pragma unroll
-  for (int o = 8; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
-  return v;
+// One wave writes LDS and then reads what its other lanes wrote.  The LDS serves a wave's accesses in the order
+// it issues them, so all that is needed is that the compiler keeps that order: a wave barrier (no wait on
+// outstanding global loads, unlike a fence, so loads issued ahead stay in flight).
+__device__ __forceinline__ void wave_lds_order() { __builtin_amdgcn_wave_barrier(); }
+
+// Both kernels compute the transposed products  S^T = K Q^T  and  O^T = V^T P^T : the MFMA result then holds, per
+// lane, 4 consecutive keys (or value elements) of ONE query row (row = lane % 16), so a row's maximum and sum
+// are 16 values in registers and two exchanges between the 4 lanes that share the row, P goes to LDS as 8-byte
+// pieces in the row-major order the second product reads, and the output leaves as 8-byte pieces.
+__device__ __forceinline__ float row4_max(float v) {  // over the 4 lanes that share lane % 16
+  v = fmaxf(v, __shfl_xor(v, 16, WAVE));
+  return fmaxf(v, __shfl_xor(v, 32, WAVE));
 }
-__device__ __forceinline__ float group16_sum(float v) {
-#pragma unroll
-  for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
-  return v;
+__device__ __forceinline__ float row4_sum(float v) {
+  v += __shfl_xor(v, 16, WAVE);
+  return v + __shfl_xor(v, 32, WAVE);
 }
+__device__ __forceinline__ uint32_t bf16_pair(float a, float b) { return pack_bf16x2(a, b); }
+// 2^x for x <= 0 (or -inf): the bare instruction, without the range handling that large arguments need
+__device__ __forceinline__ float exp2_neg(float x) { return __builtin_amdgcn_exp2f(x); }
+constexpr float LOG2E = 1.4426950408889634f;
 
 // ------------------------------------------------------------------------------------------ prefill
+// A block of 4 waves works on up to 64 consecutive rows of one request and one head, 16 rows a wave.
 template <int DP>  // head_dim rounded up to a multiple of 32
 __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, int ldq, int q_off, bf16_t* __restrict__ out, int ldo, int H, int Hk, int d,
     const bf16_t* __restrict__ cache, int P, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ positions, const int* __restrict__ row_seg, const int* __restrict__ tile_row0,
-    const int* __restrict__ tile_rows, int window, float scale) {
+    const int* __restrict__ tile_rows, int n_tiles, int window, float scale) {
   __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * (DP + KPAD)];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[DP * (KT + KPAD)];
   __shared__ __attribute__((aligned(16))) bf16_t Ps[4 * 16 * (KT + KPAD)];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
   const int li = lane % 16, lc = lane / 16;
-  const int tile = blockIdx.x, h = blockIdx.y;
+  // Workgroups go to the 8 XCDs in turn (id % 8) and each XCD has an L2 of its own: all heads that read one kv
+  // head run on one XCD, so its keys and values stay in that L2 for every query tile and head of the group.
+  // Tiles are taken from the last (longest under the causal mask) to the first.
+  int tile, h;
+  {
+    const int id = blockIdx.x, G = H / Hk;
+    if (Hk % 8 == 0) {
+      const int xcd = id % 8, slot = id / 8;
+      const int lh = slot / n_tiles;                 // head among the H/8 heads of this XCD
+      tile = n_tiles - 1 - slot % n_tiles;
+      h = (xcd + 8 * (lh / G)) * G + lh % G;
+    } else {
+      tile = n_tiles - 1 - id % n_tiles;
+      h = id / n_tiles;
+    }
+  }
   const int row0 = tile_row0[tile], nrows = tile_rows[tile];
   const int kvh = h / (H / Hk);
   const int pos0 = positions[row0];
@@ -51,126 +78,189 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   const int last = pos0 + nrows - 1;
   const int first = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
   const size_t page_stride = (size_t)2 * Hk * P * d;
-  const size_t head_off = (size_t)kvh * P * d, v_off = (size_t)Hk * P * d;
   const int dchunks = d / 8;
 
-  // the padding columns of K stay zero for the whole kernel (a padded q column is zero as well, but 0 * NaN is NaN)
+  // K and V are zero where nothing is ever stored: the padding columns of K (a padded q column is zero as well,
+  // but 0 * NaN is NaN) and the rows of V beyond d
   for (int idx = tid; idx < KT * (DP + KPAD); idx += 256) Ks[idx] = 0;
+  for (int idx = tid; idx < DP * (KT + KPAD); idx += 256) Vs[idx] = 0;
 
-  // this wave's 16 query rows as A operands
+  // this wave's 16 query rows as an MFMA operand (row = lane % 16, 8 elements of d per lane and step)
+  const int my_row = wave * 16 + li;
   Frag qf[DP / 32];
   {
-    const int r = wave * 16 + li;
-    const bf16_t* qrow = q + (size_t)(row0 + min(r, nrows - 1)) * ldq + q_off + (size_t)h * d;
+    const bf16_t* qrow = q + (size_t)(row0 + min(my_row, nrows - 1)) * ldq + q_off + (size_t)h * d;
 #pragma unroll
     for (int ks = 0; ks < DP / 32; ++ks) {
       const int e = ks * 32 + lc * 8;
-      qf[ks] = (r < nrows && e < d) ? load_frag(qrow + e) : zero_frag();
+      qf[ks] = (my_row < nrows && e < d) ? load_frag(qrow + e) : zero_frag();
     }
   }
-  floatx4 o[DP / 16];
+  const int my_pos = pos0 + my_row;
+  const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
+  // the wave's rows see every key of a tile [t0, t0 + 64) when it lies inside [wave_lo, wave_hi]
+  const int wave_hi = pos0 + wave * 16;  // smallest position of the wave's rows
+  const int wave_top = wave_hi + 15;
+  const int wave_lo = (window > 0 && wave_top - window + 1 > 0) ? wave_top - window + 1 : 0;
+  const float sc2 = scale * LOG2E;  // exponentials are taken in base 2
+  floatx4 o[DP / 16];               // O^T: element dt*16 + lc*4 + r of row li
 #pragma unroll
   for (int dt = 0; dt < DP / 16; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float mrow[4], lrow[4];
+  float m_run = -INFINITY, l_run = 0.f;
+  bf16_t* pw = Ps + wave * 16 * (KT + KPAD) + li * (KT + KPAD);  // this lane's row of P
+  const bf16_t* krd = Ks + li * (DP + KPAD) + lc * 8;            // this lane's place in a K operand
+  const bf16_t* vrd = Vs + li * (KT + KPAD) + lc * 8;            // ... and in a V operand
+
+  // A tile of 64 keys and values goes global -> registers -> LDS; the loads of the next tile are issued before
+  // the work on the current one and stored after it, and the pages of a tile are looked up one tile before its
+  // loads.  Pieces of 16 bytes: K along d, V along positions (8 of one element); DP/32 of each per thread, whose
+  // places are fixed for the whole loop.  No load is conditional: a key beyond the last one is read from the last
+  // (its scores are masked, its P is 0), a piece that lies in the padding of d is read from piece 0 and not stored.
+  constexpr int PIECES = DP / 32;
+  int k_key[PIECES], v_t[PIECES];
+  bool k_on[PIECES], v_on[PIECES];
+  const bf16_t* k_base[PIECES];
+  const bf16_t* v_base[PIECES];
+  bf16_t* k_dst[PIECES];
+  bf16_t* v_dst[PIECES];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) { mrow[r] = -INFINITY; lrow[r] = 0.f; }
-  bf16_t* pw = Ps + wave * 16 * (KT + KPAD);
-
-  for (int t0 = (first / KT) * KT; t0 <= last; t0 += KT) {
-    __syncthreads();  // the previous tile's K, V and P are no longer read
-    // K tile: 64 keys x d, 16-byte chunks along d
-    for (int idx = tid; idx < KT * dchunks; idx += 256) {
-      const int key = idx / dchunks, ch = idx % dchunks;
-      const int t = t0 + key;
-      Frag f = zero_frag();
-      if (t <= last) {
-        const int page = bt[t / P];
-        f = load_frag(cache + (size_t)page * page_stride + head_off + (size_t)(t % P) * d + ch * 8);
+  for (int j = 0; j < PIECES; ++j) {
+    const int idx = tid + j * 256;
+    k_on[j] = idx < KT * dchunks;
+    const int key = k_on[j] ? idx / dchunks : 0, ch = k_on[j] ? idx % dchunks : 0;
+    k_key[j] = key;
+    k_base[j] = cache + (size_t)kvh * P * d + ch * 8;
+    k_dst[j] = Ks + key * (DP + KPAD) + ch * 8;
+    const int dv = idx / (KT / 8), kc = idx % (KT / 8);
+    v_on[j] = dv < d;
+    v_t[j] = kc * 8;
+    v_base[j] = cache + (size_t)(Hk + kvh) * P * d + (size_t)(v_on[j] ? dv : 0) * P;
+    v_dst[j] = Vs + (v_on[j] ? dv : 0) * (KT + KPAD) + kc * 8;
+  }
+  const int p_shift = (P & (P - 1)) == 0 ? __builtin_ctz(P) : -1;
+  int k_page[PIECES], v_page[PIECES], k_slot[PIECES], v_slot[PIECES];
+  auto lookup_tile = [&](int t0) {
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) {
+      const int t = min(t0 + k_key[j], last), tv = min(t0 + v_t[j], (last / 8) * 8);
+      if (p_shift >= 0) {
+        k_page[j] = bt[t >> p_shift]; k_slot[j] = t & (P - 1);
+        v_page[j] = bt[tv >> p_shift]; v_slot[j] = tv & (P - 1);
+      } else {
+        k_page[j] = bt[t / P]; k_slot[j] = t % P;
+        v_page[j] = bt[tv / P]; v_slot[j] = tv % P;
       }
-      *reinterpret_cast<Frag*>(&Ks[key * (DP + KPAD) + ch * 8]) = f;
     }
-    // V tile, stored [d][key]: chunks of 8 consecutive positions of one element
-    for (int idx = tid; idx < d * (KT / 8); idx += 256) {
-      const int dv = idx / (KT / 8), kc = idx % (KT / 8);
-      const int t = t0 + kc * 8;
-      Frag f = zero_frag();
-      if (t <= last) {
-        const int page = bt[t / P];
-        f = load_frag(cache + (size_t)page * page_stride + v_off + head_off + (size_t)dv * P + (t % P));
-      }
-      *reinterpret_cast<Frag*>(&Vs[dv * (KT + KPAD) + kc * 8]) = f;
+  };
+  Frag kreg[PIECES], vreg[PIECES];
+  auto load_tile = [&]() {  // uses the pages found by the last lookup_tile
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) {
+      kreg[j] = load_frag(k_base[j] + (size_t)k_page[j] * page_stride + (size_t)k_slot[j] * d);
+      vreg[j] = load_frag(v_base[j] + (size_t)v_page[j] * page_stride + v_slot[j]);
     }
-    __syncthreads();
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) {
+      if (k_on[j]) *reinterpret_cast<Frag*>(k_dst[j]) = kreg[j];
+      if (v_on[j]) *reinterpret_cast<Frag*>(v_dst[j]) = vreg[j];
+    }
+  };
 
-    // scores of this wave's 16 rows against the 64 keys
+  const int t_begin = (first / KT) * KT;
+  lookup_tile(t_begin);
+  load_tile();
+  lookup_tile(t_begin + KT);
+  __syncthreads();  // the zero fills are done
+  store_tile();
+  __syncthreads();
+  for (int t0 = t_begin; t0 <= last; t0 += KT) {
+    load_tile();                 // tile t0 + 64 (beyond the last key: a harmless copy of the last)
+    lookup_tile(t0 + 2 * KT);
+
+    // S^T: lane holds keys t0 + nt*16 + lc*4 + r of row li
     floatx4 s[KT / 16];
 #pragma unroll
     for (int nt = 0; nt < KT / 16; ++nt) {
       s[nt] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < DP / 32; ++ks) {
-        const Frag kf = *reinterpret_cast<const Frag*>(&Ks[(nt * 16 + li) * (DP + KPAD) + ks * 32 + lc * 8]);
-        s[nt] = mfma16(qf[ks], kf, s[nt]);
+        const Frag kf = *reinterpret_cast<const Frag*>(krd + nt * 16 * (DP + KPAD) + ks * 32);
+        s[nt] = mfma16(kf, qf[ks], s[nt]);
       }
     }
-    // lane holds rows lc*4 + r and key nt*16 + li
-    float alpha[4];
+    float mx = -INFINITY;
+    if (t0 >= wave_lo && t0 + KT - 1 <= wave_hi) {  // every row of the wave sees the whole tile
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int pos = pos0 + wave * 16 + lc * 4 + r;
-      const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-      float mx = -INFINITY;
+      for (int nt = 0; nt < KT / 16; ++nt)
 #pragma unroll
-      for (int nt = 0; nt < KT / 16; ++nt) {
-        const int t = t0 + nt * 16 + li;
-        const float v = (t >= lo && t <= pos) ? s[nt][r] * scale : -INFINITY;
-        s[nt][r] = v;
-        mx = fmaxf(mx, v);
-      }
-      mx = group16_max(mx);
-      const float m_new = fmaxf(mrow[r], mx);
-      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      alpha[r] = __expf(mrow[r] - m_safe);
-      float sum = 0.f;
+        for (int r = 0; r < 4; ++r) {
+          s[nt][r] *= sc2;
+          mx = fmaxf(mx, s[nt][r]);
+        }
+    } else {
 #pragma unroll
-      for (int nt = 0; nt < KT / 16; ++nt) {
-        const float p = __expf(s[nt][r] - m_safe);
-        s[nt][r] = p;
-        sum += p;
-      }
-      lrow[r] = lrow[r] * alpha[r] + group16_sum(sum);
-      mrow[r] = m_new;
+      for (int nt = 0; nt < KT / 16; ++nt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int t = t0 + nt * 16 + lc * 4 + r;
+          const float v = (t >= my_lo && t <= my_pos) ? s[nt][r] * sc2 : -INFINITY;
+          s[nt][r] = v;
+          mx = fmaxf(mx, v);
+        }
     }
+    mx = row4_max(mx);
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = exp2_neg(m_run - m_safe);
+    float sum = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < KT / 16; ++nt) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        s[nt][r] = exp2_neg(s[nt][r] - m_safe);
+        sum += s[nt][r];
+      }
+      // P, row-major [row][key], 4 consecutive keys at once (read back below by this wave only)
+      uint2 pk;
+      pk.x = bf16_pair(s[nt][0], s[nt][1]);
+      pk.y = bf16_pair(s[nt][2], s[nt][3]);
+      *reinterpret_cast<uint2*>(pw + nt * 16 + lc * 4) = pk;
+    }
+    l_run = l_run * alpha + row4_sum(sum);
+    m_run = m_new;
 #pragma unroll
     for (int dt = 0; dt < DP / 16; ++dt)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) o[dt][r] *= alpha[r];
-    // P through LDS into the A operand layout
-#pragma unroll
-    for (int nt = 0; nt < KT / 16; ++nt)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) pw[(lc * 4 + r) * (KT + KPAD) + nt * 16 + li] = float_to_bf16(s[nt][r]);
-    __syncthreads();
+      for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+    wave_lds_order();
+    // O^T += V^T P^T
 #pragma unroll
     for (int kstep = 0; kstep < KT / 32; ++kstep) {
-      const Frag pf = *reinterpret_cast<const Frag*>(&pw[li * (KT + KPAD) + kstep * 32 + lc * 8]);
+      const Frag pf = *reinterpret_cast<const Frag*>(pw + kstep * 32 + lc * 8);
 #pragma unroll
       for (int dt = 0; dt < DP / 16; ++dt) {
-        const Frag vf = *reinterpret_cast<const Frag*>(&Vs[(dt * 16 + li) * (KT + KPAD) + kstep * 32 + lc * 8]);
-        o[dt] = mfma16(pf, vf, o[dt]);
+        const Frag vf = *reinterpret_cast<const Frag*>(vrd + dt * 16 * (KT + KPAD) + kstep * 32);
+        o[dt] = mfma16(vf, pf, o[dt]);
       }
     }
+    __syncthreads();  // every wave is done with this tile's K and V
+    store_tile();
+    __syncthreads();
   }
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int row = wave * 16 + lc * 4 + r;
-    if (row >= nrows) continue;
-    const float inv = 1.0f / lrow[r];
-    bf16_t* orow = out + (size_t)(row0 + row) * ldo + (size_t)h * d;
+  if (my_row < nrows) {
+    const float inv = 1.0f / l_run;
+    bf16_t* orow = out + (size_t)(row0 + my_row) * ldo + (size_t)h * d;
 #pragma unroll
     for (int dt = 0; dt < DP / 16; ++dt) {
-      const int e = dt * 16 + li;
-      if (e < d) orow[e] = float_to_bf16(o[dt][r] * inv);
+      const int e = dt * 16 + lc * 4;
+      if (e < d) {
+        uint2 pk;
+        pk.x = bf16_pair(o[dt][0] * inv, o[dt][1] * inv);
+        pk.y = bf16_pair(o[dt][2] * inv, o[dt][3] * inv);
+        *reinterpret_cast<uint2*>(orow + e) = pk;
+      }
     }
   }
 }
@@ -222,9 +312,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   floatx4 o[DP / 16];
 #pragma unroll
   for (int dt = 0; dt < DP / 16; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float mrow[4], lrow[4];
-#pragma unroll
-  for (int r = 0; r < 4; ++r) { mrow[r] = -INFINITY; lrow[r] = 0.f; }
+  float m_run = -INFINITY, l_run = 0.f;
   bf16_t* pw = Ps + wave * 16 * (32 + KPAD);
 
   // Operands of 32 keys straight from the pages.  Nothing is loaded conditionally: a key beyond the row's own
@@ -250,52 +338,55 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     for (int dt = 0; dt < DP / 16; ++dt) r.v[dt] = load_frag(vbase + (size_t)min(dt * 16 + li, d - 1) * P);
   };
 
+  // lane holds keys kb + nt*16 + lc*4 + r (scores) and elements dt*16 + lc*4 + r (output) of head li of the group
+  const float sc2 = scale * LOG2E;
   auto step = [&](const KVRegs<DP>& r, int kb) {
     floatx4 s[2];
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
       s[nt] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < DP / 32; ++ks) s[nt] = mfma16(qf[ks], r.k[nt][ks], s[nt]);
+      for (int ks = 0; ks < DP / 32; ++ks) s[nt] = mfma16(r.k[nt][ks], qf[ks], s[nt]);
     }
-    float alpha[4];
-#pragma unroll
-    for (int rr = 0; rr < 4; ++rr) {
-      float mx = -INFINITY;
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
-        const int t = kb + nt * 16 + li;
-        const float v = (t >= first && t <= pos) ? s[nt][rr] * scale : -INFINITY;
-        s[nt][rr] = v;
-        mx = fmaxf(mx, v);
-      }
-      mx = group16_max(mx);
-      const float m_new = fmaxf(mrow[rr], mx);
-      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      alpha[rr] = __expf(mrow[rr] - m_safe);
-      const float p0 = __expf(s[0][rr] - m_safe), p1 = __expf(s[1][rr] - m_safe);
-      s[0][rr] = p0;
-      s[1][rr] = p1;
-      lrow[rr] = lrow[rr] * alpha[rr] + group16_sum(p0 + p1);
-      mrow[rr] = m_new;
-    }
-#pragma unroll
-    for (int dt = 0; dt < DP / 16; ++dt)
-#pragma unroll
-      for (int rr = 0; rr < 4; ++rr) o[dt][rr] *= alpha[rr];
-    // P through this wave's LDS rows into the A operand layout
+    float mx = -INFINITY;
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-      for (int rr = 0; rr < 4; ++rr) pw[(lc * 4 + rr) * (32 + KPAD) + nt * 16 + li] = float_to_bf16(s[nt][rr]);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      for (int rr = 0; rr < 4; ++rr) {
+        const int t = kb + nt * 16 + lc * 4 + rr;
+        const float v = (t >= first && t <= pos) ? s[nt][rr] * sc2 : -INFINITY;
+        s[nt][rr] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = row4_max(mx);
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = exp2_neg(m_run - m_safe);
+    float sum = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const float pv = exp2_neg(s[nt][rr] - m_safe);
+        s[nt][rr] = pv;
+        sum += pv;
+      }
+      uint2 pk;
+      pk.x = bf16_pair(s[nt][0], s[nt][1]);
+      pk.y = bf16_pair(s[nt][2], s[nt][3]);
+      *reinterpret_cast<uint2*>(&pw[li * (32 + KPAD) + nt * 16 + lc * 4]) = pk;
+    }
+    l_run = l_run * alpha + row4_sum(sum);
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DP / 16; ++dt)
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) o[dt][rr] *= alpha;
+    wave_lds_order();
     const Frag pf = *reinterpret_cast<const Frag*>(&pw[li * (32 + KPAD) + lc * 8]);
 #pragma unroll
-    for (int dt = 0; dt < DP / 16; ++dt) o[dt] = mfma16(pf, r.v[dt], o[dt]);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+    for (int dt = 0; dt < DP / 16; ++dt) o[dt] = mfma16(r.v[dt], pf, o[dt]);
+    wave_lds_order();
   };
 
   const int nsteps = (k_hi - k_lo + 31) / 32;
@@ -318,18 +409,19 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     step(ra, kb);
   }
 
-  // this part's result for the heads of the group
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int g = gt * 16 + lc * 4 + r;
-    if (g >= G) continue;
+  // this part's result for the heads of the group (maxima are in base-2 units, as the merge expects)
+  const int g = gt * 16 + li;
+  if (g < G) {
     float* dst = parts + (((size_t)ri * H + (kvh * G + g)) * n_parts + part) * (d + 2);
 #pragma unroll
     for (int dt = 0; dt < DP / 16; ++dt) {
-      const int e = dt * 16 + li;
-      if (e < d) dst[e] = o[dt][r];
+      const int e = dt * 16 + lc * 4;
+      if (e < d) {
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) dst[e + rr] = o[dt][rr];
+      }
     }
-    if (li == 0) { dst[d] = mrow[r]; dst[d + 1] = lrow[r]; }
+    if (lc == 0) { dst[d] = m_run; dst[d + 1] = l_run; }
   }
 }
 
@@ -355,7 +447,7 @@ __global__ __launch_bounds__(MERGE_NT) void attn_merge_kernel(const float* __res
   __syncthreads();
   for (int p = tid; p < np; p += MERGE_NT) {
     const float pm = wgt[p];
-    wgt[p] = pm == -INFINITY ? 0.f : __expf(pm - m);
+    wgt[p] = pm == -INFINITY ? 0.f : exp2_neg(pm - m);
   }
   __syncthreads();
   if (tid == 0) {
@@ -390,12 +482,12 @@ APC_EXPORT int apc_attention_prefill_bf16(const void* q, int ldq, int q_off, voi
   if (n_tiles <= 0) return 0;
   int e = check_common(q, ldq, q_off, cache, H, Hk, d, page_tokens);
   if (e) return e;
-  if (H > 65535 || max_blocks <= 0 || window < 0) return APC_ERR_BAD_ARG;
-  dim3 grid(n_tiles, H), block(256);
+  if (max_blocks <= 0 || window < 0 || (long)n_tiles * H > 0x7fffffffL) return APC_ERR_BAD_ARG;
+  dim3 grid(n_tiles * H), block(256);
 #define PF_LAUNCH(DP_)                                                                                             \
   hipLaunchKernelGGL((attn_prefill_kernel<DP_>), grid, block, 0, stream, (const bf16_t*)q, ldq, q_off, (bf16_t*)out, \
                      ldo, H, Hk, d, (const bf16_t*)cache, page_tokens, block_table, max_blocks, positions, row_seg,  \
-                     tile_row0, tile_rows, window, scale)
+                     tile_row0, tile_rows, n_tiles, window, scale)
   if (d <= 32) PF_LAUNCH(32);
   else if (d <= 64) PF_LAUNCH(64);
   else if (d <= 96) PF_LAUNCH(96);

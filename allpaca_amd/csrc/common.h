@@ -23,13 +23,14 @@ typedef uint16_t bf16_t;  // storage type: the upper half of an IEEE float32
 
 __device__ __forceinline__ float bf16_to_float(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 
-// round to nearest even; NaN stays NaN
-__device__ __forceinline__ bf16_t float_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+// round to nearest even; NaN stays NaN.  gfx950 converts two values with one instruction (v_cvt_pk_bf16_f32).
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  typedef float floatx2_t __attribute__((ext_vector_type(2)));
+  const floatx2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
+__device__ __forceinline__ bf16_t float_to_bf16(float f) { return (bf16_t)(pack_bf16x2(f, 0.f) & 0xffffu); }
 
 __device__ __forceinline__ float load_f(const void* p, int dtype, size_t i) {
   return dtype == APC_F32 ? ((const float*)p)[i] : bf16_to_float(((const bf16_t*)p)[i]);

@@ -55,7 +55,7 @@ class StepInfo:
     n_tiles: int = 0
 
 
-TILE_ROWS = 64
+TILE_ROWS = 64    # rows of an attention tile (must match the prefill kernel's)
 
 
 def pack_step(entries: Sequence[Entry], pos0: Sequence[int], slots: Sequence[int],
