@@ -18,13 +18,19 @@
 constexpr int BM = 128, BN = 128, BK = 64;
 constexpr int LDS_ROW = BK + 8;  // bfloat16 elements per LDS row (144 bytes)
 
-enum { G_STORE_BF16 = 0, G_STORE_F32 = 1, G_ACC_F32 = 2, G_SWIGLU = 3 };
+enum { G_STORE_BF16 = 0, G_STORE_F32 = 1, G_ACC_F32 = 2, G_SWIGLU = 3, G_PARTIAL = 4 };
 
-template <int MODE>
+struct GemmRegs {
+  Frag a[4], w[4];
+};
+
+// EVEN_K: K is a multiple of 64, so no load needs a bound check
+template <int MODE, bool EVEN_K>
 __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda,
                                                         const bf16_t* __restrict__ W,
                                                         const bf16_t* __restrict__ W2, int chunks,
-                                                        void* __restrict__ C, int ldc, int M, int N, int K) {
+                                                        void* __restrict__ C, int ldc, int M, int N, int K,
+                                                        int k_split) {
   __shared__ __attribute__((aligned(16))) bf16_t As[2][BM * LDS_ROW];
   __shared__ __attribute__((aligned(16))) bf16_t Ws[2][BN * LDS_ROW];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
@@ -33,29 +39,31 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
   // N per block: 128 output columns, or 64 (gate and up) in SwiGLU mode
   constexpr int NB = MODE == G_SWIGLU ? BN / 2 : BN;
   const int n0 = blockIdx.x * NB;
+  // G_PARTIAL: blockIdx.z = which * k_split + slice; the block multiplies slice `slice` of K with matrix `which`
+  // (0: W, 1: W2) and leaves its float32 sums in C[which][slice][M][N]
+  const int slice = MODE == G_PARTIAL ? blockIdx.z % k_split : 0;
+  const int which = MODE == G_PARTIAL ? blockIdx.z / k_split : 0;
+  if (MODE == G_PARTIAL && which) W = W2;
 
   // global -> registers: 128 rows x 64 k per operand = 1024 pieces of 16 bytes, 4 per thread and operand.
   // A (row-major): thread -> (row within a group of 32, piece within the 128-byte row).
   // W (tiled): a wave copies one 16 x 32 tile per pass: thread -> (row in band, 8-column piece, which of the
   // two tiles along K, which of two bands); 4 passes cover the 8 bands of the block tile.
+  // Addresses are a base that is the same for the whole block (it moves along K) plus a small offset per thread.
   const int lrow = tid / 8, lchunk = tid % 8;
   const int wi = tid % 16, wc = (tid / 16) % 4, wkc = (tid / 64) % 2, wbl = tid / 128;
   const int bands = (N + 15) / 16;
-  const bf16_t* aptr[4];
-  const bf16_t* wptr[4];
+  const int band0 = n0 / 16;
+  const bf16_t* abase = A + (size_t)m0 * lda;
+  const bf16_t* wbase0 = W + (size_t)band0 * chunks * 512;
+  const bf16_t* wbase1 = (MODE == G_SWIGLU ? W2 : W) + (size_t)band0 * chunks * 512;  // passes 2, 3
+  unsigned aoff[4], woff[4];
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
-    aptr[p] = A + (size_t)min(m0 + p * 32 + lrow, M - 1) * lda + lchunk * 8;
-    const int bl = p * 2 + wbl;  // band of the block tile, 0..7
-    int band;
-    const bf16_t* base = W;
-    if (MODE == G_SWIGLU) {
-      band = n0 / 16 + (bl % 4);
-      base = bl < 4 ? W : W2;
-    } else {
-      band = n0 / 16 + bl;
-    }
-    wptr[p] = base + ((size_t)min(band, bands - 1) * chunks + wkc) * 512 + (wc * 16 + wi) * 8;
+    aoff[p] = (unsigned)(min(m0 + p * 32 + lrow, M - 1) - m0) * lda + lchunk * 8;
+    const int bl = p * 2 + wbl;                               // band of the block tile, 0..7
+    const int rel = MODE == G_SWIGLU ? bl % 4 : bl;           // SwiGLU: 4 gate bands, then the same 4 up bands
+    woff[p] = (unsigned)(min(band0 + rel, bands - 1) - band0) * chunks * 512 + wkc * 512 + (wc * 16 + wi) * 8;
   }
 
   floatx16 acc[2][2];
@@ -66,32 +74,36 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
-  Frag ra[4], rw[4];
-  auto load_global = [&](int k0) {
-    const bool in = k0 + lchunk * 8 < K;  // K is a multiple of 8: a piece is inside or outside as a whole
-    const bool win = k0 / 32 + wkc < chunks;  // W is zero-padded up to whole tiles
+  auto load_global = [&](GemmRegs& g, int kt) {  // K step kt (64 columns) of the block's rows
+    const int k0 = kt * BK;
+    const bf16_t* ak = abase + k0;
+    const bf16_t* wk0 = wbase0 + (size_t)kt * 1024;
+    const bf16_t* wk1 = wbase1 + (size_t)kt * 1024;
+    if (EVEN_K) {
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-      ra[p] = in ? load_frag(aptr[p] + k0) : zero_frag();
-      rw[p] = win ? load_frag(wptr[p] + (size_t)(k0 / 32) * 512) : zero_frag();
+      for (int p = 0; p < 4; ++p) {
+        g.a[p] = load_frag(ak + aoff[p]);
+        g.w[p] = load_frag((p < 2 ? wk0 : wk1) + woff[p]);
+      }
+    } else {
+      const bool in = k0 + lchunk * 8 < K;      // K is a multiple of 8: a piece is inside or outside as a whole
+      const bool win = kt * 2 + wkc < chunks;   // W is zero-padded up to whole tiles
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        g.a[p] = in ? load_frag(ak + aoff[p]) : zero_frag();
+        g.w[p] = win ? load_frag((p < 2 ? wk0 : wk1) + woff[p]) : zero_frag();
+      }
     }
   };
-  auto store_lds = [&](int buf) {
+  auto store_lds = [&](const GemmRegs& g, int buf) {
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
-      *reinterpret_cast<Frag*>(&As[buf][(p * 32 + lrow) * LDS_ROW + lchunk * 8]) = ra[p];
-      *reinterpret_cast<Frag*>(&Ws[buf][((p * 2 + wbl) * 16 + wi) * LDS_ROW + wkc * 32 + wc * 8]) = rw[p];
+      *reinterpret_cast<Frag*>(&As[buf][(p * 32 + lrow) * LDS_ROW + lchunk * 8]) = g.a[p];
+      *reinterpret_cast<Frag*>(&Ws[buf][((p * 2 + wbl) * 16 + wi) * LDS_ROW + wkc * 32 + wc * 8]) = g.w[p];
     }
   };
-
-  const int ktiles = ceil_div(K, BK);
-  load_global(0);
-  store_lds(0);
-  __syncthreads();
   const int li = lane % 32, lc = lane / 32;
-  for (int kt = 0; kt < ktiles; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < ktiles) load_global((kt + 1) * BK);
+  auto compute = [&](int buf) {
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
       Frag fa[2], fw[2];
@@ -107,8 +119,48 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
 #pragma unroll
         for (int b = 0; b < 2; ++b) acc[a][b] = mfma32(fa[a], fw[b], acc[a][b]);
     }
-    if (kt + 1 < ktiles) store_lds(buf ^ 1);
+  };
+
+  const int all_tiles = ceil_div(K, BK);
+  const int per_slice = MODE == G_PARTIAL ? ceil_div(all_tiles, k_split) : all_tiles;
+  const int kt0 = slice * per_slice;
+  const int ktiles = max(0, min(all_tiles, kt0 + per_slice) - kt0);
+  // K steps are loaded two ahead: while step t is multiplied out of LDS, step t+1 waits in registers for its
+  // turn in the other LDS buffer and the loads of step t+2 are in flight (register sets s0, s1 take turns).
+  // The steady loop has no branch around a load, so the waits for one set never wait for the other.
+  if (ktiles > 0) {
+    GemmRegs s0, s1;
+    load_global(s0, kt0);
+    store_lds(s0, 0);
+    if (ktiles > 1) load_global(s1, kt0 + 1);
     __syncthreads();
+    int kt = 0;
+    while (kt + 3 < ktiles) {
+      load_global(s0, kt0 + kt + 2);
+      __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, not where the compiler would sink them to
+      compute(0);
+      store_lds(s1, 1);
+      __syncthreads();
+      load_global(s1, kt0 + kt + 3);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(1);
+      store_lds(s0, 0);
+      __syncthreads();
+      kt += 2;
+    }
+    const int rem = ktiles - kt;  // 1..3 steps left: step kt in LDS buffer 0, step kt+1 (if any) in s1
+    if (rem == 3) load_global(s0, kt0 + kt + 2);
+    compute(0);
+    if (rem >= 2) {
+      store_lds(s1, 1);
+      __syncthreads();
+      compute(1);
+      if (rem == 3) {
+        store_lds(s0, 0);
+        __syncthreads();
+        compute(0);
+      }
+    }
   }
 
   // D[i][j]: i = row of A (m), j = row of W (n); lane holds column j = lane%32 and rows (r/4)*8 + (lane/32)*4 + r%4
@@ -129,7 +181,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
           const size_t o = (size_t)m * ldc + n;
           if (MODE == G_STORE_BF16) ((bf16_t*)C)[o] = float_to_bf16(acc[a][b][r]);
           else if (MODE == G_STORE_F32) ((float*)C)[o] = acc[a][b][r];
-          else ((float*)C)[o] += acc[a][b][r];
+          else if (MODE == G_ACC_F32) ((float*)C)[o] += acc[a][b][r];
+          else ((float*)C)[((size_t)blockIdx.z * M + m) * N + n] = acc[a][b][r];
         }
       }
     }
@@ -144,8 +197,58 @@ static int launch_gemm(const bf16_t* A, int lda, const bf16_t* W, const bf16_t* 
   constexpr int NB = MODE == G_SWIGLU ? BN / 2 : BN;
   const int gy = ceil_div(M, BM);
   if (gy > 65535) return APC_ERR_BAD_ARG;
-  hipLaunchKernelGGL((gemm_bf16_kernel<MODE>), dim3(ceil_div(N, NB), gy), dim3(256), 0, stream, A, lda, W, W2,
-                     ceil_div(K, 32), C, ldc, M, N, K);
+  if (K % BK == 0)
+    hipLaunchKernelGGL((gemm_bf16_kernel<MODE, true>), dim3(ceil_div(N, NB), gy), dim3(256), 0, stream, A, lda, W, W2,
+                       ceil_div(K, 32), C, ldc, M, N, K, 1);
+  else
+    hipLaunchKernelGGL((gemm_bf16_kernel<MODE, false>), dim3(ceil_div(N, NB), gy), dim3(256), 0, stream, A, lda, W, W2,
+                       ceil_div(K, 32), C, ldc, M, N, K, 1);
+  APC_LAUNCH_CHECK();
+  return 0;
+}
+
+// Sums the float32 sums that G_PARTIAL blocks left ([which][slice][M][N], slices in order) and finishes:
+// store bfloat16 / float32, add into a float32 residual, or SwiGLU of the two matrices' sums.
+__global__ __launch_bounds__(256) void gemm_finish_kernel(const float* __restrict__ partials, int k_split, int M, int N,
+                                                          int mode, void* __restrict__ C, int ldc) {
+  const int n = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
+  if (n >= N) return;
+  const size_t plane = (size_t)M * N;
+  const float* src = partials + (size_t)m * N + n;
+  float g = 0.f;
+  for (int s = 0; s < k_split; ++s) g += src[s * plane];
+  const size_t o = (size_t)m * ldc + n;
+  if (mode == G_STORE_BF16) ((bf16_t*)C)[o] = float_to_bf16(g);
+  else if (mode == G_STORE_F32) ((float*)C)[o] = g;
+  else if (mode == G_ACC_F32) ((float*)C)[o] += g;
+  else {
+    float u = 0.f;
+    for (int s = 0; s < k_split; ++s) u += src[(k_split + s) * plane];
+    ((bf16_t*)C)[o] = float_to_bf16(silu_f(g) * u);
+  }
+}
+
+// Product for 17..128 rows: K is cut into `k_split` slices that different blocks multiply, so that matrices with
+// few output columns still give the chip enough blocks; `workspace` holds (Wu ? 2 : 1) * k_split * M * N floats.
+// mode as below, or 3 for SwiGLU (W = gate, Wu = up).
+APC_EXPORT int apc_gemm_splitk_bf16(const void* A, int lda, const void* W, const void* Wu, void* C, int ldc, int M,
+                                    int N, int K, int mode, int k_split, float* workspace, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || lda < K || ldc < N || k_split < 1 || !workspace || M > 65535) return APC_ERR_BAD_ARG;
+  if (mode < 0 || mode > G_SWIGLU || (mode == G_SWIGLU) != (Wu != nullptr)) return APC_ERR_BAD_ARG;
+  if (K % 8 || lda % 8 || !aligned16(A) || !aligned16(W) || (Wu && !aligned16(Wu))) return APC_ERR_UNSUPPORTED;
+  const int n_mats = Wu ? 2 : 1;
+  if (k_split * n_mats > 65535) return APC_ERR_BAD_ARG;
+  const dim3 grid(ceil_div(N, BN), ceil_div(M, BM), k_split * n_mats);
+  if (K % BK == 0)
+    hipLaunchKernelGGL((gemm_bf16_kernel<G_PARTIAL, true>), grid, dim3(256), 0, stream, (const bf16_t*)A, lda,
+                       (const bf16_t*)W, (const bf16_t*)Wu, ceil_div(K, 32), workspace, N, M, N, K, k_split);
+  else
+    hipLaunchKernelGGL((gemm_bf16_kernel<G_PARTIAL, false>), grid, dim3(256), 0, stream, (const bf16_t*)A, lda,
+                       (const bf16_t*)W, (const bf16_t*)Wu, ceil_div(K, 32), workspace, N, M, N, K, k_split);
+  APC_LAUNCH_CHECK();
+  hipLaunchKernelGGL(gemm_finish_kernel, dim3(ceil_div(N, 256), M), dim3(256), 0, stream, workspace, k_split, M, N, mode,
+                     C, ldc);
   APC_LAUNCH_CHECK();
   return 0;
 }

@@ -40,6 +40,7 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
     "tuned": {
         "apc_gemm_bf16": [P, I, P, P, I, I, I, I, I, P],
         "apc_gemm_swiglu_bf16": [P, I, P, P, P, I, I, I, I, P],
+        "apc_gemm_splitk_bf16": [P, I, P, P, P, I, I, I, I, I, I, P, P],
         "apc_skinny_gemm_bf16": [P, I, P, P, I, I, I, I, I, P],
         "apc_skinny_swiglu_bf16": [P, I, P, P, P, I, I, I, I, P],
         "apc_attention_prefill_bf16": [P, I, I, P, I, I, I, I, P, I, P, I, P, P, P, P, I, I, F, P],

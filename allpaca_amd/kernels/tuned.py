@@ -15,7 +15,15 @@ from . import lib as _lib
 from . import ops as _ops
 from .packing import PackedWeight
 
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 16     # the streaming kernel: up to one 16-row tile of activations
+SPLITK_MAX_ROWS = 128    # the tiled kernel with K cut into slices: 17..128 rows
+
+
+def _k_split(M: int, N: int, K: int) -> int:
+    """Slices of K for the split kernel: enough blocks for the chip (about 512), at least 4 K-steps of 64 each."""
+    blocks = -(-N // 128) * -(-M // 128)
+    s = max(1, min(8, -(-512 // blocks)))
+    return max(1, min(s, K // 256))
 
 
 def _aligned(*ts: torch.Tensor) -> bool:
@@ -43,6 +51,13 @@ def gemm_bf16(a: torch.Tensor, w: PackedWeight, out: torch.Tensor, accumulate: b
     lda, ldc = _ops._rows(a, "a"), _ops._rows(out, "out")
     mode = 2 if accumulate else (0 if out.dtype == torch.bfloat16 else 1)
     L = _lib.load("tuned")
+    if SKINNY_MAX_ROWS < M <= SPLITK_MAX_ROWS:
+        ks = _k_split(M, N, K)
+        if ks > 1:
+            ws = torch.empty(ks * M * N, dtype=torch.float32, device=a.device)
+            _lib.check(L.apc_gemm_splitk_bf16(a.data_ptr(), lda, w.data.data_ptr(), 0, out.data_ptr(), ldc, M, N, K,
+                                              mode, ks, ws.data_ptr(), _ops._stream()), "gemm_splitk_bf16")
+            return
     fn = L.apc_skinny_gemm_bf16 if M <= SKINNY_MAX_ROWS else L.apc_gemm_bf16
     _lib.check(fn(a.data_ptr(), lda, w.data.data_ptr(), out.data_ptr(), ldc, M, N, K, mode, _ops._stream()),
                "gemm_bf16")
@@ -60,6 +75,12 @@ def swiglu_bf16(h: torch.Tensor, wg: PackedWeight, wu: PackedWeight, out: torch.
                          "of 8, 16-byte aligned")
     lda, ldc = _ops._rows(h, "h"), _ops._rows(out, "out")
     L = _lib.load("tuned")
+    if SKINNY_MAX_ROWS < M <= SPLITK_MAX_ROWS:
+        ks = _k_split(M, 2 * F, K)
+        ws = torch.empty(2 * ks * M * F, dtype=torch.float32, device=h.device)
+        _lib.check(L.apc_gemm_splitk_bf16(h.data_ptr(), lda, wg.data.data_ptr(), wu.data.data_ptr(), out.data_ptr(), ldc,
+                                          M, F, K, 3, ks, ws.data_ptr(), _ops._stream()), "gemm_splitk_bf16")
+        return
     fn = L.apc_skinny_swiglu_bf16 if M <= SKINNY_MAX_ROWS else L.apc_gemm_swiglu_bf16
     _lib.check(fn(h.data_ptr(), lda, wg.data.data_ptr(), wu.data.data_ptr(), out.data_ptr(), ldc, M, F, K,
                   _ops._stream()), "swiglu_bf16")
