@@ -5,47 +5,75 @@
 // contiguous 1 KiB load into a row-major LDS tile.
 // A block of 256 threads (4 waves, 2 x 2) computes a 128 x 128 tile of C; K runs in steps of 64
 // through a double-buffered LDS tile of A and of W (rows padded by 16 bytes so that the 16-byte
-// operand reads of 8 consecutive rows fall into different banks).  Each wave owns 64 x 64 of the tile
-// as 2 x 2 v_mfma_f32_32x32x16_bf16 accumulators.  Global loads of the next K step are issued before
-// the MFMAs of the current one and stored to the other LDS buffer after them.
+// operand reads of 8 consecutive rows fall into different banks).  Each wave owns a quarter of the tile
+// as 2 x 2 v_mfma_f32_32x32x16_bf16 accumulators.  Global loads run two K steps ahead of the MFMAs, and
+// loads and LDS stores are spread between the MFMAs of a step: LDS bandwidth (reads of operands plus stores of
+// the next step) and the load path are each about as busy as the matrix cores, so none of them may wait for another.
 // Epilogues: store bfloat16 / float32, add into a float32 residual, or SwiGLU: then the W tile is
 // 64 gate rows and the matching 64 up rows, each wave computes gate and up of the same 64 x 32 outputs,
 // and the block writes a 128 x 64 tile of silu(gate) * up.
-// The K order of every output is fixed (k = 0, 16, 32, ... inside one accumulator), whatever M.
+// With 17..128 rows and a long K, K is cut into slices for different blocks and a second kernel adds the slices in
+// order.  The order of additions for an output depends on N, K and on whether the step has up to 128 rows or more,
+// never on which other rows are in the batch.
 // Reference counterpart: gemm_nt_bf16_tiled_kernel, hip/src/kernels.cpp:634 (no matrix cores there).
+#include <type_traits>
+
 #include "mfma.h"
 
-constexpr int BM = 128, BN = 128, BK = 64;
+constexpr int BN = 128, BK = 64;
+// Rows of the block tile.  The kernel also builds with 256 (4 x 2 accumulators a wave, one block a compute unit);
+// on the shapes of an 8B model with 2,048 rows that was no faster than two 128-row blocks sharing a unit.
+constexpr int BM_ROWS = 128;
 constexpr int LDS_ROW = BK + 8;  // bfloat16 elements per LDS row (144 bytes)
 
 enum { G_STORE_BF16 = 0, G_STORE_F32 = 1, G_ACC_F32 = 2, G_SWIGLU = 3, G_PARTIAL = 4 };
 
+template <int BM>
 struct GemmRegs {
-  Frag a[4], w[4];
+  Frag a[BM / 32], w[4];
 };
 
-// EVEN_K: K is a multiple of 64, so no load needs a bound check
-template <int MODE, bool EVEN_K>
+// EVEN_K: K is a multiple of 64, so no load needs a bound check.  BM: rows of the block tile, 128 or 256.
+template <int MODE, bool EVEN_K, int BM>
 __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda,
                                                         const bf16_t* __restrict__ W,
                                                         const bf16_t* __restrict__ W2, int chunks,
                                                         void* __restrict__ C, int ldc, int M, int N, int K,
                                                         int k_split) {
+  constexpr int AP = BM / 32;          // 16-byte pieces of A per thread and K step
+  constexpr int WM = BM / 64;          // 32-row accumulators of a wave along M
+  constexpr int PIECES = AP + 4;       // pieces of A and W per thread and K step
+  constexpr int PER_GROUP = PIECES / 4;
   __shared__ __attribute__((aligned(16))) bf16_t As[2][BM * LDS_ROW];
   __shared__ __attribute__((aligned(16))) bf16_t Ws[2][BN * LDS_ROW];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
   const int wm = wave / 2, wn = wave % 2;
-  const int m0 = blockIdx.y * BM;
   // N per block: 128 output columns, or 64 (gate and up) in SwiGLU mode
   constexpr int NB = MODE == G_SWIGLU ? BN / 2 : BN;
-  const int n0 = blockIdx.x * NB;
+  int mt, nt;
+  if (MODE == G_PARTIAL) {
+    mt = blockIdx.y;
+    nt = blockIdx.x;
+  } else {
+    // Order of the blocks: consecutive block ids go to the 8 XCDs in turn, each with an L2 of its own.  XCD x takes
+    // the column tiles x, x+8, ..; inside it, groups of up to 8 row tiles sweep those columns, row tile fastest, so
+    // the blocks that run on an XCD at one time share a few tiles of W and of A.
+    const int MT = ceil_div(M, BM), NT = ceil_div(N, NB), NL = ceil_div(NT, 8);
+    constexpr int GM = 8;
+    const int xcd = blockIdx.x % 8, j = blockIdx.x / 8;
+    const int first_m = j / (GM * NL) * GM, gsz = min(MT - first_m, GM), jj = j % (GM * NL);
+    mt = first_m + jj % gsz;
+    nt = jj / gsz * 8 + xcd;
+    if (nt >= NT || mt >= MT) return;
+  }
+  const int m0 = mt * BM, n0 = nt * NB;
   // G_PARTIAL: blockIdx.z = which * k_split + slice; the block multiplies slice `slice` of K with matrix `which`
   // (0: W, 1: W2) and leaves its float32 sums in C[which][slice][M][N]
   const int slice = MODE == G_PARTIAL ? blockIdx.z % k_split : 0;
   const int which = MODE == G_PARTIAL ? blockIdx.z / k_split : 0;
   if (MODE == G_PARTIAL && which) W = W2;
 
-  // global -> registers: 128 rows x 64 k per operand = 1024 pieces of 16 bytes, 4 per thread and operand.
+  // global -> registers: BM rows of A and 128 rows of W x 64 k = pieces of 16 bytes, BM/32 + 4 per thread.
   // A (row-major): thread -> (row within a group of 32, piece within the 128-byte row).
   // W (tiled): a wave copies one 16 x 32 tile per pass: thread -> (row in band, 8-column piece, which of the
   // two tiles along K, which of two bands); 4 passes cover the 8 bands of the block tile.
@@ -57,118 +85,127 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
   const bf16_t* abase = A + (size_t)m0 * lda;
   const bf16_t* wbase0 = W + (size_t)band0 * chunks * 512;
   const bf16_t* wbase1 = (MODE == G_SWIGLU ? W2 : W) + (size_t)band0 * chunks * 512;  // passes 2, 3
-  unsigned aoff[4], woff[4];
+  unsigned aoff[AP], woff[4];
+#pragma unroll
+  for (int p = 0; p < AP; ++p) aoff[p] = (unsigned)(min(m0 + p * 32 + lrow, M - 1) - m0) * lda + lchunk * 8;
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
-    aoff[p] = (unsigned)(min(m0 + p * 32 + lrow, M - 1) - m0) * lda + lchunk * 8;
     const int bl = p * 2 + wbl;                               // band of the block tile, 0..7
     const int rel = MODE == G_SWIGLU ? bl % 4 : bl;           // SwiGLU: 4 gate bands, then the same 4 up bands
     woff[p] = (unsigned)(min(band0 + rel, bands - 1) - band0) * chunks * 512 + wkc * 512 + (wc * 16 + wi) * 8;
   }
 
-  floatx16 acc[2][2];
+  floatx16 acc[WM][2];
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+  for (int a = 0; a < WM; ++a)
 #pragma unroll
     for (int b = 0; b < 2; ++b)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
-  auto load_global = [&](GemmRegs& g, int kt) {  // K step kt (64 columns) of the block's rows
-    const int k0 = kt * BK;
-    const bf16_t* ak = abase + k0;
-    const bf16_t* wk0 = wbase0 + (size_t)kt * 1024;
-    const bf16_t* wk1 = wbase1 + (size_t)kt * 1024;
-    if (EVEN_K) {
-#pragma unroll
-      for (int p = 0; p < 4; ++p) {
-        g.a[p] = load_frag(ak + aoff[p]);
-        g.w[p] = load_frag((p < 2 ? wk0 : wk1) + woff[p]);
-      }
+  // piece j of K step kt (64 columns): j < AP a piece of A, else of W
+  auto load_piece = [&](GemmRegs<BM>& g, int kt, int j) {
+    if (j < AP) {
+      const bf16_t* src = abase + kt * BK + aoff[j];
+      // K is a multiple of 8: a piece is inside or outside as a whole
+      g.a[j] = (EVEN_K || kt * BK + lchunk * 8 < K) ? load_frag(src) : zero_frag();
     } else {
-      const bool in = k0 + lchunk * 8 < K;      // K is a multiple of 8: a piece is inside or outside as a whole
-      const bool win = kt * 2 + wkc < chunks;   // W is zero-padded up to whole tiles
-#pragma unroll
-      for (int p = 0; p < 4; ++p) {
-        g.a[p] = in ? load_frag(ak + aoff[p]) : zero_frag();
-        g.w[p] = win ? load_frag((p < 2 ? wk0 : wk1) + woff[p]) : zero_frag();
-      }
+      const int p = j - AP;
+      const bf16_t* src = (p < 2 ? wbase0 : wbase1) + (size_t)kt * 1024 + woff[p];
+      g.w[p] = (EVEN_K || kt * 2 + wkc < chunks) ? load_frag(src) : zero_frag();  // W is zero-padded to whole tiles
     }
   };
-  auto store_lds = [&](const GemmRegs& g, int buf) {
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-      *reinterpret_cast<Frag*>(&As[buf][(p * 32 + lrow) * LDS_ROW + lchunk * 8]) = g.a[p];
+  auto store_piece = [&](const GemmRegs<BM>& g, int buf, int j) {
+    if (j < AP) {
+      *reinterpret_cast<Frag*>(&As[buf][(j * 32 + lrow) * LDS_ROW + lchunk * 8]) = g.a[j];
+    } else {
+      const int p = j - AP;
       *reinterpret_cast<Frag*>(&Ws[buf][((p * 2 + wbl) * 16 + wi) * LDS_ROW + wkc * 32 + wc * 8]) = g.w[p];
     }
   };
   const int li = lane % 32, lc = lane / 32;
-  auto compute = [&](int buf) {
+  // One K step out of LDS buffer `buf` in four groups of MFMAs.  Between the groups the loads of step `kt_load` go
+  // out into `ld` (if LD) and the pieces of `st`, loaded a step earlier, go into the other LDS buffer (if ST): the
+  // memory pipeline and LDS work while the matrix cores do, instead of in a burst around the barrier.
+  auto step = [&](auto LD, auto ST, int buf, GemmRegs<BM>& ld, int kt_load, const GemmRegs<BM>& st) {
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
-      Frag fa[2], fw[2];
+      if constexpr (decltype(LD)::value) {
+#pragma unroll
+        for (int j = kk * PER_GROUP; j < (kk + 1) * PER_GROUP; ++j) load_piece(ld, kt_load, j);
+      }
+      Frag fa[WM], fw[2];
+#pragma unroll
+      for (int t = 0; t < WM; ++t)
+        fa[t] = *reinterpret_cast<const Frag*>(&As[buf][(wm * (BM / 2) + t * 32 + li) * LDS_ROW + kk * 16 + lc * 8]);
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        fa[t] = *reinterpret_cast<const Frag*>(&As[buf][(wm * 64 + t * 32 + li) * LDS_ROW + kk * 16 + lc * 8]);
         // SwiGLU: tile 0 = gate rows wn*32.., tile 1 = the up rows of the same outputs
         const int wrow = MODE == G_SWIGLU ? t * 64 + wn * 32 + li : wn * 64 + t * 32 + li;
         fw[t] = *reinterpret_cast<const Frag*>(&Ws[buf][wrow * LDS_ROW + kk * 16 + lc * 8]);
       }
 #pragma unroll
-      for (int a = 0; a < 2; ++a)
+      for (int a = 0; a < WM; ++a)
 #pragma unroll
         for (int b = 0; b < 2; ++b) acc[a][b] = mfma32(fa[a], fw[b], acc[a][b]);
+      if constexpr (decltype(ST)::value) {
+#pragma unroll
+        for (int j = kk * PER_GROUP; j < (kk + 1) * PER_GROUP; ++j) store_piece(st, buf ^ 1, j);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // keeps each group's memory work in its group
     }
   };
+  constexpr std::true_type yes{};
+  constexpr std::false_type no{};
 
   const int all_tiles = ceil_div(K, BK);
   const int per_slice = MODE == G_PARTIAL ? ceil_div(all_tiles, k_split) : all_tiles;
   const int kt0 = slice * per_slice;
   const int ktiles = max(0, min(all_tiles, kt0 + per_slice) - kt0);
-  // K steps are loaded two ahead: while step t is multiplied out of LDS, step t+1 waits in registers for its
-  // turn in the other LDS buffer and the loads of step t+2 are in flight (register sets s0, s1 take turns).
-  // The steady loop has no branch around a load, so the waits for one set never wait for the other.
+  // K steps are loaded two ahead: while step t is multiplied out of one LDS buffer, step t+1 moves from registers
+  // into the other and the loads of step t+2 go out (register sets s0, s1 take turns).  The steady loop has no
+  // branch around a load, so the waits for one set never wait for the other.
   if (ktiles > 0) {
-    GemmRegs s0, s1;
-    load_global(s0, kt0);
-    store_lds(s0, 0);
-    if (ktiles > 1) load_global(s1, kt0 + 1);
+    GemmRegs<BM> s0, s1;
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) load_piece(s0, kt0, j);
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) store_piece(s0, 0, j);
+    if (ktiles > 1) {
+#pragma unroll
+      for (int j = 0; j < PIECES; ++j) load_piece(s1, kt0 + 1, j);
+    }
     __syncthreads();
     int kt = 0;
     while (kt + 3 < ktiles) {
-      load_global(s0, kt0 + kt + 2);
-      __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, not where the compiler would sink them to
-      compute(0);
-      store_lds(s1, 1);
+      step(yes, yes, 0, s0, kt0 + kt + 2, s1);
       __syncthreads();
-      load_global(s1, kt0 + kt + 3);
-      __builtin_amdgcn_sched_barrier(0);
-      compute(1);
-      store_lds(s0, 0);
+      step(yes, yes, 1, s1, kt0 + kt + 3, s0);
       __syncthreads();
       kt += 2;
     }
     const int rem = ktiles - kt;  // 1..3 steps left: step kt in LDS buffer 0, step kt+1 (if any) in s1
-    if (rem == 3) load_global(s0, kt0 + kt + 2);
-    compute(0);
-    if (rem >= 2) {
-      store_lds(s1, 1);
+    if (rem == 3) {
+      step(yes, yes, 0, s0, kt0 + kt + 2, s1);
       __syncthreads();
-      compute(1);
-      if (rem == 3) {
-        store_lds(s0, 0);
-        __syncthreads();
-        compute(0);
-      }
+      step(no, yes, 1, s1, 0, s0);
+      __syncthreads();
+      step(no, no, 0, s0, 0, s1);
+    } else if (rem == 2) {
+      step(no, yes, 0, s0, 0, s1);
+      __syncthreads();
+      step(no, no, 1, s0, 0, s1);
+    } else {
+      step(no, no, 0, s0, 0, s1);
     }
   }
 
   // D[i][j]: i = row of A (m), j = row of W (n); lane holds column j = lane%32 and rows (r/4)*8 + (lane/32)*4 + r%4
 #pragma unroll
-  for (int a = 0; a < 2; ++a) {
+  for (int a = 0; a < WM; ++a) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int m = m0 + wm * 64 + a * 32 + (r / 4) * 8 + lc * 4 + (r % 4);
+      const int m = m0 + wm * (BM / 2) + a * 32 + (r / 4) * 8 + lc * 4 + (r % 4);
       if (m >= M) continue;
       if (MODE == G_SWIGLU) {
         const int n = n0 + wn * 32 + li;
@@ -195,14 +232,14 @@ template <int MODE>
 static int launch_gemm(const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M, int N,
                        int K, hipStream_t stream) {
   constexpr int NB = MODE == G_SWIGLU ? BN / 2 : BN;
-  const int gy = ceil_div(M, BM);
-  if (gy > 65535) return APC_ERR_BAD_ARG;
+  const long blocks = 8L * ceil_div(ceil_div(N, NB), 8) * ceil_div(M, BM_ROWS);
+  if (blocks > 0x7fffffffL) return APC_ERR_BAD_ARG;
   if (K % BK == 0)
-    hipLaunchKernelGGL((gemm_bf16_kernel<MODE, true>), dim3(ceil_div(N, NB), gy), dim3(256), 0, stream, A, lda, W, W2,
-                       ceil_div(K, 32), C, ldc, M, N, K, 1);
+    hipLaunchKernelGGL((gemm_bf16_kernel<MODE, true, BM_ROWS>), dim3((unsigned)blocks), dim3(256), 0, stream, A, lda, W,
+                       W2, ceil_div(K, 32), C, ldc, M, N, K, 1);
   else
-    hipLaunchKernelGGL((gemm_bf16_kernel<MODE, false>), dim3(ceil_div(N, NB), gy), dim3(256), 0, stream, A, lda, W, W2,
-                       ceil_div(K, 32), C, ldc, M, N, K, 1);
+    hipLaunchKernelGGL((gemm_bf16_kernel<MODE, false, BM_ROWS>), dim3((unsigned)blocks), dim3(256), 0, stream, A, lda, W,
+                       W2, ceil_div(K, 32), C, ldc, M, N, K, 1);
   APC_LAUNCH_CHECK();
   return 0;
 }
@@ -239,12 +276,12 @@ APC_EXPORT int apc_gemm_splitk_bf16(const void* A, int lda, const void* W, const
   if (K % 8 || lda % 8 || !aligned16(A) || !aligned16(W) || (Wu && !aligned16(Wu))) return APC_ERR_UNSUPPORTED;
   const int n_mats = Wu ? 2 : 1;
   if (k_split * n_mats > 65535) return APC_ERR_BAD_ARG;
-  const dim3 grid(ceil_div(N, BN), ceil_div(M, BM), k_split * n_mats);
+  const dim3 grid(ceil_div(N, BN), ceil_div(M, BM_ROWS), k_split * n_mats);
   if (K % BK == 0)
-    hipLaunchKernelGGL((gemm_bf16_kernel<G_PARTIAL, true>), grid, dim3(256), 0, stream, (const bf16_t*)A, lda,
+    hipLaunchKernelGGL((gemm_bf16_kernel<G_PARTIAL, true, BM_ROWS>), grid, dim3(256), 0, stream, (const bf16_t*)A, lda,
                        (const bf16_t*)W, (const bf16_t*)Wu, ceil_div(K, 32), workspace, N, M, N, K, k_split);
   else
-    hipLaunchKernelGGL((gemm_bf16_kernel<G_PARTIAL, false>), grid, dim3(256), 0, stream, (const bf16_t*)A, lda,
+    hipLaunchKernelGGL((gemm_bf16_kernel<G_PARTIAL, false, BM_ROWS>), grid, dim3(256), 0, stream, (const bf16_t*)A, lda,
                        (const bf16_t*)W, (const bf16_t*)Wu, ceil_div(K, 32), workspace, N, M, N, K, k_split);
   APC_LAUNCH_CHECK();
   hipLaunchKernelGGL(gemm_finish_kernel, dim3(ceil_div(N, 256), M), dim3(256), 0, stream, workspace, k_split, M, N, mode,
