@@ -167,6 +167,9 @@ def main() -> int:
     ap.add_argument("--preset", default="llama-3.1-8b")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points and the prefill")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--only", choices=["decode", "prefill"], default=None,
+                    help="for profiling: only the decode steps at --batch (as --no-points), or only the 2,048-token "
+                         "prefill (prints its figures as the line's value)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
@@ -181,6 +184,19 @@ def main() -> int:
     layers = args.layers or full_layers
     klib.load("plain")
     klib.load("tuned")
+
+    if args.only == "decode":
+        args.no_points = True
+    if args.only == "prefill":
+        T = 2048
+        cfg, eng = build_engine(cfg_json, args.dtype, 1, T, 64, layers, use_graphs=not args.no_graphs)
+        psec = prefill_run(eng, cfg, T)
+        fl = prefill_flops(cfg, layers, T)
+        print(json.dumps({"metric": "prefill tok/s @ 2048 tokens", "value": round(T / psec, 1), "unit": "tok/s",
+                          "n_gpus": 1, "ms_per_step": round(psec * 1e3, 3), "dtype": args.dtype,
+                          "frac_of_mfma_peak": round(fl / psec / PEAK_FLOPS[args.dtype], 4),
+                          "config": {"model": args.preset, "layers": layers}}), flush=True)
+        return 0
 
     points = {}
     batches = [args.batch] + ([] if args.no_points else [b for b in (1, 64) if b != args.batch])
