@@ -31,7 +31,9 @@ def rnd(*shape, seed=0, scale=1.0):
 
 
 def tol(dtype):
-    return dict(atol=2e-5, rtol=1e-5) if dtype == "float32" else dict(atol=2e-2, rtol=2.0 ** -7)
+    """An output computed in 32-bit from exact inputs: float32 rounding noise, plus, if it is stored in bfloat16,
+    one rounding to nearest (half a unit in the 8th bit)."""
+    return dict(atol=2e-5, rtol=1e-5) if dtype == "float32" else dict(atol=2e-5, rtol=2.0 ** -9 * 1.01)
 
 
 def assert_part_close(got, exact, stored, dtype, what=""):
@@ -45,15 +47,6 @@ def assert_part_close(got, exact, stored, dtype, what=""):
     else:
         lim = 2.5 * np.abs(np.asarray(stored, np.float64) - exact).max() + 2.0 ** -8 * np.abs(exact).max()
         assert d <= lim, f"{what}: max diff {d:.3e}, limit {lim:.3e}"
-
-
-def one_step(lens_rows, page_tokens, needs, max_requests=4):
-    """A cache manager and storage for `needs`, and a packed step: sequence s has pos0 = lens_rows[s][0] rows already
-    committed and brings lens_rows[s][1] rows."""
-    from allpaca_amd.cache import CacheManager, CacheStorage
-    from allpaca_amd.engine.batch import Entry, pack_step
-    cm = CacheManager(needs, page_tokens, 64, max_requests)
-    return cm
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
