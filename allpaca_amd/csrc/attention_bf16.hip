@@ -5,7 +5,9 @@
 //   decode kernel    one row x one kv head (the H/Hk query heads of the group are the 16 rows of the MFMA
 //                    tile, so keys and values are read once per group); each wave is a "part" that covers
 //                    KW consecutive keys straight from global memory; parts are merged by a second kernel
-//                    in key order.
+//                    in key order.  (Merging in the same kernel, by the part that arrives last, was tried: the
+//                    device-wide fences it needs write back and invalidate the XCDs' L2 caches and cost ten
+//                    times what the second launch does.)
 // Cache pages: keys [kv_head][slot][d] (d contiguous), values [kv_head][d][slot] (slots contiguous): both
 // MFMA operands want the summed axis contiguous per lane, d for the scores and positions for the values.
 // Masking: a row at position p sees keys max(0, p - window + 1) .. p.  Scores are scaled on the finished
@@ -19,11 +21,6 @@
 constexpr int KT = 64;            // keys per tile in the prefill kernel
 constexpr int QT = 64;            // rows per tile in the prefill kernel (4 waves x 16)
 constexpr int KPAD = 8;
-
-// One wave writes LDS and then reads what its other lanes wrote.  The LDS serves a wave's accesses in the order
-// it issues them, so all that is needed is that the compiler keeps that order: a wave barrier (no wait on
-// outstanding global loads, unlike a fence, so loads issued ahead stay in flight).
-__device__ __forceinline__ void wave_lds_order() { __builtin_amdgcn_wave_barrier(); }
 
 // Both kernels compute the transposed products  S^T = K Q^T  and  O^T = V^T P^T : the MFMA result then holds, per
 // lane, 4 consecutive keys (or value elements) of ONE query row (row = lane % 16), so a row's maximum and sum

@@ -24,6 +24,11 @@ __device__ __forceinline__ bf16x8_t as_bf16x8(const Frag& f) { return __builtin_
 __device__ __forceinline__ Frag load_frag(const bf16_t* p) { return *reinterpret_cast<const Frag*>(p); }
 __device__ __forceinline__ Frag zero_frag() { Frag f; f.w[0] = f.w[1] = f.w[2] = f.w[3] = 0u; return f; }
 
+// One wave writes LDS and then reads what its other lanes wrote.  The LDS serves a wave's accesses in the order
+// it issues them, so all that is needed is that the compiler keeps that order: a wave barrier (no wait on
+// outstanding global loads, unlike a fence, so loads issued ahead stay in flight).
+__device__ __forceinline__ void wave_lds_order() { __builtin_amdgcn_wave_barrier(); }
+
 __device__ __forceinline__ floatx4 mfma16(const Frag& a, const Frag& b, floatx4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0);
 }

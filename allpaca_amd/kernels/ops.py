@@ -247,10 +247,17 @@ def prepare_matrix(w: torch.Tensor, run_dtype: torch.dtype):
     return w.contiguous()
 
 
-def linear(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False) -> None:
-    """out = a . w^T (or out += ..., out float32).  A tiled bfloat16 weight runs on the MFMA kernels."""
+def linear(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False, emit=None) -> None:
+    """out = a . w^T (or out += ..., out float32).  A tiled bfloat16 weight runs on the MFMA kernels.
+    `emit` (with accumulate): an object with `weight` (an RMS norm's) whose `raw` and `ss` are filled with what
+    that norm's next product needs, where there is a kernel for these sizes; else it is left as it is."""
     if isinstance(w, PackedWeight):
         from . import tuned
+        if emit is not None and accumulate:
+            left = tuned.gemm_emit_bf16(a, w, out, emit.weight)
+            if left is not None:
+                emit.raw, emit.ss = left
+                return
         tuned.gemm_bf16(a, w, out, accumulate)
     else:
         gemm_plain(a, w, out, accumulate)
@@ -267,6 +274,22 @@ def swiglu(h: torch.Tensor, w_gate_up, out: torch.Tensor) -> None:
     gu = torch.empty((T, 2 * F), dtype=torch.float32 if h.dtype == torch.float32 else out.dtype, device=h.device)
     gemm_plain(h, w_gate_up, gu)
     silu_mul(gu, out)
+
+
+def linear_pre(raw: torch.Tensor, ss: torch.Tensor, eps: float, w, out: torch.Tensor) -> bool:
+    """The product of a normalised row from what `linear(..., emit=...)` left; False if there is no kernel for
+    these sizes (nothing is done then)."""
+    if isinstance(w, PackedWeight) and not FORCE_PLAIN:
+        from . import tuned
+        return tuned.gemm_pre_bf16(raw, ss, eps, w, out)
+    return False
+
+
+def swiglu_pre(raw: torch.Tensor, ss: torch.Tensor, eps: float, w_gate_up, out: torch.Tensor) -> bool:
+    if isinstance(w_gate_up, tuple) and not FORCE_PLAIN:
+        from . import tuned
+        return tuned.swiglu_pre_bf16(raw, ss, eps, w_gate_up[0], w_gate_up[1], out)
+    return False
 
 
 def paged_attention(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,

@@ -86,6 +86,63 @@ def swiglu_bf16(h: torch.Tensor, wg: PackedWeight, wu: PackedWeight, out: torch.
                   _ops._stream()), "swiglu_bf16")
 
 
+def gemm_emit_bf16(a: torch.Tensor, w: PackedWeight, residual: torch.Tensor, g: torch.Tensor):
+    """residual += a . w^T, and for the RMS norm with weight g that reads the residual next: the row
+    bfloat16(residual * g) and the sums of residual^2 per band of 16 columns and row.  Returns (raw [M, N],
+    ss [16, ceil(N/16) rounded up to 4]) or None, with nothing done, for sizes the kernel does not take (more than 16 rows)."""
+    _ops._gpu(a, w.data, residual, g)
+    M, K = a.shape
+    N = w.N
+    if (M > SKINNY_MAX_ROWS or not _act_ok(a) or residual.dtype != torch.float32 or g.dtype != torch.float32
+            or g.numel() != N or not g.is_contiguous()):
+        return None
+    _ops._need(w.K == K and residual.shape == (M, N), f"gemm: a [{M}, {K}], w {w.shape}, residual {tuple(residual.shape)}")
+    raw = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
+    ss = torch.empty((16, -(-(-(-N // 16)) // 4) * 4), dtype=torch.float32, device=a.device)
+    L = _lib.load("tuned")
+    _lib.check(L.apc_skinny_gemm_emit_bf16(a.data_ptr(), _ops._rows(a, "a"), w.data.data_ptr(), residual.data_ptr(),
+                                           _ops._rows(residual, "residual"), M, N, K, g.data_ptr(), raw.data_ptr(), N,
+                                           ss.data_ptr(), _ops._stream()), "skinny_gemm_emit_bf16")
+    return raw, ss
+
+
+def _pre_ok(raw: torch.Tensor, ss: torch.Tensor, K: int) -> bool:
+    return (raw.shape[0] <= SKINNY_MAX_ROWS and _act_ok(raw) and ss.dtype == torch.float32 and ss.is_contiguous()
+            and tuple(ss.shape) == (16, -(-(-(-K // 16)) // 4) * 4))
+
+
+def gemm_pre_bf16(raw: torch.Tensor, ss: torch.Tensor, eps: float, w: PackedWeight, out: torch.Tensor) -> bool:
+    """out = (raw . w^T) / sqrt(sum(ss) / K + eps) for a row that `gemm_emit_bf16` left: the product of the
+    normalised row.  False, with nothing done, for sizes the kernel does not take."""
+    _ops._gpu(raw, ss, w.data, out)
+    M, K = raw.shape
+    if not _pre_ok(raw, ss, K) or out.dtype not in (torch.bfloat16, torch.float32):
+        return False
+    _ops._need(w.K == K and out.shape == (M, w.N), f"gemm: raw [{M}, {K}], w {w.shape}, out {tuple(out.shape)}")
+    L = _lib.load("tuned")
+    _lib.check(L.apc_skinny_gemm_pre_bf16(raw.data_ptr(), _ops._rows(raw, "raw"), ss.data_ptr(), -(-K // 16), float(eps),
+                                          w.data.data_ptr(), out.data_ptr(), _ops._rows(out, "out"), M, w.N, K,
+                                          0 if out.dtype == torch.bfloat16 else 1, _ops._stream()),
+               "skinny_gemm_pre_bf16")
+    return True
+
+
+def swiglu_pre_bf16(raw: torch.Tensor, ss: torch.Tensor, eps: float, wg: PackedWeight, wu: PackedWeight,
+                    out: torch.Tensor) -> bool:
+    """SwiGLU of the normalised row, from what `gemm_emit_bf16` left (see `gemm_pre_bf16`)."""
+    _ops._gpu(raw, ss, wg.data, wu.data, out)
+    M, K = raw.shape
+    F = out.shape[1]
+    if not _pre_ok(raw, ss, K) or out.dtype != torch.bfloat16:
+        return False
+    _ops._need(wg.shape == (F, K) and wu.shape == (F, K) and out.shape[0] == M, f"swiglu: weights must both be [{F}, {K}]")
+    L = _lib.load("tuned")
+    _lib.check(L.apc_skinny_swiglu_pre_bf16(raw.data_ptr(), _ops._rows(raw, "raw"), ss.data_ptr(), -(-K // 16),
+                                            float(eps), wg.data.data_ptr(), wu.data.data_ptr(), out.data_ptr(),
+                                            _ops._rows(out, "out"), M, F, K, _ops._stream()), "skinny_swiglu_pre_bf16")
+    return True
+
+
 def _keys_per_part(n_rows: int, n_kv_heads: int, max_context: int, page_tokens: int = 16) -> int:
     """Keys one wave covers in the decode kernel.  A wave that walks through many keys overlaps its loads
     with its work, so: the longest range that still leaves about a thousand waves on the chip (four per

@@ -71,8 +71,11 @@ class DecoderModel:
         T = step.n_rows
         x = torch.empty((T, self.spec.hidden_size), dtype=torch.float32, device=rt.device)
         self.embedding.forward(step.tokens, x)
-        for i, e in enumerate(self.spec.plan):
-            self.blocks[e.block].run(x, step, caches[i])
+        plan = self.spec.plan
+        left = None  # what a layer's last product left for the next layer's first norm
+        for i, e in enumerate(plan):
+            nxt = self.blocks[plan[i + 1].block].first_norm() if i + 1 < len(plan) else None
+            left = self.blocks[e.block].run(x, step, caches[i], pre=left, next_norm=nxt)
         R = step.n_logit_rows
         if R == 0:
             return None

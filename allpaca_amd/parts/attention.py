@@ -13,13 +13,15 @@ from typing import Dict, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedKV, Runtime, build_part, to_device
+from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedKV, Runtime, as_normed, build_part, to_device
 from .spec import ParamSpec, PartSpec
 
 
 @MIXERS.register("attention")
 class Attention(Mixer):
     graph_safe = True
+    takes_normed_input = True
+    emits_next_norm = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: Optional[PartSpec] = None, window: Optional[int] = None, scale: Optional[float] = None):
@@ -53,10 +55,11 @@ class Attention(Mixer):
         if self.position is not None:
             self.position.bind({}, rt)
 
-    def forward_add(self, h: torch.Tensor, step, cache, residual: torch.Tensor) -> None:
+    def forward_add(self, h, step, cache, residual: torch.Tensor, emit=None) -> None:
+        h = as_normed(h)
         T = h.shape[0]
         qkv = torch.empty((T, self.qkv_width), dtype=self.rt.dtype, device=h.device)
-        ops.linear(h, self.w_qkv, qkv)
+        h.linear(self.w_qkv, qkv)
         rot, table = (0, None)
         if self.position is not None:
             fused = self.position.fused()
@@ -71,7 +74,7 @@ class Attention(Mixer):
         attn = torch.empty((T, self.H * self.d), dtype=self.rt.dtype, device=h.device)
         ops.paged_attention(qkv, self.q_off, attn, self.H, self.Hk, self.d, cache.kv, cache.page_tokens,
                             cache.block_table, step, window=self.window or 0, scale=self.scale)
-        ops.linear(attn, self.w_o, residual, accumulate=True)
+        ops.linear(attn, self.w_o, residual, accumulate=True, emit=emit)
 
     def forward(self, h, step, cache):
         out = torch.zeros((h.shape[0], self.D), dtype=torch.float32, device=h.device)

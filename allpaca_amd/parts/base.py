@@ -79,6 +79,74 @@ class Norm(Part):
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
         raise NotImplementedError
 
+    def rms_params(self):
+        """(weight, eps) if this norm is x / sqrt(mean(x^2) + eps) * weight, which the products around it can
+        fold in; None for any other norm."""
+        return None
+
+
+class NormEmit:
+    """What a product that adds into the residual leaves for the RMS norm that reads the residual next: the row
+    bfloat16(x * weight) and sums of x^2, from which that norm's first product gets the product of the normalised
+    row without a kernel for the norm.  Made by an arrangement for a part that sets `emits_next_norm`; the part
+    passes it to `ops.linear(..., accumulate=True, emit=...)`.  Unfilled, it means nothing."""
+
+    def __init__(self, norm: "Norm"):
+        self.norm = norm
+        self.weight, self.eps = norm.rms_params()
+        self.raw: Optional[torch.Tensor] = None
+        self.ss: Optional[torch.Tensor] = None
+
+    @staticmethod
+    def of(norm: Optional["Norm"]) -> Optional["NormEmit"]:
+        return NormEmit(norm) if norm is not None and norm.rms_params() is not None else None
+
+    @property
+    def filled(self) -> bool:
+        return self.raw is not None
+
+
+class NormedInput:
+    """The normalised input of a part, not computed yet.  An arrangement hands it to a part that sets
+    `takes_normed_input`; the part's first product goes through `linear` / `swiglu`, which use what the
+    product before the norm left for it (`pre`, a filled `NormEmit`) and otherwise normalise first (`tensor()`)."""
+
+    def __init__(self, x: torch.Tensor, norm: Norm, dtype: torch.dtype, pre: Optional[NormEmit] = None):
+        self.x, self.norm, self.dtype = x, norm, dtype
+        self.shape, self.device = x.shape, x.device
+        self.pre = pre if pre is not None and pre.filled and pre.norm is norm else None
+        self._h: Optional[torch.Tensor] = None
+
+    def tensor(self) -> torch.Tensor:
+        if self._h is None:
+            self._h = torch.empty(self.x.shape, dtype=self.dtype, device=self.x.device)
+            self.norm.forward(self.x, self._h)
+        return self._h
+
+    def linear(self, w, out: torch.Tensor) -> None:
+        from ..kernels import ops
+        p = self.pre
+        if p is None or self._h is not None or not ops.linear_pre(p.raw, p.ss, p.eps, w, out):
+            ops.linear(self.tensor(), w, out)
+
+    def swiglu(self, w_gate_up, out: torch.Tensor) -> None:
+        from ..kernels import ops
+        p = self.pre
+        if p is None or self._h is not None or not ops.swiglu_pre(p.raw, p.ss, p.eps, w_gate_up, out):
+            ops.swiglu(self.tensor(), w_gate_up, out)
+
+
+def as_normed(h) -> "NormedInput":
+    """A part's input as a `NormedInput`, whether the arrangement gave one or a finished tensor."""
+    return h if isinstance(h, NormedInput) else _Finished(h)
+
+
+class _Finished(NormedInput):
+    def __init__(self, h: torch.Tensor):
+        self.x, self.norm, self.dtype, self.pre = None, None, h.dtype, None
+        self.shape, self.device = h.shape, h.device
+        self._h = h
+
 
 class PositionEncoding(Part):
     """`fused()` returns (rot, cos_sin table) when the encoding is a pairwise rotation
@@ -94,6 +162,10 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    # True if `forward_add` takes its input as a `NormedInput` (see there) instead of a tensor
+    takes_normed_input = False
+    # True if `forward_add` takes `emit=` (a `NormEmit` or None) for its product into the residual
+    emits_next_norm = False
     # True if `forward_add` only launches kernels whose arguments stay valid when the step's device
     # buffers are refilled (nothing read back to the host, no host-side branching on the batch): such a
     # mixer's decode steps can be replayed as a HIP graph
@@ -111,6 +183,9 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    takes_normed_input = False
+    emits_next_norm = False
+
     def forward(self, h: torch.Tensor, step) -> torch.Tensor:
         raise NotImplementedError
 

@@ -7,7 +7,7 @@ from typing import Dict, Mapping
 
 import torch
 
-from .base import ARRANGEMENTS, FEED_FORWARDS, MIXERS, NORMS, Part, build_part
+from .base import ARRANGEMENTS, FEED_FORWARDS, MIXERS, NORMS, NormEmit, NormedInput, Part, build_part
 from .spec import BlockSpec
 
 
@@ -20,7 +20,22 @@ class Block:
         self.parts: Dict[str, Part] = {}
         for role, pspec in spec.parts.items():
             self.parts[role] = build_part(arrangement.registries[role], pspec)
-        self.run = lambda x, step, cache: arrangement.run(self.parts, x, step, cache)
+        self.arrangement = arrangement
+        self.chains_norms = bool(getattr(arrangement, "chains_norms", False))
+
+    def run(self, x: torch.Tensor, step, cache, pre=None, next_norm=None):
+        """Runs the layer on the residual stream x.  `pre`: what the layer before left for this layer's first norm
+        (a filled `NormEmit`) or None; `next_norm`: the norm that reads x after this layer.  Returns what this
+        layer left for `next_norm`, or None.  Only arrangements with `chains_norms` take part in that."""
+        if self.chains_norms:
+            return self.arrangement.run(self.parts, x, step, cache, pre=pre, next_norm=next_norm)
+        self.arrangement.run(self.parts, x, step, cache)
+        return None
+
+    def first_norm(self):
+        """The norm that reads the residual stream first in this layer, if the layer can use what the product
+        before it leaves for that norm."""
+        return self.arrangement.first_norm(self.parts) if self.chains_norms else None
 
     @property
     def mixer(self):
@@ -45,12 +60,26 @@ class Block:
 class PreNorm:
     """x += mixer(norm(x)); x += ffn(norm(x))  (crates/allpaca-core/src/model.rs:8447-8455, 8667-8696)."""
     registries = {"mixer_norm": NORMS, "mixer": MIXERS, "ffn_norm": NORMS, "ffn": FEED_FORWARDS}
+    chains_norms = True
 
     @staticmethod
-    def run(parts, x: torch.Tensor, step, cache) -> None:
-        rt = parts["mixer"].rt
-        h = torch.empty(x.shape, dtype=rt.dtype, device=x.device)
-        parts["mixer_norm"].forward(x, h)
-        parts["mixer"].forward_add(h, step, cache, x)
-        parts["ffn_norm"].forward(x, h)
-        parts["ffn"].forward_add(h, step, x)
+    def first_norm(parts):
+        return parts["mixer_norm"] if parts["mixer"].takes_normed_input else None
+
+    @staticmethod
+    def run(parts, x: torch.Tensor, step, cache, pre=None, next_norm=None):
+        mixer, ffn = parts["mixer"], parts["ffn"]
+        rt = mixer.rt
+        h = NormedInput(x, parts["mixer_norm"], rt.dtype, pre)
+        emit = NormEmit.of(parts["ffn_norm"]) if mixer.emits_next_norm and ffn.takes_normed_input else None
+        if mixer.emits_next_norm:
+            mixer.forward_add(h if mixer.takes_normed_input else h.tensor(), step, cache, x, emit=emit)
+        else:
+            mixer.forward_add(h if mixer.takes_normed_input else h.tensor(), step, cache, x)
+        h = NormedInput(x, parts["ffn_norm"], rt.dtype, emit)
+        emit = NormEmit.of(next_norm) if ffn.emits_next_norm else None
+        if ffn.emits_next_norm:
+            ffn.forward_add(h if ffn.takes_normed_input else h.tensor(), step, x, emit=emit)
+        else:
+            ffn.forward_add(h if ffn.takes_normed_input else h.tensor(), step, x)
+        return emit if emit is not None and emit.filled else None

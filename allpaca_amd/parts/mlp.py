@@ -8,12 +8,15 @@ from typing import Dict, Mapping
 import torch
 
 from ..kernels import ops
-from .base import FEED_FORWARDS, FeedForward, Runtime, to_device
+from .base import FEED_FORWARDS, FeedForward, Runtime, as_normed, to_device
 from .spec import ParamSpec
 
 
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(FeedForward):
+    takes_normed_input = True
+    emits_next_norm = True
+
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.D, self.F = int(hidden_size), int(intermediate_size)
 
@@ -37,10 +40,11 @@ class SwiGLU(FeedForward):
             self.w_gate_up = (wg, wu)
         self.w_down = ops.prepare_matrix(to_device(tensors["down_proj.weight"], rt), rt.dtype)
 
-    def forward_add(self, h: torch.Tensor, step, residual: torch.Tensor) -> None:
+    def forward_add(self, h, step, residual: torch.Tensor, emit=None) -> None:
+        h = as_normed(h)
         act = torch.empty((h.shape[0], self.F), dtype=self.rt.dtype, device=h.device)
-        ops.swiglu(h, self.w_gate_up, act)
-        ops.linear(act, self.w_down, residual, accumulate=True)
+        h.swiglu(self.w_gate_up, act)
+        ops.linear(act, self.w_down, residual, accumulate=True, emit=emit)
 
     def forward(self, h, step):
         out = torch.zeros((h.shape[0], self.D), dtype=torch.float32, device=h.device)

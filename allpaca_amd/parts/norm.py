@@ -26,3 +26,6 @@ class RMSNorm(Norm):
 
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
         ops.rmsnorm_rows(x, self.weight, self.eps, out, rows)
+
+    def rms_params(self):
+        return self.weight, self.eps

@@ -112,6 +112,96 @@ def test_skinny_rows_together_equal_each_row_alone():
         assert torch.equal(some, tog[3:8])
 
 
+def bf16_round(a):
+    """float64 array rounded to bfloat16 (nearest even), as float64."""
+    return f64(torch.from_numpy(np.asarray(a, np.float32)).to(BF))
+
+
+def emit_reference(a, w, res, g):
+    """What the emitting product leaves: the new residual, the row bfloat16(residual * g), sums of squares."""
+    x = res + f64(a) @ f64(w).T
+    return x, bf16_round(x * f64(g)), (x ** 2).sum(axis=1, keepdims=True)
+
+
+@pytest.mark.parametrize("M,D,K", [(1, 64, 32), (8, 4096, 512), (16, 104, 1208), (5, 40, 72), (3, 8192, 264)])
+def test_product_into_the_residual_leaves_the_next_norms_row(M, D, K):
+    """residual += a . w^T; raw = bfloat16(residual * g); ss[band][row] = sum of residual^2 over the band."""
+    t = tuned()
+    a, w = gen(M, K, seed=1, dtype=BF).to(DEV), gen(D, K, seed=2, dtype=BF).to(DEV)
+    res = gen(M, D, seed=3, scale=2.0).to(DEV)
+    res[0] *= 30.0
+    g = (1 + 0.2 * gen(D, seed=4)).to(DEV)
+    x, raw_want, ss_want = emit_reference(a, w, f64(res), g)
+    left = t.gemm_emit_bf16(a, pack(w), res, g)
+    assert left is not None
+    raw, ss = left
+    check(f64(res), x, torch.float32)
+    bands = -(-D // 16)
+    assert tuple(ss.shape) == (16, -(-bands // 4) * 4) and tuple(raw.shape) == (M, D)
+    assert np.allclose(f64(ss)[:M, :bands].sum(axis=1), ss_want[:, 0], rtol=1e-5)
+    band = f64(ss)[:M, 1] if D >= 32 else None
+    if band is not None:
+        assert np.allclose(band, (x[:, 16:32] ** 2).sum(axis=1), rtol=1e-5, atol=1e-6)
+    # the rounding of x * g sits on a float32 x that is itself within float32 noise of the reference
+    d = np.abs(f64(raw) - raw_want)
+    assert (d <= 2.0 ** -7 * np.abs(raw_want) + 1e-6).all() and (d > 0).mean() < 0.01
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 40, 64), (8, 4096, 512), (16, 100, 1200), (5, 34, 72), (2, 36, 104), (3, 6144, 4096),
+                                   (16, 2050 * 16, 136), (7, 48, 8192)])
+def test_product_of_the_normalised_row_from_what_was_left(M, N, K):
+    """out = (raw . W^T) / sqrt(sum(ss) / K + eps), which is rmsnorm(x) . W^T up to the rounding of x * g."""
+    t = tuned()
+    x = f64(gen(M, K, seed=1, scale=3.0))
+    x[0, : K // 2] *= 40.0                               # rows of very different size: one root per row
+    g = f64(1 + 0.2 * gen(K, seed=2))
+    w = gen(N, K, seed=3, dtype=BF).to(DEV)
+    eps = 3e-4
+    raw64 = bf16_round(x * g)
+    raw = torch.from_numpy(raw64).to(BF).to(DEV)
+    bands = -(-K // 16)
+    xp = np.zeros((M, bands * 16)); xp[:, :K] = x
+    ss64 = np.full((16, -(-bands // 4) * 4), 1e30); ss64[:M, :bands] = (xp.reshape(M, bands, 16) ** 2).sum(axis=2)
+    ss64[M:, :bands] = 0.0                              # beyond the bands: never read, whatever it holds
+    ss = torch.from_numpy(ss64).float().to(DEV)
+    rstd = 1.0 / np.sqrt((x ** 2).mean(axis=1, keepdims=True) + eps)
+    want = (raw64 @ f64(w).T) * rstd
+    for out_dtype in (BF, torch.float32):
+        out = torch.full((M, N), 7.0, dtype=out_dtype, device=DEV)
+        assert t.gemm_pre_bf16(raw, ss, eps, pack(w), out)
+        check(f64(out), want, out_dtype)
+    exact = (x * rstd * g) @ f64(w).T
+    assert np.abs(f64(out) - exact).max() <= 2.0 ** -8 * np.abs(x * rstd * g).max() * np.abs(f64(w)).sum(axis=1).max()
+
+
+@pytest.mark.parametrize("M,F,K", [(1, 24, 64), (8, 176, 512), (16, 200, 112), (4, 14336 // 8, 1024)])
+def test_swiglu_of_the_normalised_row_from_what_was_left(M, F, K):
+    t = tuned()
+    x = f64(gen(M, K, seed=1, scale=2.0))
+    g = f64(1 + 0.2 * gen(K, seed=2))
+    w = gen(2 * F, K, seed=3, scale=0.3, dtype=BF).to(DEV)
+    eps = 1e-5
+    raw64 = bf16_round(x * g)
+    bands = -(-K // 16)
+    ss64 = np.zeros((16, -(-bands // 4) * 4)); ss64[:M, :bands] = (x.reshape(M, bands, 16) ** 2).sum(axis=2)
+    rstd = 1.0 / np.sqrt((x ** 2).mean(axis=1, keepdims=True) + eps)
+    out = torch.empty(M, F, dtype=BF, device=DEV)
+    assert t.swiglu_pre_bf16(torch.from_numpy(raw64).to(BF).to(DEV), torch.from_numpy(ss64).float().to(DEV), eps,
+                             pack(w[:F].contiguous()), pack(w[F:].contiguous()), out)
+    check(f64(out), P.silu(raw64 @ f64(w[:F]).T * rstd) * (raw64 @ f64(w[F:]).T * rstd), BF)
+
+
+def test_folded_norm_refuses_what_it_does_not_take():
+    t = tuned()
+    w = pack(gen(32, 64, dtype=BF).to(DEV))
+    g = torch.ones(32, device=DEV)
+    assert t.gemm_emit_bf16(gen(17, 64, dtype=BF).to(DEV), w, torch.zeros(17, 32, device=DEV), g) is None   # > 16 rows
+    ss = torch.zeros(16, 4, device=DEV)
+    out = torch.empty(17, 32, dtype=BF, device=DEV)
+    assert not t.gemm_pre_bf16(gen(17, 64, dtype=BF).to(DEV), ss, 1e-5, w, out)
+    assert not t.gemm_pre_bf16(gen(4, 64, dtype=BF).to(DEV), ss[:, :3], 1e-5, w, out[:4])                   # ss too short
+
+
 def test_embedding_from_the_tiled_table():
     from allpaca_amd.kernels import ops
     table = gen(515, 120, seed=1, dtype=BF).to(DEV)

@@ -32,8 +32,8 @@ def rnd(*shape, seed=0, scale=1.0):
 
 def tol(dtype):
     """An output computed in 32-bit from exact inputs: float32 rounding noise, plus, if it is stored in bfloat16,
-    one rounding to nearest (half a unit in the 8th bit)."""
-    return dict(atol=2e-5, rtol=1e-5) if dtype == "float32" else dict(atol=2e-5, rtol=2.0 ** -9 * 1.01)
+    one rounding to nearest (half a unit of an 8-bit significand: 2^-8 of the value at most)."""
+    return dict(atol=2e-5, rtol=1e-5) if dtype == "float32" else dict(atol=2e-5, rtol=2.0 ** -8 * 1.01)
 
 
 def assert_part_close(got, exact, stored, dtype, what=""):
