@@ -7,7 +7,9 @@
 //                    KW consecutive keys straight from global memory; parts are merged by a second kernel
 //                    in key order.  (Merging in the same kernel, by the part that arrives last, was tried: the
 //                    device-wide fences it needs write back and invalidate the XCDs' L2 caches and cost ten
-//                    times what the second launch does.)
+//                    times what the second launch does.  Turning q and k and writing the row's own key and value
+//                    into the cache inside this kernel, instead of in a kernel before it, was tried too: the
+//                    dependent loads it puts in front of the stream of keys cost more than that kernel.)
 // Cache pages: keys [kv_head][slot][d] (d contiguous), values [kv_head][d][slot] (slots contiguous): both
 // MFMA operands want the summed axis contiguous per lane, d for the scores and positions for the values.
 // Masking: a row at position p sees keys max(0, p - window + 1) .. p.  Scores are scaled on the finished
