@@ -124,13 +124,19 @@ def cmd_generate(args) -> int:
     for p, o in zip(prompts, outs):
         if args.json:
             print(json.dumps(dict(prompt_tokens=o.prompt_tokens, completion_tokens=o.completion_tokens,
-                                  token_ids=o.token_ids, finish_reason=o.finish_reason)))
+                                  token_ids=o.token_ids, finish_reason=o.finish_reason,
+                                  queue_ms=_ms(o.timing["queue"]), ttft_ms=_ms(o.timing["ttft"]),
+                                  itl_ms=_ms(o.timing["itl"]))))
         else:
             print(" ".join(str(t) for t in o.token_ids))
     n = sum(o.completion_tokens for o in outs)
     print(f"{n} tokens in {dt:.3f} s ({n / dt:.1f} tok/s), {engine.stats['steps']} steps, "
           f"{engine.stats['preemptions']} preemptions", file=sys.stderr)
     return 0
+
+
+def _ms(seconds):
+    return None if seconds is None else round(seconds * 1e3, 3)
 
 
 def main(argv: Optional[List[str]] = None) -> int:

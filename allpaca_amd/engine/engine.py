@@ -6,6 +6,7 @@ from __future__ import annotations
 
 import os
 import tempfile
+import time
 from typing import Dict, Iterator, List, Mapping, Optional, Sequence
 
 import torch
@@ -67,7 +68,7 @@ class Engine:
                              f"{self.runner.rt.max_positions} positions this engine was set up for")
         rid = self._next_id
         self._next_id += 1
-        req = Request(rid, prompt, params)
+        req = Request(rid, prompt, params, t_added=time.perf_counter())
         self.scheduler.add(req)
         self.requests[rid] = req
         return rid
@@ -91,8 +92,11 @@ class Engine:
             self.runner.storage.zero_slot(self.runner.cache.slot_of(req.id))
         if not plan.scheduled:
             return []
+        now = time.perf_counter()
         entries = []
         for s in plan.scheduled:
+            if s.request.t_first_scheduled is None:
+                s.request.t_first_scheduled = now
             toks = s.request.tokens[s.start:s.start + s.count]
             entries.append(Entry(s.request.id, toks, [s.count - 1] if s.samples else []))
         logits = self.runner.step(entries)
@@ -105,7 +109,9 @@ class Engine:
         if sampled:
             tokens = self.sampler.sample(logits, [s.request.params for s in sampled],
                                          [len(s.request.output) for s in sampled])
+            now = time.perf_counter()       # the token ids are on the host: the step is over
             for s, tok in zip(sampled, tokens):
+                s.request.t_tokens.append(now)
                 reason = self.scheduler.append_token(s.request, tok)
                 events.append(TokenEvent(s.request.id, int(tok), reason, len(s.request.prompt)))
                 if reason is not None:
@@ -135,5 +141,5 @@ class Engine:
         out = []
         for i in ids:
             r = self.requests.pop(i)
-            out.append(GenerationOutput(list(r.output), len(r.prompt), len(r.output), r.finish_reason))
+            out.append(GenerationOutput(list(r.output), len(r.prompt), len(r.output), r.finish_reason, r.timing()))
         return out

@@ -46,6 +46,19 @@ class Request:
     finish_reason: Optional[str] = None
     preemptions: int = 0
     order: int = 0                    # admission order (for the choice of a victim)
+    # times (time.perf_counter): added, first scheduled, every token; the reference keeps a mean wait per poll and
+    # counts of prefill and decode picks (crates/allpaca-core/src/engine.rs:3848-3872), here per request
+    t_added: float = 0.0
+    t_first_scheduled: Optional[float] = None
+    t_tokens: List[float] = field(default_factory=list)
+
+    def timing(self) -> dict:
+        """Seconds: `queue` (added to first scheduled), `ttft` (added to first token), `itl` (mean time between
+        tokens after the first); None where the event has not happened."""
+        queue = None if self.t_first_scheduled is None else self.t_first_scheduled - self.t_added
+        ttft = self.t_tokens[0] - self.t_added if self.t_tokens else None
+        itl = ((self.t_tokens[-1] - self.t_tokens[0]) / (len(self.t_tokens) - 1)) if len(self.t_tokens) > 1 else None
+        return {"queue": queue, "ttft": ttft, "itl": itl}
 
     @property
     def tokens(self) -> List[int]:

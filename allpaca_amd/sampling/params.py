@@ -48,3 +48,4 @@ class GenerationOutput:
     prompt_tokens: int
     completion_tokens: int
     finish_reason: str
+    timing: Optional[dict] = None     # seconds: queue, ttft, itl (see `Request.timing`)

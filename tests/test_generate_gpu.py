@@ -129,6 +129,7 @@ def test_command_line_generate():
     assert r.returncode == 0, r.stderr[-2000:]
     lines = [json.loads(ln) for ln in r.stdout.strip().splitlines()]
     assert [ln["token_ids"] for ln in lines] == [P.greedy_generate(cfg, w, p, 6) for p in (p1, p2)]
+    assert all(0 <= ln["queue_ms"] <= ln["ttft_ms"] and ln["itl_ms"] > 0 for ln in lines)   # times per request
     r = subprocess.run(cmd[:2] + ["generate", "--synthetic", "--cpu-only", "--prompt-tokens", "1"],
                        capture_output=True, text=True, timeout=120)
     assert r.returncode == 2 and "no CPU path" in r.stderr or "not available" in r.stderr
