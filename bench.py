@@ -97,6 +97,11 @@ def kv_bytes_per_token(cfg, layers, elem=2):
     return layers * 2 * cfg.num_key_value_heads * cfg.head_dim * elem
 
 
+def decode_during_prefill(batch, context, chunk=2048):
+    """Tokens the first request may decode while the other prompts are still running in portions of `chunk`."""
+    return batch * -(-context // chunk) + batch
+
+
 def decode_run(eng, cfg, batch, context, steps, warmup):
     """Fills `batch` requests to `context` tokens, then times `steps` decode steps."""
     import numpy as np
@@ -105,7 +110,7 @@ def decode_run(eng, cfg, batch, context, steps, warmup):
     from allpaca_amd.sampling import GenerationParams
     rng = np.random.default_rng(0)
     # requests that finish their prompt first decode while the others still prefill: leave room for that
-    gp = GenerationParams(max_tokens=warmup + steps + 2 * batch + 8, temperature=0.0)
+    gp = GenerationParams(max_tokens=warmup + steps + decode_during_prefill(batch, context) + 8, temperature=0.0)
     for _ in range(batch):
         eng.add_request(rng.integers(0, cfg.vocab_size, size=context - 1).tolist(), gp)
     while any(not r.decoding for r in eng.scheduler.running) or eng.scheduler.waiting:
@@ -204,7 +209,7 @@ def main() -> int:
     prefill = None
     roof = None
     for b in batches:
-        extra = args.warmup + args.steps + 2 * b + 16
+        extra = args.warmup + args.steps + decode_during_prefill(b, args.context) + 16
         cfg, eng = build_engine(cfg_json, args.dtype, max(b, 1), args.context, extra, layers,
                                 use_graphs=not args.no_graphs)
         sec = decode_run(eng, cfg, b, args.context, args.steps, args.warmup)
