@@ -43,7 +43,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
   constexpr int AP = BM / 32;          // 16-byte pieces of A per thread and K step
   constexpr int WM = BM / 64;          // 32-row accumulators of a wave along M
   constexpr int PIECES = AP + 4;       // pieces of A and W per thread and K step
-  constexpr int PER_GROUP = PIECES / 4;
+  constexpr int PER_GROUP = (PIECES + 3) / 4;
   __shared__ __attribute__((aligned(16))) bf16_t As[2][BM * LDS_ROW];
   __shared__ __attribute__((aligned(16))) bf16_t Ws[2][BN * LDS_ROW];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
@@ -132,7 +132,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
     for (int kk = 0; kk < BK / 16; ++kk) {
       if constexpr (decltype(LD)::value) {
 #pragma unroll
-        for (int j = kk * PER_GROUP; j < (kk + 1) * PER_GROUP; ++j) load_piece(ld, kt_load, j);
+        for (int j = kk * PER_GROUP; j < (kk + 1) * PER_GROUP; ++j)
+          if (j < PIECES) load_piece(ld, kt_load, j);
       }
       Frag fa[WM], fw[2];
 #pragma unroll
@@ -150,7 +151,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
         for (int b = 0; b < 2; ++b) acc[a][b] = mfma32(fa[a], fw[b], acc[a][b]);
       if constexpr (decltype(ST)::value) {
 #pragma unroll
-        for (int j = kk * PER_GROUP; j < (kk + 1) * PER_GROUP; ++j) store_piece(st, buf ^ 1, j);
+        for (int j = kk * PER_GROUP; j < (kk + 1) * PER_GROUP; ++j)
+          if (j < PIECES) store_piece(st, buf ^ 1, j);
       }
       __builtin_amdgcn_sched_barrier(0);  // keeps each group's memory work in its group
     }
@@ -276,13 +278,19 @@ APC_EXPORT int apc_gemm_splitk_bf16(const void* A, int lda, const void* W, const
   if (K % 8 || lda % 8 || !aligned16(A) || !aligned16(W) || (Wu && !aligned16(Wu))) return APC_ERR_UNSUPPORTED;
   const int n_mats = Wu ? 2 : 1;
   if (k_split * n_mats > 65535) return APC_ERR_BAD_ARG;
-  const dim3 grid(ceil_div(N, BN), ceil_div(M, BM_ROWS), k_split * n_mats);
-  if (K % BK == 0)
-    hipLaunchKernelGGL((gemm_bf16_kernel<G_PARTIAL, true, BM_ROWS>), grid, dim3(256), 0, stream, (const bf16_t*)A, lda,
-                       (const bf16_t*)W, (const bf16_t*)Wu, ceil_div(K, 32), workspace, N, M, N, K, k_split);
-  else
-    hipLaunchKernelGGL((gemm_bf16_kernel<G_PARTIAL, false, BM_ROWS>), grid, dim3(256), 0, stream, (const bf16_t*)A, lda,
-                       (const bf16_t*)W, (const bf16_t*)Wu, ceil_div(K, 32), workspace, N, M, N, K, k_split);
+  // up to 64 rows: tiles of 64 rows (half the loads of activations and half the MFMAs of a 128-row tile)
+#define PARTIAL_LAUNCH(EVEN_, BM_)                                                                                  \
+  hipLaunchKernelGGL((gemm_bf16_kernel<G_PARTIAL, EVEN_, BM_>), dim3(ceil_div(N, BN), ceil_div(M, BM_), k_split * n_mats), \
+                     dim3(256), 0, stream, (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)Wu, ceil_div(K, 32), \
+                     workspace, N, M, N, K, k_split)
+  if (M <= 64) {
+    if (K % BK == 0) PARTIAL_LAUNCH(true, 64);
+    else PARTIAL_LAUNCH(false, 64);
+  } else {
+    if (K % BK == 0) PARTIAL_LAUNCH(true, BM_ROWS);
+    else PARTIAL_LAUNCH(false, BM_ROWS);
+  }
+#undef PARTIAL_LAUNCH
   APC_LAUNCH_CHECK();
   hipLaunchKernelGGL(gemm_finish_kernel, dim3(ceil_div(N, 256), M), dim3(256), 0, stream, workspace, k_split, M, N, mode,
                      C, ldc);
