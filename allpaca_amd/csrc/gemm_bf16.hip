@@ -246,32 +246,67 @@ static int launch_gemm(const bf16_t* A, int lda, const bf16_t* W, const bf16_t* 
   return 0;
 }
 
+// What the folded RMS norm needs in the finishing kernel (see skinny_gemm_bf16.hip for the idea).
+// PRE: the activations were the row bfloat16(x * g) that an emitting product left; pre_ss[m][pre_parts] are that
+// product's sums of x^2 per row and block of 256 columns; the sums of this product are scaled by
+// 1 / sqrt(sum(pre_ss[m]) / K + eps).  EMIT (mode G_ACC_F32): beside C = x the kernel writes raw[m, n] =
+// bfloat16(x * g[n]) and emit_ss[m][blocks of 256 columns] = sums of x^2.
+struct FinishNorm {
+  const float* pre_ss;
+  int pre_parts;
+  float eps;
+  const float* g;
+  bf16_t* raw;
+  int ld_raw;
+  float* emit_ss;
+};
+
 // Sums the float32 sums that G_PARTIAL blocks left ([which][slice][M][N], slices in order) and finishes:
 // store bfloat16 / float32, add into a float32 residual, or SwiGLU of the two matrices' sums.
+template <bool PRE, bool EMIT>
 __global__ __launch_bounds__(256) void gemm_finish_kernel(const float* __restrict__ partials, int k_split, int M, int N,
-                                                          int mode, void* __restrict__ C, int ldc) {
+                                                          int K, int mode, void* __restrict__ C, int ldc,
+                                                          FinishNorm norm) {
+  __shared__ float red[4];
   const int n = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
-  if (n >= N) return;
+  const bool on = n < N;
+  float rstd = 1.f;
+  if constexpr (PRE) {  // pre_parts <= 256: one value a thread, added in a fixed order
+    const float v = threadIdx.x < norm.pre_parts ? norm.pre_ss[(size_t)m * norm.pre_parts + threadIdx.x] : 0.f;
+    rstd = 1.0f / sqrtf(block_sum<256>(v, red) / (float)K + norm.eps);
+  }
   const size_t plane = (size_t)M * N;
-  const float* src = partials + (size_t)m * N + n;
+  const float* src = partials + (size_t)m * N + (on ? n : 0);
   float g = 0.f;
   for (int s = 0; s < k_split; ++s) g += src[s * plane];
+  g *= rstd;
   const size_t o = (size_t)m * ldc + n;
-  if (mode == G_STORE_BF16) ((bf16_t*)C)[o] = float_to_bf16(g);
-  else if (mode == G_STORE_F32) ((float*)C)[o] = g;
-  else if (mode == G_ACC_F32) ((float*)C)[o] += g;
-  else {
-    float u = 0.f;
-    for (int s = 0; s < k_split; ++s) u += src[(k_split + s) * plane];
-    ((bf16_t*)C)[o] = float_to_bf16(silu_f(g) * u);
+  float sq = 0.f;
+  if (on) {
+    if (mode == G_STORE_BF16) ((bf16_t*)C)[o] = float_to_bf16(g);
+    else if (mode == G_STORE_F32) ((float*)C)[o] = g;
+    else if (mode == G_ACC_F32) {
+      const float x = ((float*)C)[o] + g;
+      ((float*)C)[o] = x;
+      if constexpr (EMIT) {
+        norm.raw[(size_t)m * norm.ld_raw + n] = float_to_bf16(x * norm.g[n]);
+        sq = x * x;
+      }
+    } else {
+      float u = 0.f;
+      for (int s = 0; s < k_split; ++s) u += src[(k_split + s) * plane];
+      ((bf16_t*)C)[o] = float_to_bf16(silu_f(g) * (u * rstd));
+    }
+  }
+  if constexpr (EMIT) {
+    const float total = block_sum<256>(sq, red);
+    if (threadIdx.x == 0) norm.emit_ss[(size_t)m * gridDim.x + blockIdx.x] = total;
   }
 }
 
-// Product for 17..128 rows: K is cut into `k_split` slices that different blocks multiply, so that matrices with
-// few output columns still give the chip enough blocks; `workspace` holds (Wu ? 2 : 1) * k_split * M * N floats.
-// mode as below, or 3 for SwiGLU (W = gate, Wu = up).
-APC_EXPORT int apc_gemm_splitk_bf16(const void* A, int lda, const void* W, const void* Wu, void* C, int ldc, int M,
-                                    int N, int K, int mode, int k_split, float* workspace, hipStream_t stream) {
+static int launch_splitk(const void* A, int lda, const void* W, const void* Wu, void* C, int ldc, int M, int N, int K,
+                         int mode, int k_split, float* workspace, int pre, int emit, FinishNorm norm,
+                         hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || lda < K || ldc < N || k_split < 1 || !workspace || M > 65535) return APC_ERR_BAD_ARG;
   if (mode < 0 || mode > G_SWIGLU || (mode == G_SWIGLU) != (Wu != nullptr)) return APC_ERR_BAD_ARG;
@@ -292,10 +327,45 @@ APC_EXPORT int apc_gemm_splitk_bf16(const void* A, int lda, const void* W, const
   }
 #undef PARTIAL_LAUNCH
   APC_LAUNCH_CHECK();
-  hipLaunchKernelGGL(gemm_finish_kernel, dim3(ceil_div(N, 256), M), dim3(256), 0, stream, workspace, k_split, M, N, mode,
-                     C, ldc);
+  const dim3 grid(ceil_div(N, 256), M);
+#define FINISH(PRE_, EMIT_)                                                                                     \
+  hipLaunchKernelGGL((gemm_finish_kernel<PRE_, EMIT_>), grid, dim3(256), 0, stream, workspace, k_split, M, N, K, mode, \
+                     C, ldc, norm)
+  if (pre) FINISH(true, false);
+  else if (emit) FINISH(false, true);
+  else FINISH(false, false);
+#undef FINISH
   APC_LAUNCH_CHECK();
   return 0;
+}
+
+// Product for 17..128 rows: K is cut into `k_split` slices that different blocks multiply, so that matrices with
+// few output columns still give the chip enough blocks; `workspace` holds (Wu ? 2 : 1) * k_split * M * N floats.
+// mode as below, or 3 for SwiGLU (W = gate, Wu = up).
+APC_EXPORT int apc_gemm_splitk_bf16(const void* A, int lda, const void* W, const void* Wu, void* C, int ldc, int M,
+                                    int N, int K, int mode, int k_split, float* workspace, hipStream_t stream) {
+  return launch_splitk(A, lda, W, Wu, C, ldc, M, N, K, mode, k_split, workspace, 0, 0, FinishNorm{}, stream);
+}
+
+// C += A . W^T into the float32 residual, and for the RMS norm (weight g) that reads C next: raw[m, n] =
+// bfloat16(C[m, n] * g[n]) and ss[m][ceil(N / 256)] = sums of C^2 per row and block of 256 columns.
+APC_EXPORT int apc_gemm_splitk_emit_bf16(const void* A, int lda, const void* W, void* C, int ldc, int M, int N, int K,
+                                         int k_split, float* workspace, const float* g, void* raw, int ld_raw,
+                                         float* ss, hipStream_t stream) {
+  if (!g || !raw || !ss || ld_raw < N) return APC_ERR_BAD_ARG;
+  const FinishNorm norm{nullptr, 0, 0.f, g, (bf16_t*)raw, ld_raw, ss};
+  return launch_splitk(A, lda, W, nullptr, C, ldc, M, N, K, G_ACC_F32, k_split, workspace, 0, 1, norm, stream);
+}
+
+// The storing products (mode 0, 1 or 3) on a row that apc_gemm_splitk_emit_bf16 left: A = raw [M, K],
+// ss = [M][ss_parts] sums of x^2 (ss_parts <= 256); the sums are scaled by 1 / sqrt(sum(ss[m]) / K + eps).
+APC_EXPORT int apc_gemm_splitk_pre_bf16(const void* A, int lda, const float* ss, int ss_parts, float eps,
+                                        const void* W, const void* Wu, void* C, int ldc, int M, int N, int K, int mode,
+                                        int k_split, float* workspace, hipStream_t stream) {
+  if (!ss || ss_parts <= 0 || mode == G_ACC_F32) return APC_ERR_BAD_ARG;
+  if (ss_parts > 256) return APC_ERR_UNSUPPORTED;
+  const FinishNorm norm{ss, ss_parts, eps, nullptr, nullptr, 0, nullptr};
+  return launch_splitk(A, lda, W, Wu, C, ldc, M, N, K, mode, k_split, workspace, 1, 0, norm, stream);
 }
 
 // W: tiled layout of an [N, K] matrix.  mode: 0 store bfloat16, 1 store float32, 2 add into float32

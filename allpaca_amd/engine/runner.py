@@ -9,6 +9,7 @@ mixes a prompt portion with decode rows in one of them
 (crates/allpaca-core/src/engine.rs:5451-5607); this is the one generalisation."""
 from __future__ import annotations
 
+import gc
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
@@ -176,8 +177,17 @@ class DecodeGraph:
         torch.cuda.current_stream(dev).wait_stream(side)
         torch.cuda.synchronize(dev)
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
-            self.logits = runner.model.forward(self.info, views)
+        # No garbage collection while the stream is capturing: a collection may free device objects of engines that
+        # are no longer used (other graphs, events), which is not allowed during a capture and ends the process.
+        gc_was_on = gc.isenabled()
+        gc.collect()
+        gc.disable()
+        try:
+            with torch.cuda.graph(self.graph):
+                self.logits = runner.model.forward(self.info, views)
+        finally:
+            if gc_was_on:
+                gc.enable()
         torch.cuda.synchronize(dev)
 
     def _part(self, i: int) -> np.ndarray:

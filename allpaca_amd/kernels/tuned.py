@@ -89,15 +89,29 @@ def swiglu_bf16(h: torch.Tensor, wg: PackedWeight, wu: PackedWeight, out: torch.
 def gemm_emit_bf16(a: torch.Tensor, w: PackedWeight, residual: torch.Tensor, g: torch.Tensor):
     """residual += a . w^T, and for the RMS norm with weight g that reads the residual next: the row
     bfloat16(residual * g) and the sums of residual^2 per band of 16 columns and row.  Returns (raw [M, N],
-    ss [16, ceil(N/16) rounded up to 4]) or None, with nothing done, for sizes the kernel does not take (more than 16 rows)."""
+    ss) or None, with nothing done, for sizes no kernel takes.  ss is [16, ceil(N/16) rounded up to 4] from the
+    streaming kernel (up to 16 rows) and [M, ceil(N/256)] from the tiled kernel with K in slices (17..128 rows); the
+    products below take either."""
     _ops._gpu(a, w.data, residual, g)
     M, K = a.shape
     N = w.N
-    if (M > SKINNY_MAX_ROWS or not _act_ok(a) or residual.dtype != torch.float32 or g.dtype != torch.float32
+    if (M > SPLITK_MAX_ROWS or not _act_ok(a) or residual.dtype != torch.float32 or g.dtype != torch.float32
             or g.numel() != N or not g.is_contiguous()):
         return None
     _ops._need(w.K == K and residual.shape == (M, N), f"gemm: a [{M}, {K}], w {w.shape}, residual {tuple(residual.shape)}")
     raw = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
+    if M > SKINNY_MAX_ROWS:   # the tiled kernel with K in slices: sums per row and block of 256 columns
+        ks = _k_split(M, N, K)
+        if ks == 1:
+            return None
+        ss = torch.empty((M, -(-N // 256)), dtype=torch.float32, device=a.device)
+        ws = torch.empty(ks * M * N, dtype=torch.float32, device=a.device)
+        L = _lib.load("tuned")
+        _lib.check(L.apc_gemm_splitk_emit_bf16(a.data_ptr(), _ops._rows(a, "a"), w.data.data_ptr(), residual.data_ptr(),
+                                               _ops._rows(residual, "residual"), M, N, K, ks, ws.data_ptr(),
+                                               g.data_ptr(), raw.data_ptr(), N, ss.data_ptr(), _ops._stream()),
+                   "gemm_splitk_emit_bf16")
+        return raw, ss
     ss = torch.empty((16, -(-(-(-N // 16)) // 4) * 4), dtype=torch.float32, device=a.device)
     L = _lib.load("tuned")
     _lib.check(L.apc_skinny_gemm_emit_bf16(a.data_ptr(), _ops._rows(a, "a"), w.data.data_ptr(), residual.data_ptr(),
@@ -111,14 +125,36 @@ def _pre_ok(raw: torch.Tensor, ss: torch.Tensor, K: int) -> bool:
             and tuple(ss.shape) == (16, -(-(-(-K // 16)) // 4) * 4))
 
 
+def _pre_splitk(raw: torch.Tensor, ss: torch.Tensor, eps: float, w, wu, out: torch.Tensor, n_cols: int, mode: int) -> bool:
+    """The same on the tiled kernel with K in slices (17..128 rows): ss is [M, ceil(K / 256)]."""
+    M, K = raw.shape
+    if not (SKINNY_MAX_ROWS < M <= SPLITK_MAX_ROWS and _act_ok(raw) and ss.dtype == torch.float32
+            and ss.is_contiguous() and tuple(ss.shape) == (M, -(-K // 256)) and ss.shape[1] <= 256):
+        return False
+    ks = _k_split(M, n_cols * (2 if wu is not None else 1), K)
+    if ks == 1 and wu is None:
+        return False
+    ws = torch.empty((2 if wu is not None else 1) * ks * M * n_cols, dtype=torch.float32, device=raw.device)
+    L = _lib.load("tuned")
+    _lib.check(L.apc_gemm_splitk_pre_bf16(raw.data_ptr(), _ops._rows(raw, "raw"), ss.data_ptr(), ss.shape[1], float(eps),
+                                          w.data.data_ptr(), wu.data.data_ptr() if wu is not None else 0, out.data_ptr(),
+                                          _ops._rows(out, "out"), M, n_cols, K, mode, ks, ws.data_ptr(), _ops._stream()),
+               "gemm_splitk_pre_bf16")
+    return True
+
+
 def gemm_pre_bf16(raw: torch.Tensor, ss: torch.Tensor, eps: float, w: PackedWeight, out: torch.Tensor) -> bool:
     """out = (raw . w^T) / sqrt(sum(ss) / K + eps) for a row that `gemm_emit_bf16` left: the product of the
     normalised row.  False, with nothing done, for sizes the kernel does not take."""
     _ops._gpu(raw, ss, w.data, out)
     M, K = raw.shape
-    if not _pre_ok(raw, ss, K) or out.dtype not in (torch.bfloat16, torch.float32):
+    if out.dtype not in (torch.bfloat16, torch.float32):
         return False
     _ops._need(w.K == K and out.shape == (M, w.N), f"gemm: raw [{M}, {K}], w {w.shape}, out {tuple(out.shape)}")
+    if M > SKINNY_MAX_ROWS:
+        return _pre_splitk(raw, ss, eps, w, None, out, w.N, 0 if out.dtype == torch.bfloat16 else 1)
+    if not _pre_ok(raw, ss, K):
+        return False
     L = _lib.load("tuned")
     _lib.check(L.apc_skinny_gemm_pre_bf16(raw.data_ptr(), _ops._rows(raw, "raw"), ss.data_ptr(), -(-K // 16), float(eps),
                                           w.data.data_ptr(), out.data_ptr(), _ops._rows(out, "out"), M, w.N, K,
@@ -133,9 +169,13 @@ def swiglu_pre_bf16(raw: torch.Tensor, ss: torch.Tensor, eps: float, wg: PackedW
     _ops._gpu(raw, ss, wg.data, wu.data, out)
     M, K = raw.shape
     F = out.shape[1]
-    if not _pre_ok(raw, ss, K) or out.dtype != torch.bfloat16:
+    if out.dtype != torch.bfloat16:
         return False
     _ops._need(wg.shape == (F, K) and wu.shape == (F, K) and out.shape[0] == M, f"swiglu: weights must both be [{F}, {K}]")
+    if M > SKINNY_MAX_ROWS:
+        return _pre_splitk(raw, ss, eps, wg, wu, out, F, 3)
+    if not _pre_ok(raw, ss, K):
+        return False
     L = _lib.load("tuned")
     _lib.check(L.apc_skinny_swiglu_pre_bf16(raw.data_ptr(), _ops._rows(raw, "raw"), ss.data_ptr(), -(-K // 16),
                                             float(eps), wg.data.data_ptr(), wu.data.data_ptr(), out.data_ptr(),
