@@ -4,6 +4,8 @@
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 2048] [--layers L]
 
 A step is one decode step of the whole engine (schedule, batch upload, model, sampling, token ids back).
+The engine is set up for sequences of up to 8,192 tokens (--max-context), page size 16; the timed decode steps
+run with every sequence at 2,048 tokens (--context).
 Prints one JSON line: `value` = decoded tokens per second at the given batch; `prefill` = a 2,048-token
 prompt in one step; `roofline` = bytes a decode step has to read (every weight once, and the cache of the
 live requests) over its time, against 8 TB/s; `points` = decode at batch 1 and 64.  The way of reporting
@@ -23,7 +25,7 @@ HBM_PEAK_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 
-def build_engine(cfg_json, dtype, batch, context, extra_tokens, layers, seed=0, use_graphs=True):
+def build_engine(cfg_json, dtype, batch, context, extra_tokens, layers, seed=0, use_graphs=True, max_context=0):
     """An engine on random weights made directly on the GPU (no model folder is written for 16 GB)."""
     import torch
 
@@ -42,7 +44,8 @@ def build_engine(cfg_json, dtype, batch, context, extra_tokens, layers, seed=0, 
     model = DecoderModel(spec)
     tdt = torch.bfloat16 if dtype == "bf16" else torch.float32
     page = 16
-    per_seq = -(-(context + extra_tokens) // page) * page
+    # every sequence may grow to `max_context` tokens (positions, block table, pages of the pool)
+    per_seq = -(-max(context + extra_tokens, max_context) // page) * page
     ec = EngineConfig(dtype="bfloat16" if dtype == "bf16" else "float32", page_tokens=page,
                       num_pages=batch * per_seq // page + 8, max_active_requests=max(batch, 1),
                       max_batch_tokens=2048, chunk_tokens=2048, use_graphs=use_graphs)
@@ -166,7 +169,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--context", type=int, default=2048)
+    ap.add_argument("--context", type=int, default=2048, help="tokens every sequence holds when the decode steps are timed")
+    ap.add_argument("--max-context", type=int, default=8192,
+                    help="tokens a sequence may grow to: positions, block tables and the page pool are made for it")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0: all)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--preset", default="llama-3.1-8b")
@@ -194,7 +199,8 @@ def main() -> int:
         args.no_points = True
     if args.only == "prefill":
         T = 2048
-        cfg, eng = build_engine(cfg_json, args.dtype, 1, T, 64, layers, use_graphs=not args.no_graphs)
+        cfg, eng = build_engine(cfg_json, args.dtype, 1, T, 64, layers, use_graphs=not args.no_graphs,
+                                max_context=args.max_context)
         psec = prefill_run(eng, cfg, T)
         fl = prefill_flops(cfg, layers, T)
         print(json.dumps({"metric": "prefill tok/s @ 2048 tokens", "value": round(T / psec, 1), "unit": "tok/s",
@@ -211,7 +217,7 @@ def main() -> int:
     for b in batches:
         extra = args.warmup + args.steps + decode_during_prefill(b, args.context) + 16
         cfg, eng = build_engine(cfg_json, args.dtype, max(b, 1), args.context, extra, layers,
-                                use_graphs=not args.no_graphs)
+                                use_graphs=not args.no_graphs, max_context=args.max_context)
         sec = decode_run(eng, cfg, b, args.context, args.steps, args.warmup)
         ms[b] = sec * 1e3
         if b == args.batch:
@@ -245,7 +251,8 @@ def main() -> int:
             "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
             "rope_theta": cfg.rope_theta, "rope_scaling_factor": cfg.rope_scaling.factor if cfg.rope_scaling else 1.0,
             "rms_norm_eps": cfg.rms_norm_eps, "tied_head": cfg.tie_word_embeddings, "global_batch": args.batch,
-            "seq_len": args.context, "page_tokens": 16, "parallelism": "single GPU",
+            "seq_len": args.context, "max_context": max(args.max_context, args.context), "page_tokens": 16,
+            "parallelism": "single GPU",
             "graphs": not args.no_graphs,
         },
     }
