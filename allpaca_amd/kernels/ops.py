@@ -152,6 +152,17 @@ def rope_kv_write(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads
         _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
               "block table must be contiguous int32 [segments, blocks]")
         max_blocks = block_table.shape[1]
+    if (not FORCE_PLAIN and qkv.dtype == torch.bfloat16 and (cache is None or cache.dtype == torch.bfloat16)
+            and head_dim % 8 == 0 and rot % 16 == 0 and ld % 8 == 0 and q_off % 8 == 0 and k_off % 8 == 0
+            and v_off % 8 == 0 and qkv.data_ptr() % 16 == 0):
+        # the same operation 16 bytes a lane (library `tuned`)
+        _lib.check(_lib.load("tuned").apc_rope_kv_write_bf16(
+            qkv.data_ptr(), ld, q_off, k_off, v_off, T, n_heads, n_kv_heads, head_dim, rot,
+            cos_sin.data_ptr() if rot else 0, _i32(positions, T, "positions"),
+            _i32(row_seg, T, "row_seg") if row_seg is not None else 0,
+            block_table.data_ptr() if block_table is not None else 0, max_blocks,
+            cache.data_ptr() if cache is not None else 0, page_tokens, _stream()), "rope_kv_write_bf16")
+        return
     L = _lib.load("plain")
     _lib.check(L.apc_rope_kv_write(
         qkv.data_ptr(), _code(qkv), ld, q_off, k_off, v_off, T, n_heads, n_kv_heads, head_dim, rot,

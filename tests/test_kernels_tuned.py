@@ -274,6 +274,48 @@ def test_swiglu_bf16(M, F, K):
     check(f64(out), P.silu(g) * u, BF)
 
 
+@pytest.mark.parametrize("H,Hk,d,rot,P_,with_cache", [(32, 8, 128, 128, 16, True), (5, 1, 64, 32, 8, True),
+                                                      (6, 2, 80, 0, 16, True), (4, 4, 256, 256, 32, False),
+                                                      (3, 3, 48, 48, 24, True)])
+def test_rotation_and_cache_write_16_bytes_a_lane_equals_the_plain_kernel(H, Hk, d, rot, P_, with_cache):
+    """`ops.rope_kv_write` on bfloat16 rows takes the kernel of the MFMA library; the plain kernel on the same input
+    gives the same rows and the same cache (the same float32 formula; a rounding may fall the other way where the
+    compiler fused a multiply and an add differently: few elements, one unit of bfloat16)."""
+    from allpaca_amd.kernels import lib, ops
+    T = 70
+    rng = np.random.default_rng(d + rot)
+    lens = [33, 20, 17]                                 # three segments: rows are their last positions
+    pos_list = [p for n, first in zip(lens, (40, 0, 100)) for p in range(first, first + n)]
+    seg_list = [s_ for s_, n in enumerate(lens) for _ in range(n)]
+    pos = torch.tensor(pos_list, dtype=torch.int32, device=DEV)
+    seg = torch.tensor(seg_list, dtype=torch.int32, device=DEV)
+    max_blocks = -(-140 // P_)
+    bt = torch.from_numpy(rng.permutation(3 * max_blocks).reshape(3, max_blocks).astype(np.int32)).to(DEV)
+    width = (H + 2 * Hk) * d + 8
+    qkv0 = gen(T, width, seed=1, dtype=BF).to(DEV)
+    ang = np.arange(140)[:, None] * (1.0 / 300.0 ** (np.arange(rot // 2) / max(rot // 2, 1)))[None, :]
+    table = torch.from_numpy(np.stack([np.cos(ang), np.sin(ang)], 1).astype(np.float32)).to(DEV) if rot else None
+    offs = (8, 8 + H * d, 8 + (H + Hk) * d)
+    results = []
+    for which in ("tuned", "plain"):
+        qkv = qkv0.clone()
+        cache = torch.zeros(3 * max_blocks, 2, Hk, P_, d, dtype=BF, device=DEV) if with_cache else None
+        if which == "tuned":
+            ops.rope_kv_write(qkv, *offs, H, Hk, d, rot, table, pos, seg, bt, cache, P_)
+        else:
+            lib.check(lib.load("plain").apc_rope_kv_write(
+                qkv.data_ptr(), 1, width, *offs, T, H, Hk, d, rot, table.data_ptr() if rot else 0, pos.data_ptr(),
+                seg.data_ptr(), bt.data_ptr(), max_blocks, cache.data_ptr() if with_cache else 0, 1, P_,
+                torch.cuda.current_stream().cuda_stream), "rope")
+        results.append((f64(qkv), f64(cache) if with_cache else np.zeros(1)))
+    for a, b in zip(results[0], results[1]):
+        diff = np.abs(a - b)
+        assert (diff <= 2.0 ** -7 * np.abs(b) + 1e-30).all() and (diff > 0).mean() < 0.005
+    assert np.array_equal(results[0][0][:, :8], f64(qkv0)[:, :8])              # columns beside the heads stay
+    if with_cache:
+        assert (results[0][1] != 0).any()
+
+
 def run_attention(H, Hk, d, P_, lens, rows_per_seg, window=0, seed=0):
     """Sequences of `lens` keys in the cache; the last `rows_per_seg[s]` positions of sequence s are the step's rows."""
     from allpaca_amd.engine.batch import Entry, pack_step
