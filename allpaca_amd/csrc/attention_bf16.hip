@@ -481,6 +481,7 @@ APC_EXPORT int apc_attention_prefill_bf16(const void* q, int ldq, int q_off, voi
   if (n_tiles <= 0) return 0;
   int e = check_common(q, ldq, q_off, cache, H, Hk, d, page_tokens);
   if (e) return e;
+  if (ldo % 4 || ((uintptr_t)out & 7u)) return APC_ERR_UNSUPPORTED;  // outputs are stored 8 bytes at a time
   if (max_blocks <= 0 || window < 0 || (long)n_tiles * H > 0x7fffffffL) return APC_ERR_BAD_ARG;
   dim3 grid(n_tiles * H), block(256);
 #define PF_LAUNCH(DP_)                                                                                             \
