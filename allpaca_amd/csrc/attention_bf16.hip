@@ -49,7 +49,10 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const bf16_t* __restrict__ cache, int P, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ positions, const int* __restrict__ row_seg, const int* __restrict__ tile_row0,
     const int* __restrict__ tile_rows, int n_tiles, int window, float scale) {
-  __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * (DP + KPAD)];
+  // elements of a row of K in LDS: a stride of 36 banks modulo 64 (as the rows of V and P have), so that the 16-byte
+  // operand reads of 16 consecutive rows and of neighbouring pieces fall into different banks
+  constexpr int KROW = DP + (DP % 128 == 0 ? 72 : DP % 128 == 64 ? 8 : DP % 128 == 32 ? 40 : 104);
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KROW];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[DP * (KT + KPAD)];
   __shared__ __attribute__((aligned(16))) bf16_t Ps[4 * 16 * (KT + KPAD)];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
@@ -81,7 +84,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 
   // K and V are zero where nothing is ever stored: the padding columns of K (a padded q column is zero as well,
   // but 0 * NaN is NaN) and the rows of V beyond d
-  for (int idx = tid; idx < KT * (DP + KPAD); idx += 256) Ks[idx] = 0;
+  for (int idx = tid; idx < KT * KROW; idx += 256) Ks[idx] = 0;
   for (int idx = tid; idx < DP * (KT + KPAD); idx += 256) Vs[idx] = 0;
 
   // this wave's 16 query rows as an MFMA operand (row = lane % 16, 8 elements of d per lane and step)
@@ -107,7 +110,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   for (int dt = 0; dt < DP / 16; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
   bf16_t* pw = Ps + wave * 16 * (KT + KPAD) + li * (KT + KPAD);  // this lane's row of P
-  const bf16_t* krd = Ks + li * (DP + KPAD) + lc * 8;            // this lane's place in a K operand
+  const bf16_t* krd = Ks + li * KROW + lc * 8;            // this lane's place in a K operand
   const bf16_t* vrd = Vs + li * (KT + KPAD) + lc * 8;            // ... and in a V operand
 
   // A tile of 64 keys and values goes global -> registers -> LDS; the loads of the next tile are issued before
@@ -129,7 +132,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const int key = k_on[j] ? idx / dchunks : 0, ch = k_on[j] ? idx % dchunks : 0;
     k_key[j] = key;
     k_base[j] = cache + (size_t)kvh * P * d + ch * 8;
-    k_dst[j] = Ks + key * (DP + KPAD) + ch * 8;
+    k_dst[j] = Ks + key * KROW + ch * 8;
     const int dv = idx / (KT / 8), kc = idx % (KT / 8);
     v_on[j] = dv < d;
     v_t[j] = kc * 8;
@@ -185,7 +188,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
       s[nt] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < DP / 32; ++ks) {
-        const Frag kf = *reinterpret_cast<const Frag*>(krd + nt * 16 * (DP + KPAD) + ks * 32);
+        const Frag kf = *reinterpret_cast<const Frag*>(krd + nt * 16 * KROW + ks * 32);
         s[nt] = mfma16(kf, qf[ks], s[nt]);
       }
     }
