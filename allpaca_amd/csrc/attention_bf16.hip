@@ -114,71 +114,60 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   const bf16_t* vrd = Vs + li * (KT + KPAD) + lc * 8;            // ... and in a V operand
 
   // A tile of 64 keys and values goes global -> registers -> LDS; the loads of the next tile are issued before
-  // the work on the current one and stored after it, and the pages of a tile are looked up one tile before its
-  // loads.  Pieces of 16 bytes: K along d, V along positions (8 of one element); DP/32 of each per thread, whose
-  // places are fixed for the whole loop.  No load is conditional: a key beyond the last one is read from the last
-  // (its scores are masked, its P is 0), a piece that lies in the padding of d is read from piece 0 and not stored.
-  constexpr int PIECES = DP / 32;
-  int k_key[PIECES], v_t[PIECES];
-  bool k_on[PIECES], v_on[PIECES];
-  const bf16_t* k_base[PIECES];
-  const bf16_t* v_base[PIECES];
-  bf16_t* k_dst[PIECES];
-  bf16_t* v_dst[PIECES];
+  // the work on the current one and stored after it.  The tile is 8 groups of 8 consecutive keys, and a group lies
+  // in one page (page sizes are multiples of 8): the 32 threads of group tid / 32 copy its keys (8 slots x d
+  // elements, one run of consecutive bytes in the page) and its values (d rows of 8 slots, 16 bytes each).  So a
+  // thread looks up one page per tile, one tile ahead, and its addresses are that page's base plus constants.
+  // No load is conditional: a group beyond the last key is read from the last key's group (scores are masked, P is
+  // 0 there), a piece beyond d from piece 0 (it is not stored).
+  constexpr int PIECES = DP / 32;  // 16-byte pieces of K and of V per thread and tile
+  const int grp = tid / 32, gl = tid % 32;
+  const int last_group = (last / 8) * 8;
+  int k_ldst[PIECES], v_ldst[PIECES];  // where this thread's pieces go in LDS (elements)
+  bool on[PIECES];                     // piece j exists: gl + 32 j < d
 #pragma unroll
   for (int j = 0; j < PIECES; ++j) {
-    const int idx = tid + j * 256;
-    k_on[j] = idx < KT * dchunks;
-    const int key = k_on[j] ? idx / dchunks : 0, ch = k_on[j] ? idx % dchunks : 0;
-    k_key[j] = key;
-    k_base[j] = cache + (size_t)kvh * P * d + ch * 8;
-    k_dst[j] = Ks + key * KROW + ch * 8;
-    const int dv = idx / (KT / 8), kc = idx % (KT / 8);
-    v_on[j] = dv < d;
-    v_t[j] = kc * 8;
-    v_base[j] = cache + (size_t)(Hk + kvh) * P * d + (size_t)(v_on[j] ? dv : 0) * P;
-    v_dst[j] = Vs + (v_on[j] ? dv : 0) * (KT + KPAD) + kc * 8;
+    const int idx = gl + 32 * j;       // K: piece idx of the group's 8 x d elements; V: element idx of the head
+    on[j] = idx < d;
+    const int key = on[j] ? idx / dchunks : 0, ch = on[j] ? idx % dchunks : 0;
+    k_ldst[j] = (grp * 8 + key) * KROW + ch * 8;
+    v_ldst[j] = (on[j] ? idx : 0) * (KT + KPAD) + grp * 8;
   }
-  const int p_shift = (P & (P - 1)) == 0 ? __builtin_ctz(P) : -1;
-  int k_page[PIECES], v_page[PIECES], k_slot[PIECES], v_slot[PIECES];
-  auto lookup_tile = [&](int t0) {
-#pragma unroll
-    for (int j = 0; j < PIECES; ++j) {
-      const int t = min(t0 + k_key[j], last), tv = min(t0 + v_t[j], (last / 8) * 8);
-      if (p_shift >= 0) {
-        k_page[j] = bt[t >> p_shift]; k_slot[j] = t & (P - 1);
-        v_page[j] = bt[tv >> p_shift]; v_slot[j] = tv & (P - 1);
-      } else {
-        k_page[j] = bt[t / P]; k_slot[j] = t % P;
-        v_page[j] = bt[tv / P]; v_slot[j] = tv % P;
-      }
-    }
-  };
+  const bf16_t* k_head = cache + (size_t)kvh * P * d;
+  const bf16_t* v_head = cache + (size_t)(Hk + kvh) * P * d;
+  int page_next = 0;  // page of this thread's group in the tile that is loaded next
+  auto lookup_tile = [&](int t0) { page_next = bt[min(t0 + grp * 8, last_group) / P]; };
   Frag kreg[PIECES], vreg[PIECES];
-  auto load_tile = [&]() {  // uses the pages found by the last lookup_tile
+  auto load_tile = [&](int t0) {  // uses the page found by the last lookup_tile, which was for this t0
+    const int tg = min(t0 + grp * 8, last_group), slot0 = tg % P;
+    const bf16_t* kp = k_head + (size_t)page_next * page_stride + (size_t)slot0 * d;
+    const bf16_t* vp = v_head + (size_t)page_next * page_stride + slot0;
 #pragma unroll
     for (int j = 0; j < PIECES; ++j) {
-      kreg[j] = load_frag(k_base[j] + (size_t)k_page[j] * page_stride + (size_t)k_slot[j] * d);
-      vreg[j] = load_frag(v_base[j] + (size_t)v_page[j] * page_stride + v_slot[j]);
+      const int idx = on[j] ? gl + 32 * j : 0;
+      kreg[j] = load_frag(kp + idx * 8);
+      vreg[j] = load_frag(vp + (size_t)idx * P);
     }
   };
   auto store_tile = [&]() {
 #pragma unroll
     for (int j = 0; j < PIECES; ++j) {
-      if (k_on[j]) *reinterpret_cast<Frag*>(k_dst[j]) = kreg[j];
-      if (v_on[j]) *reinterpret_cast<Frag*>(v_dst[j]) = vreg[j];
+      if (on[j]) {
+        *reinterpret_cast<Frag*>(Ks + k_ldst[j]) = kreg[j];
+        *reinterpret_cast<Frag*>(Vs + v_ldst[j]) = vreg[j];
+      }
     }
   };
 
   const int t_begin = (first / KT) * KT;
   lookup_tile(t_begin);
-  load_tile();
+  load_tile(t_begin);
   lookup_tile(t_begin + KT);
   __syncthreads();  // the zero fills are done
   store_tile();
   __syncthreads();
   for (int t0 = t_begin; t0 <= last; t0 += KT) {
-    load_tile();                 // tile t0 + 64 (beyond the last key: a harmless copy of the last)
+    load_tile(t0 + KT);          // beyond the last key: a harmless copy of the last group
     lookup_tile(t0 + 2 * KT);
 
     // S^T: lane holds keys t0 + nt*16 + lc*4 + r of row li

@@ -29,8 +29,12 @@ HEADERS = ["common.h", "mfma.h"]
 
 ARCH = "gfx950"
 # -packed-fp32-ops is switched off for device code: some packed forms have given wrong results on this hardware.
+# MFMA accumulators stay in ordinary vector registers (-amdgpu-mfma-vgpr-form): the attention kernels rescale their
+# accumulators with vector instructions every step, and from accumulation registers every value would have to be
+# moved there and back.
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", f"--offload-arch={ARCH}",
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result"]
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-mllvm", "-amdgpu-mfma-vgpr-form=1",
+         "-Wno-unused-result"]
 
 
 class KernelBuildError(RuntimeError):
