@@ -181,27 +181,26 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         s[nt] = mfma16(kf, qf[ks], s[nt]);
       }
     }
+    // The scale (positive) goes into the exponent: max over the bare scores, one multiply for the maximum, and
+    // 2^(s * sc2 - m) with one fused multiply-add a score.
     float mx = -INFINITY;
     if (t0 >= wave_lo && t0 + KT - 1 <= wave_hi) {  // every row of the wave sees the whole tile
 #pragma unroll
       for (int nt = 0; nt < KT / 16; ++nt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          s[nt][r] *= sc2;
-          mx = fmaxf(mx, s[nt][r]);
-        }
+        for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[nt][r]);
     } else {
 #pragma unroll
       for (int nt = 0; nt < KT / 16; ++nt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int t = t0 + nt * 16 + lc * 4 + r;
-          const float v = (t >= my_lo && t <= my_pos) ? s[nt][r] * sc2 : -INFINITY;
+          const float v = (t >= my_lo && t <= my_pos) ? s[nt][r] : -INFINITY;
           s[nt][r] = v;
           mx = fmaxf(mx, v);
         }
     }
-    mx = row4_max(mx);
+    mx = row4_max(mx) * sc2;
     const float m_new = fmaxf(m_run, mx);
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
     const float alpha = exp2_neg(m_run - m_safe);
@@ -210,7 +209,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     for (int nt = 0; nt < KT / 16; ++nt) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        s[nt][r] = exp2_neg(s[nt][r] - m_safe);
+        s[nt][r] = exp2_neg(fmaf(s[nt][r], sc2, -m_safe));
         sum += s[nt][r];
       }
       // P, row-major [row][key], 4 consecutive keys at once (read back below by this wave only)
@@ -221,10 +220,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     }
     l_run = l_run * alpha + row4_sum(sum);
     m_run = m_new;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {  // some row's maximum rose: O shrinks (else every factor is 1)
 #pragma unroll
-    for (int dt = 0; dt < DP / 16; ++dt)
+      for (int dt = 0; dt < DP / 16; ++dt)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+        for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+    }
     wave_lds_order();
     // O^T += V^T P^T
 #pragma unroll
@@ -475,6 +476,7 @@ APC_EXPORT int apc_attention_prefill_bf16(const void* q, int ldq, int q_off, voi
   if (e) return e;
   if (ldo % 4 || ((uintptr_t)out & 7u)) return APC_ERR_UNSUPPORTED;  // outputs are stored 8 bytes at a time
   if (max_blocks <= 0 || window < 0 || (long)n_tiles * H > 0x7fffffffL) return APC_ERR_BAD_ARG;
+  if (!(scale > 0.f)) return APC_ERR_UNSUPPORTED;  // the kernel takes the maximum before it scales
   dim3 grid(n_tiles * H), block(256);
 #define PF_LAUNCH(DP_)                                                                                             \
   hipLaunchKernelGGL((attn_prefill_kernel<DP_>), grid, block, 0, stream, (const bf16_t*)q, ldq, q_off, (bf16_t*)out, \

@@ -204,6 +204,8 @@ def attention_bf16(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int,
     _ops._gpu(q, out, cache, block_table)
     ldq, ldo = _ops._rows(q, "attention q"), _ops._rows(out, "attention out")
     T = q.shape[0]
+    if scale is not None and not scale > 0:
+        return False
     if (head_dim % 16 or head_dim > 256 or page_tokens % 8 or ldq % 8 or q_off % 8 or not _aligned(q, cache)
             or q.dtype != torch.bfloat16 or cache.dtype != torch.bfloat16 or out.dtype != torch.bfloat16):
         return False
