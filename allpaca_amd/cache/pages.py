@@ -103,6 +103,7 @@ class _Sequence:
     length: int = 0                    # positions committed
     reserved: int = 0                  # positions that pages exist for
     tables: List[List[int]] = field(default_factory=list)   # per paged group: page ids, FREED where a window passed
+    version: int = 0                   # changes whenever an entry of a table was taken away or replaced
 
 
 def group_needs(needs: Sequence[CacheNeed]) -> Tuple[List[Tuple[PagedKV, List[int]]], List[Tuple[FixedState, List[int]]]]:
@@ -137,6 +138,7 @@ class CacheManager:
         self.slots = SlotPool(max_requests)
         self.max_requests = max_requests
         self._seqs: Dict[Hashable, _Sequence] = {}
+        self._versions = 0
         # plan entry -> ("paged", group index, index inside the group) | ("state", ...) ; filled for owners only
         self.location: Dict[int, Tuple[str, int, int]] = {}
         for gi, g in enumerate(self.paged_groups):
@@ -158,7 +160,8 @@ class CacheManager:
         if seq in self._seqs:
             raise CacheError(f"request {seq!r} is already live")
         slot = self.slots.alloc()
-        self._seqs[seq] = _Sequence(slot, tables=[[] for _ in self.paged_groups])
+        self._versions += 1
+        self._seqs[seq] = _Sequence(slot, tables=[[] for _ in self.paged_groups], version=self._versions)
         return slot
 
     def slot_of(self, seq) -> int:
@@ -210,6 +213,8 @@ class CacheManager:
                 if t[i] != FREED:
                     g.pool.free(t[i])
                     t[i] = FREED
+                    self._versions += 1
+                    s.version = self._versions
 
     def truncate(self, seq, length: int) -> None:
         """Forgets positions >= length (pages wholly beyond go back).  Not possible below a window's edge."""
@@ -222,6 +227,8 @@ class CacheManager:
                 raise CacheError("truncate below pages that a window has already given back")
             while len(t) > keep:
                 p = t.pop()
+                self._versions += 1
+                s.version = self._versions
                 if p != FREED:
                     g.pool.free(p)
         s.length = length
@@ -237,6 +244,11 @@ class CacheManager:
 
     def block_table(self, seq, group: int) -> List[int]:
         return self._seqs[seq].tables[group]
+
+    def table_version(self, seq) -> int:
+        """A number that is the same as at an earlier call only if the request's block tables have only grown since
+        (no page taken away or replaced, and it is the same admission of the request)."""
+        return self._seqs[seq].version
 
     def free_pages(self, group: int = 0) -> int:
         return self.paged_groups[group].pool.free_count

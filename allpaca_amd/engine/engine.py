@@ -17,9 +17,16 @@ from ..sampling.params import FinishReason, GenerationOutput, GenerationParams, 
 from ..sampling.sampler import Sampler
 from .batch import Entry
 from .runner import ModelRunner
-from .scheduler import FINISHED, Request, Scheduler
+from .scheduler import FINISHED, RUNNING, Request, Scheduled, Scheduler
 
 _DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+class _PreparedStep:
+    """A decode step whose plan and batch description are ready; the tokens are still being sampled."""
+
+    def __init__(self, handle, scheduled):
+        self.handle, self.scheduled = handle, scheduled
 
 
 class Engine:
@@ -43,6 +50,7 @@ class Engine:
         self.scheduler = Scheduler(self.runner.cache, cfg.max_active_requests, cfg.max_batch_tokens, cfg.chunk_tokens)
         self.sampler = Sampler(self.runner.rt.device, cfg.seed)
         self.requests: Dict[int, Request] = {}
+        self._prepared: Optional[_PreparedStep] = None
         self._next_id = 0
         self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0}
 
@@ -76,6 +84,7 @@ class Engine:
     begin_request = add_request
 
     def abort(self, request_id: int) -> None:
+        self._prepared = None
         req = self.requests.pop(request_id, None)
         if req is not None and req.status != FINISHED:
             self.scheduler.abort(req)
@@ -86,29 +95,40 @@ class Engine:
     # ---- one tick ---------------------------------------------------------------
     def step(self) -> List[TokenEvent]:
         """One batch through the model: every decoding request advances by a token, prompts by a portion."""
-        plan = self.scheduler.plan()
-        self.stats["preemptions"] += len(plan.preempted)
-        for req in plan.admitted:
-            self.runner.storage.zero_slot(self.runner.cache.slot_of(req.id))
-        if not plan.scheduled:
-            return []
-        now = time.perf_counter()
-        entries = []
-        for s in plan.scheduled:
-            if s.request.t_first_scheduled is None:
-                s.request.t_first_scheduled = now
-            toks = s.request.tokens[s.start:s.start + s.count]
-            entries.append(Entry(s.request.id, toks, [s.count - 1] if s.samples else []))
-        logits = self.runner.step(entries)
-        sampled = [s for s in plan.scheduled if s.samples]
-        for s in plan.scheduled:
+        prepared, self._prepared = self._prepared, None
+        if prepared is not None and self.scheduler.waiting:
+            prepared = None     # a request arrived: the scheduler decides (what was reserved stays with its requests)
+        if prepared is not None:
+            # the step was planned and set up while the GPU worked on the one before: only the tokens were missing
+            scheduled = prepared.scheduled
+            logits = self.runner.run_prepared(prepared.handle, [s.request.tokens[s.start] for s in scheduled])
+        else:
+            plan = self.scheduler.plan()
+            self.stats["preemptions"] += len(plan.preempted)
+            for req in plan.admitted:
+                self.runner.storage.zero_slot(self.runner.cache.slot_of(req.id))
+            if not plan.scheduled:
+                return []
+            scheduled = plan.scheduled
+            now = time.perf_counter()
+            entries = []
+            for s in scheduled:
+                if s.request.t_first_scheduled is None:
+                    s.request.t_first_scheduled = now
+                toks = s.request.tokens[s.start:s.start + s.count]
+                entries.append(Entry(s.request.id, toks, [s.count - 1] if s.samples else []))
+            logits = self.runner.step(entries)
+        sampled = [s for s in scheduled if s.samples]
+        for s in scheduled:
             self.scheduler.advance(s)
             self.stats["decode_tokens" if s.request.output and s.count == 1 else "prefill_tokens"] += s.count
         self.stats["steps"] += 1
         events: List[TokenEvent] = []
         if sampled:
-            tokens = self.sampler.sample(logits, [s.request.params for s in sampled],
-                                         [len(s.request.output) for s in sampled])
+            pending = self.sampler.launch(logits, [s.request.params for s in sampled],
+                                          [len(s.request.output) for s in sampled])
+            self._prepared = self._prepare_next(scheduled)   # host work for the next step while the GPU runs this one
+            tokens = pending.wait()
             now = time.perf_counter()       # the token ids are on the host: the step is over
             for s, tok in zip(sampled, tokens):
                 s.request.t_tokens.append(now)
@@ -116,7 +136,25 @@ class Engine:
                 events.append(TokenEvent(s.request.id, int(tok), reason, len(s.request.prompt)))
                 if reason is not None:
                     self.scheduler.finish(s.request, reason)
+                    self._prepared = None   # the next step is not the one that was prepared
         return events
+
+    def _prepare_next(self, scheduled) -> Optional["_PreparedStep"]:
+        """If the next step is sure to be one more token for exactly the requests that run now (nothing waits, every
+        running request samples a token in this step and none reaches its `max_tokens` with it), its plan and the
+        runner's first half of it are made now.  A stop token or an abort cancels it."""
+        sch = self.scheduler
+        if sch.waiting or len(scheduled) != len(sch.running):
+            return None
+        for s in scheduled:
+            r = s.request
+            if not s.samples or r.status != RUNNING or len(r.output) + 1 >= r.params.max_tokens:
+                return None
+        order = sorted((s.request for s in scheduled), key=lambda r: r.order)   # as the scheduler orders decodes
+        handle = self.runner.prepare_decode([r.id for r in order])
+        if handle is None:
+            return None
+        return _PreparedStep(handle, [Scheduled(r, r.computed, 1, True) for r in order])
 
     poll = step
 

@@ -121,9 +121,15 @@ class ModelRunner:
         """A step in which every request brings one token and wants its logits: the launches of the whole
         model are replayed from a graph captured for (rows rounded up to a power of two, context rounded
         up to a power of two); only the batch description is copied in."""
-        n = len(entries)
+        seqs = [e.seq for e in entries]
+        g = self._graph_for(seqs)
+        g.fill(seqs)
+        return self._launch(g, [e.tokens[0] for e in entries])
+
+    def _graph_for(self, seqs: Sequence[Hashable]) -> "DecodeGraph":
+        n = len(seqs)
         rows = 1 << max(0, (n - 1).bit_length())
-        longest = max(self.cache.length(e.seq) for e in entries) + 1
+        longest = max(self.cache.length(s) for s in seqs) + 1
         span = max(256, 1 << (longest - 1).bit_length())
         span = min(span, -(-self.rt.max_positions // self.cache.page_tokens) * self.cache.page_tokens)
         span = max(span, longest)
@@ -131,10 +137,59 @@ class ModelRunner:
         g = self.graphs.get(key)
         if g is None:
             g = self.graphs[key] = DecodeGraph(self, rows, span)
-        g.fill(entries)
+        return g
+
+    def _launch(self, g: "DecodeGraph", tokens: Sequence[int]) -> torch.Tensor:
+        g.set_tokens(tokens)
+        g.upload()
         g.replay()
         self.graph_replays += 1
-        return g.logits[:n]
+        return g.logits[:len(tokens)]
+
+    # A decode-only step in two halves, so that the host can do the first half while the GPU still works on the step
+    # before and the tokens are not known yet.
+    def prepare_decode(self, seqs: Sequence[Hashable]) -> Optional["PreparedDecode"]:
+        """Everything of a step of one token per request that does not need the tokens: pages taken, the graph
+        chosen, positions and block tables written into its description.  None if this step cannot be prepared
+        (no graphs, no page free, a position beyond the run's limit): the caller then goes the ordinary way, which
+        says what is wrong.  What was reserved stays reserved for its request."""
+        if not self.use_graphs or not seqs:
+            return None
+        need = [0] * len(self.cache.paged_groups)
+        for s in seqs:
+            if s not in self.cache or self.cache.length(s) + 1 > self.rt.max_positions:
+                return None
+            for gi, k in enumerate(self.cache.pages_needed(s, 1)):
+                need[gi] += k
+        if any(k > self.cache.free_pages(gi) for gi, k in enumerate(need)):
+            return None
+        for s in seqs:
+            self.cache.reserve(s, 1)
+        g = self._graph_for(seqs)
+        g.fill(seqs)
+        return PreparedDecode(g, list(seqs))
+
+    def run_prepared(self, prepared: "PreparedDecode", tokens: Sequence[int]) -> torch.Tensor:
+        """The second half: the tokens go in, the step runs.  Nothing may have happened to the requests since
+        `prepare_decode`."""
+        if len(tokens) != len(prepared.seqs):
+            raise StepError("a prepared step needs one token for each of its requests")
+        for t in tokens:
+            if not (0 <= int(t) < self.vocab_size):
+                raise StepError(f"token {t} is outside the vocabulary of {self.vocab_size}")
+        logits = self._launch(prepared.graph, tokens)
+        for s in prepared.seqs:
+            self.cache.commit(s, 1)
+        self.steps += 1
+        return logits
+
+
+class PreparedDecode:
+    def __init__(self, graph: "DecodeGraph", seqs: List[Hashable]):
+        self.graph, self.seqs = graph, seqs
+
+
+HEAD_ENTRIES = 2   # plan entries in the first of a decode step's two graphs
 
 
 class DecodeGraph:
@@ -167,7 +222,15 @@ class DecodeGraph:
             max_context=span, max_rows=1, decode_only=True, decode_rows=None, n_decode_rows=rows,
             max_decode_context=span, n_tiles=0)
         self.copied = torch.cuda.Event()
+        # what the pinned block tables hold: the request of every row and how many of its pages (per group), so that
+        # a step writes only what is new (`CacheManager.table_version` changes when pages were taken away)
+        self.row_key: List[Optional[tuple]] = [None] * rows
+        self.row_pages = [[0] * rows for _ in self.widths]
+        self.rows_used = rows
+        for g, w in enumerate(self.widths):
+            self._part(8 + g)[:] = runner.pad_pages[g]
         self.fill([])
+        self.upload()
         views = runner.bind_views(self.info)
         # one eager run on a side stream (allocations settle), then the capture
         side = torch.cuda.Stream(device=dev)
@@ -176,15 +239,28 @@ class DecodeGraph:
             runner.model.forward(self.info, views)
         torch.cuda.current_stream(dev).wait_stream(side)
         torch.cuda.synchronize(dev)
-        self.graph = torch.cuda.CUDAGraph()
+        # Two graphs: a short head (the embedding and the first layers) and the rest.  Launching a graph costs the
+        # host time in proportion to its launches, and the GPU starts only when the launch call is through: with the
+        # head launched first, the long launch of the rest overlaps with the head's work on the GPU.
+        model = runner.model
+        n_plan = len(model.spec.plan)
+        cut = min(HEAD_ENTRIES, n_plan - 1) if n_plan > 1 else n_plan
+        self.graphs = [torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()] if cut < n_plan else [torch.cuda.CUDAGraph()]
         # No garbage collection while the stream is capturing: a collection may free device objects of engines that
         # are no longer used (other graphs, events), which is not allowed during a capture and ends the process.
         gc_was_on = gc.isenabled()
         gc.collect()
         gc.disable()
         try:
-            with torch.cuda.graph(self.graph):
-                self.logits = runner.model.forward(self.info, views)
+            with torch.cuda.graph(self.graphs[0]):
+                x = model.embed(self.info)
+                left = model.run_plan(x, self.info, views, 0, cut, None)
+                if len(self.graphs) == 1:
+                    self.logits = model.logits(x, self.info)
+            if len(self.graphs) == 2:
+                with torch.cuda.graph(self.graphs[1], pool=self.graphs[0].pool()):
+                    model.run_plan(x, self.info, views, cut, n_plan, left)
+                    self.logits = model.logits(x, self.info)
         finally:
             if gc_was_on:
                 gc.enable()
@@ -193,34 +269,54 @@ class DecodeGraph:
     def _part(self, i: int) -> np.ndarray:
         return self.np[self.cuts[i]: self.cuts[i + 1]]
 
-    def fill(self, entries: Sequence[Entry]) -> None:
+    def fill(self, seqs: Sequence[Hashable]) -> None:
+        """Positions, state slots and block tables of the requests `seqs`, one row each (tokens: `set_tokens`)."""
         r = self.runner
         cache = r.cache
-        n = len(entries)
+        n = len(seqs)
         self.copied.synchronize()      # the last upload has read the pinned buffer
         tokens, positions, pos0, slots = self._part(0), self._part(1), self._part(5), self._part(6)
         tokens[n:] = 0
         positions[n:] = 0
         pos0[n:] = 0
         slots[n:] = cache.max_requests
-        for i, e in enumerate(entries):
-            tokens[i] = e.tokens[0]
-            positions[i] = pos0[i] = cache.length(e.seq)
-            slots[i] = cache.slot_of(e.seq)
+        for i, seq in enumerate(seqs):
+            positions[i] = pos0[i] = cache.length(seq)
+            slots[i] = cache.slot_of(seq)
+        keys = [(seq, cache.table_version(seq)) for seq in seqs]
+        used = max(n, self.rows_used)
         for g, w in enumerate(self.widths):
             bt = self._part(8 + g).reshape(self.rows, w)
             pad = r.pad_pages[g]
-            bt[n:] = pad
-            for i, e in enumerate(entries):
-                t = cache.block_table(e.seq, g)
+            windowed = cache.paged_groups[g].need.window is not None
+            if used > n:
+                bt[n:used] = pad           # rows that held a request last time and hold none now
+            held = self.row_pages[g]
+            for i, seq in enumerate(seqs):
+                t = cache.block_table(seq, g)
                 k = len(t)
                 row = bt[i]
-                row[:k] = t
-                row[k:] = pad
-                if cache.paged_groups[g].need.window is not None:
-                    row[:k][row[:k] < 0] = pad
+                if not windowed and self.row_key[i] == keys[i] and held[i] <= k:
+                    if k > held[i]:        # the same request with the same pages as last time: only the new ones
+                        row[held[i]:k] = t[held[i]:]
+                else:
+                    row[:k] = t
+                    row[k:] = pad
+                    if windowed:
+                        row[:k][row[:k] < 0] = pad
+                held[i] = k
+        self.row_key[:n] = keys
+        for i in range(n, used):
+            self.row_key[i] = None
+        self.rows_used = n
+
+    def set_tokens(self, tokens: Sequence[int]) -> None:
+        self._part(0)[:len(tokens)] = tokens
+
+    def upload(self) -> None:
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
 
     def replay(self) -> None:
-        self.graph.replay()
+        for g in self.graphs:
+            g.replay()

@@ -67,18 +67,31 @@ class DecoderModel:
     def forward(self, step, caches) -> Optional[torch.Tensor]:
         """`step`: the batch on the device (tokens, positions, segments); `caches[i]`: the
         cache view of plan entry i.  Returns float32 logits [wanted rows, vocab], or None."""
-        rt = self.rt
-        T = step.n_rows
-        x = torch.empty((T, self.spec.hidden_size), dtype=torch.float32, device=rt.device)
+        x = self.embed(step)
+        self.run_plan(x, step, caches, 0, len(self.spec.plan), None)
+        return self.logits(x, step)
+
+    # The same in three pieces, for callers that record the step's launches in more than one graph.
+    def embed(self, step) -> torch.Tensor:
+        """The float32 residual stream [rows, hidden] of the step's tokens."""
+        x = torch.empty((step.n_rows, self.spec.hidden_size), dtype=torch.float32, device=self.rt.device)
         self.embedding.forward(step.tokens, x)
+        return x
+
+    def run_plan(self, x: torch.Tensor, step, caches, lo: int, hi: int, left):
+        """Plan entries lo .. hi-1 on the stream x.  `left`: what entry lo-1 left for entry lo's first norm (or
+        None); returns what entry hi-1 left for entry hi's."""
         plan = self.spec.plan
-        left = None  # what a layer's last product left for the next layer's first norm
-        for i, e in enumerate(plan):
+        for i in range(lo, hi):
             nxt = self.blocks[plan[i + 1].block].first_norm() if i + 1 < len(plan) else None
-            left = self.blocks[e.block].run(x, step, caches[i], pre=left, next_norm=nxt)
+            left = self.blocks[plan[i].block].run(x, step, caches[i], pre=left, next_norm=nxt)
+        return left
+
+    def logits(self, x: torch.Tensor, step) -> Optional[torch.Tensor]:
         R = step.n_logit_rows
         if R == 0:
             return None
+        rt = self.rt
         h = torch.empty((R, self.spec.hidden_size), dtype=rt.dtype, device=rt.device)
         self.final_norm.forward(x, h, rows=step.logit_rows)
         logits = torch.empty((R, self.spec.vocab_size), dtype=torch.float32, device=rt.device)

@@ -37,23 +37,45 @@ class Sampler:
     def __init__(self, device: torch.device, default_seed: int):
         self.device = device
         self.default_seed = default_seed
+        self._pinned = None   # token ids come back through pinned memory (one copy in flight at a time)
 
     def sample(self, logits: torch.Tensor, params: Sequence[GenerationParams], indices: Sequence[int]) -> List[int]:
         """logits: float32 [R, V] on the GPU; params[r] and indices[r] (how many tokens row r's request
         has generated so far) choose the rule and the random number of row r."""
+        return self.launch(logits, params, indices).wait()
+
+    def launch(self, logits: torch.Tensor, params: Sequence[GenerationParams], indices: Sequence[int]) -> "Pending":
+        """The same without waiting: the kernels and the copy of the token ids to the host are queued; `wait()` of
+        the result gives the ids.  The caller may do other work on the host in between."""
         R = logits.shape[0]
         out = torch.empty(R, dtype=torch.int32, device=self.device)
         if all(p.greedy for p in params):
             ops.argmax_rows(logits, out)
-            return out.cpu().tolist()
-        host = np.empty((4, R), dtype=np.float32)
-        ks = np.empty(R, dtype=np.int32)
-        for r, (p, i) in enumerate(zip(params, indices)):
-            host[0, r] = p.temperature
-            host[1, r] = p.top_p
-            host[2, r] = uniform_for(self.default_seed if p.seed is None else p.seed, i)
-            ks[r] = p.top_k
-        f = torch.from_numpy(host).to(self.device)
-        k = torch.from_numpy(ks).to(self.device)
-        ops.sample_rows(logits, f[0], k, f[1], f[2], out)
-        return out.cpu().tolist()
+        else:
+            host = np.empty((4, R), dtype=np.float32)
+            ks = np.empty(R, dtype=np.int32)
+            for r, (p, i) in enumerate(zip(params, indices)):
+                host[0, r] = p.temperature
+                host[1, r] = p.top_p
+                host[2, r] = uniform_for(self.default_seed if p.seed is None else p.seed, i)
+                ks[r] = p.top_k
+            f = torch.from_numpy(host).to(self.device)
+            k = torch.from_numpy(ks).to(self.device)
+            ops.sample_rows(logits, f[0], k, f[1], f[2], out)
+        if self._pinned is None or self._pinned.numel() < R:
+            self._pinned = torch.empty(max(R, 64), dtype=torch.int32).pin_memory()
+        self._pinned[:R].copy_(out, non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+        return Pending(self._pinned, R, done)
+
+
+class Pending:
+    """Token ids on their way to the host."""
+
+    def __init__(self, pinned: torch.Tensor, n: int, done: torch.cuda.Event):
+        self.pinned, self.n, self.done = pinned, n, done
+
+    def wait(self) -> List[int]:
+        self.done.synchronize()
+        return self.pinned[:self.n].tolist()

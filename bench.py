@@ -62,7 +62,7 @@ def build_engine(cfg_json, dtype, batch, context, extra_tokens, layers, seed=0, 
     eng.runner = ModelRunner(model, ec.page_tokens, ec.num_pages, ec.max_active_requests, use_graphs=use_graphs)
     eng.scheduler = Scheduler(eng.runner.cache, ec.max_active_requests, ec.max_batch_tokens, ec.chunk_tokens)
     eng.sampler = Sampler(rt.device, ec.seed)
-    eng.requests, eng._next_id = {}, 0
+    eng.requests, eng._next_id, eng._prepared = {}, 0, None
     eng.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0}
     return cfg, eng
 

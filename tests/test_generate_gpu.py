@@ -257,3 +257,42 @@ def test_generation_with_graphs_equals_the_plain_implementation():
     outs = eng.generate(prompts, params(max_tokens=16, temperature=0.0))
     assert [o.token_ids for o in outs] == want
     assert eng.runner.graph_replays > 0
+
+
+def test_steps_prepared_ahead_give_the_same_tokens_when_requests_stop_arrive_and_are_aborted():
+    """With graphs on, the engine sets up the next decode step while the GPU works on the current one.  A stop token,
+    a request that arrives between two steps and an abort each cancel what was set up; the tokens are those of the
+    plain implementation all the same."""
+    folder = H.model_folder("A", "float32", True)
+    cfg, w = H.oracle(folder)
+    prompts = [H.random_tokens(256, n, seed=40 + n) for n in (5, 9, 3, 12)]
+    full = [P.greedy_generate(cfg, w, p, 24) for p in prompts]
+    eng = engine_for(folder, use_graphs=True)
+    # request 0 stops at the token it would produce 10th, request 1 runs to its length
+    stop = full[0][9]
+    cut0 = full[0][: full[0].index(stop) + 1]
+    r0 = eng.add_request(prompts[0], params(max_tokens=24, temperature=0.0, stop_token_ids=[stop]))
+    r1 = eng.add_request(prompts[1], params(max_tokens=24, temperature=0.0))
+    got = {r0: [], r1: []}
+    used_prepared = 0
+    steps = 0
+    r2 = r3 = None
+    while eng.has_unfinished():
+        used_prepared += eng._prepared is not None
+        for ev in eng.step():
+            got.setdefault(ev.request_id, []).append(ev.token_id)
+        steps += 1
+        if steps == 6:                                   # arrives while a prepared step exists
+            assert eng._prepared is not None
+            r2 = eng.add_request(prompts[2], params(max_tokens=24, temperature=0.0))
+            got[r2] = []
+        if steps == 12:
+            r3 = eng.add_request(prompts[3], params(max_tokens=24, temperature=0.0))
+            got[r3] = []
+        if steps == 16:
+            eng.abort(r3)                                # leaves mid-way
+    assert used_prepared > 10
+    assert got[r0] == cut0 and got[r1] == full[1] and got[r2] == full[2]
+    assert got[r3] == full[3][: len(got[r3])] and 0 < len(got[r3]) < 24
+    assert eng.runner.cache.free_pages(0) == eng.runner.cache.paged_groups[0].pool.num_pages
+    eng.runner.cache.check()
