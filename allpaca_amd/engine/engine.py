@@ -101,7 +101,7 @@ class Engine:
         if prepared is not None:
             # the step was planned and set up while the GPU worked on the one before: only the tokens were missing
             scheduled = prepared.scheduled
-            logits = self.runner.run_prepared(prepared.handle, [s.request.tokens[s.start] for s in scheduled])
+            logits = self.runner.run_prepared(prepared.handle, [s.request.token_slice(s.start, 1)[0] for s in scheduled])
         else:
             plan = self.scheduler.plan()
             self.stats["preemptions"] += len(plan.preempted)
@@ -115,7 +115,7 @@ class Engine:
             for s in scheduled:
                 if s.request.t_first_scheduled is None:
                     s.request.t_first_scheduled = now
-                toks = s.request.tokens[s.start:s.start + s.count]
+                toks = s.request.token_slice(s.start, s.count)
                 entries.append(Entry(s.request.id, toks, [s.count - 1] if s.samples else []))
             logits = self.runner.step(entries)
         sampled = [s for s in scheduled if s.samples]

@@ -68,6 +68,15 @@ class Request:
     def n_tokens(self) -> int:
         return len(self.prompt) + len(self.output)
 
+    def token_slice(self, start: int, count: int) -> List[int]:
+        """tokens[start : start + count] without building the whole list (a step asks for this every time)."""
+        n = len(self.prompt)
+        if start >= n:
+            return self.output[start - n:start - n + count]
+        if start + count <= n:
+            return self.prompt[start:start + count]
+        return self.prompt[start:] + self.output[:start + count - n]
+
     @property
     def left(self) -> int:
         """Tokens that must still run before the next token can be sampled."""
