@@ -88,6 +88,35 @@ def test_truncate():
     cm.check()
 
 
+def test_table_version_stays_while_tables_only_grow():
+    """Who keeps a copy of a block table may add the new pages only, as long as the version is the same."""
+    cm = CacheManager([FULL, WIN], page_tokens=4, num_pages=[8, 8], max_requests=2)
+    cm.admit("a")
+    v0 = cm.table_version("a")
+    cm.reserve("a", 6)
+    cm.commit("a", 6)
+    assert cm.table_version("a") == v0                  # grown, nothing taken away (the window of 10 is not passed)
+    cm.reserve("a", 9)
+    cm.commit("a", 9)                                   # position 15: keys 6.. are needed, page 0 is passed
+    v1 = cm.table_version("a")
+    assert v1 != v0 and cm.block_table("a", 1)[0] == FREED
+    cm.truncate("a", 14)                                # nothing popped: still 4 pages
+    assert cm.table_version("a") == v1
+    cm.admit("b")
+    assert cm.table_version("b") not in (v0, v1)
+    cm.release("a")
+    cm.admit("a")                                       # the same name, another admission
+    assert cm.table_version("a") not in (v0, v1, cm.table_version("b"))
+    cm.release("a")
+    cm2 = CacheManager([FULL], page_tokens=4, num_pages=6, max_requests=1)
+    cm2.admit("a")
+    cm2.reserve("a", 14)
+    cm2.commit("a", 14)
+    v = cm2.table_version("a")
+    cm2.truncate("a", 5)                                # two pages popped
+    assert cm2.table_version("a") != v
+
+
 @pytest.mark.parametrize("seed", range(8))
 def test_random_orders_lose_no_page(seed):
     """Admissions, steps of random sizes, releases and truncations in random order: after every operation
