@@ -12,7 +12,8 @@
 //  * the loads of the next step are in flight while the current one is multiplied (two register sets that
 //    swap roles; no branch around a load in the steady state);
 //  * the waves' partial sums are added in wave order through LDS, then the epilogue runs: store (bfloat16 or
-//    float32), add into a float32 residual, or SwiGLU of a gate band and an up band.
+//    float32), add into a float32 residual, SwiGLU of a gate band and an up band, or rotation of q and k and the
+//    write of k and v into the paged cache (SK_QKV_ROPE, see SkRope).
 //  * the RMS norm between a product that adds into the residual x and the product that reads the normalised row
 //    is folded into the two (EMIT and PRE): the first writes, beside x, the row bfloat16(x[m,n] * g[n]) (g: the
 //    norm's weight) and, per band of 16 columns, the sum of x^2 of each row; the second multiplies with that row
@@ -28,7 +29,7 @@
 constexpr int SK_U = 4;              // tiles (32 k each) per band per step
 constexpr int TILE_ELEMS = 16 * 32;  // elements of a tile
 
-enum { SK_STORE_BF16 = 0, SK_STORE_F32 = 1, SK_ACC_F32 = 2, SK_SWIGLU = 3 };
+enum { SK_STORE_BF16 = 0, SK_STORE_F32 = 1, SK_ACC_F32 = 2, SK_SWIGLU = 3, SK_QKV_ROPE = 4 };
 
 template <int MT, int NB>
 struct SkRegs {
@@ -52,12 +53,29 @@ struct SkNorm {
   int ld_raw;
 };
 
+// SK_QKV_ROPE: the product that gives q, k and v of a row also turns q and k by the row's position and writes k
+// and v into the paged cache, so no kernel of its own does that.  W is [(H + 2 Hk) d, K], heads in the order q, k, v;
+// the whole head is rotated (pairs (e, e + d/2)); d is a multiple of 32.  A block takes the bands j and j + d/32 of
+// one head, so a lane of the finishing wave holds both elements of 4 pairs.  Rotated q goes to C; k to
+// cache[page][0][kv head][slot][:], v to cache[page][1][kv head][:][slot], page = block_table[row_seg][pos / P],
+// slot = pos % P.  The sums are rounded to bfloat16 before the rotation, as a product that stores them would.
+struct SkRope {
+  const float* cos_sin;    // [positions][2][d / 2]
+  const int* positions;    // [M]
+  const int* row_seg;      // [M]
+  const int* block_table;  // [segments][max_blocks]
+  int max_blocks;
+  bf16_t* cache;
+  int P, H, Hk, d;
+};
+
 template <int MT, int MODE, int NB, int WPB, bool PRE, bool EMIT>
 __global__ __launch_bounds__(WPB * 64) void skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda,
                                                                const bf16_t* __restrict__ W,
                                                                const bf16_t* __restrict__ W2, int chunks,
                                                                void* __restrict__ C, int ldc, int M, int N, int K,
-                                                               SkNorm norm, int vec_c) {
+                                                               SkNorm norm, int vec_c, SkRope rope) {
+  static_assert(MODE != SK_QKV_ROPE || NB == 2, "the two bands of a block hold the two halves of the pairs");
   static_assert(!EMIT || MODE == SK_ACC_F32, "only a product that adds into the residual emits the next norm's row");
   static_assert(!PRE || MODE != SK_ACC_F32, "a product that reads a normalised row stores its result");
   static_assert(MT == 1, "written for one tile of rows (the finishing wave's early loads, the folded norm)");
@@ -65,15 +83,29 @@ __global__ __launch_bounds__(WPB * 64) void skinny_gemm_kernel(const bf16_t* __r
   __shared__ float row_ss[WPB * MT * 16];
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const int i = lane % 16, c = lane / 16;
-  constexpr int OUT_BANDS = MODE == SK_SWIGLU ? 1 : NB;
+  constexpr int OUT_BANDS = (MODE == SK_SWIGLU || MODE == SK_QKV_ROPE) ? 1 : NB;
   const int band0 = blockIdx.x * OUT_BANDS;
   const int bands = (N + 15) / 16;
+  // SK_QKV_ROPE: head and first element of this lane's 4 pairs; position and segment of the finishing wave's row
+  // are asked for before the stream starts, what depends on them behind its first loads
+  int qkv_head = 0, qkv_e = 0, qkv_pos = 0, qkv_seg = 0;
+  if constexpr (MODE == SK_QKV_ROPE) {
+    const int hb = rope.d / 32;
+    qkv_head = blockIdx.x / hb;
+    qkv_e = (blockIdx.x % hb) * 16 + c * 4;
+    if (wave == 0 && i < M) {
+      qkv_pos = rope.positions[i];
+      qkv_seg = rope.row_seg[i];
+    }
+  }
 
   // band pointers (bands beyond the matrix are clamped to the last: what they compute is never stored)
   const bf16_t* wb[NB];
 #pragma unroll
   for (int b = 0; b < NB; ++b) {
     if (MODE == SK_SWIGLU) wb[b] = (b == 0 ? W : W2) + (size_t)band0 * chunks * TILE_ELEMS + lane * 8;
+    else if (MODE == SK_QKV_ROPE)
+      wb[b] = W + (size_t)(qkv_head * (rope.d / 16) + blockIdx.x % (rope.d / 32) + b * (rope.d / 32)) * chunks * TILE_ELEMS + lane * 8;
     else wb[b] = W + (size_t)min(band0 + b, bands - 1) * chunks * TILE_ELEMS + lane * 8;
   }
   const bf16_t* arow[MT];
@@ -143,6 +175,18 @@ __global__ __launch_bounds__(WPB * 64) void skinny_gemm_kernel(const bf16_t* __r
     c_old = *reinterpret_cast<const floatx4*>((const float*)C + (size_t)i * ldc + fin_n);
     if constexpr (EMIT) g_next = *reinterpret_cast<const floatx4*>(norm.g + fin_n);
   }
+  floatx4 cosv = floatx4{0.f, 0.f, 0.f, 0.f}, sinv = floatx4{0.f, 0.f, 0.f, 0.f};
+  int qkv_page = 0;
+  if constexpr (MODE == SK_QKV_ROPE) {
+    if (wave == 0 && i < M) {
+      if (qkv_head < rope.H + rope.Hk) {
+        const float* cs = rope.cos_sin + (size_t)qkv_pos * rope.d;
+        cosv = *reinterpret_cast<const floatx4*>(cs + qkv_e);
+        sinv = *reinterpret_cast<const floatx4*>(cs + rope.d / 2 + qkv_e);
+      }
+      if (qkv_head >= rope.H) qkv_page = rope.block_table[(size_t)qkv_seg * rope.max_blocks + qkv_pos / rope.P];
+    }
+  }
   if (nsteps > 0) {
     int at = c_lo, done = 0;
     while (done + 3 < nsteps) {  // steps done, done+1 are loaded; done+2, done+3 exist
@@ -184,13 +228,13 @@ __global__ __launch_bounds__(WPB * 64) void skinny_gemm_kernel(const bf16_t* __r
     for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<floatx4*>(&mine[((b * MT + mt) * 64 + lane) * 4]) = acc[b][mt];
   __syncthreads();
 
-  constexpr int NSUM = MODE == SK_SWIGLU ? 2 : 1;
+  constexpr int NSUM = (MODE == SK_SWIGLU || MODE == SK_QKV_ROPE) ? 2 : 1;
   if (wave < ITEMS) {
     const int b = wave;
     floatx4 sum[NSUM];
 #pragma unroll
     for (int s = 0; s < NSUM; ++s) {
-      const int bb = MODE == SK_SWIGLU ? s : b;
+      const int bb = NSUM == 2 ? s : b;
       sum[s] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int w = 0; w < WPB; ++w)
@@ -204,6 +248,45 @@ __global__ __launch_bounds__(WPB * 64) void skinny_gemm_kernel(const bf16_t* __r
       const float rstd = 1.0f / sqrtf(total / (float)K + norm.eps);
 #pragma unroll
       for (int s2 = 0; s2 < NSUM; ++s2) sum[s2] *= rstd;
+    }
+    if constexpr (MODE == SK_QKV_ROPE) {
+      if (m < M) {
+        float lo[4], hi[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          lo[r] = bf16_to_float(float_to_bf16(sum[0][r]));
+          hi[r] = bf16_to_float(float_to_bf16(sum[1][r]));
+        }
+        const int half = rope.d / 2, slot = qkv_pos % rope.P;
+        bf16_t* page = rope.cache + (size_t)qkv_page * ((size_t)2 * rope.Hk * rope.P * rope.d);
+        if (qkv_head < rope.H + rope.Hk) {
+          float ya[4], yb[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float av = lo[r], bv = hi[r], cc = cosv[r], sn = sinv[r];
+            ya[r] = av * cc - bv * sn;
+            yb[r] = av * sn + bv * cc;
+          }
+          bf16_t* dst = qkv_head < rope.H ? (bf16_t*)C + (size_t)m * ldc + (size_t)qkv_head * rope.d
+                                          : page + ((size_t)(qkv_head - rope.H) * rope.P + slot) * rope.d;
+          uint2 pa, pb;
+          pa.x = pack_bf16x2(ya[0], ya[1]);
+          pa.y = pack_bf16x2(ya[2], ya[3]);
+          pb.x = pack_bf16x2(yb[0], yb[1]);
+          pb.y = pack_bf16x2(yb[2], yb[3]);
+          *reinterpret_cast<uint2*>(dst + qkv_e) = pa;
+          *reinterpret_cast<uint2*>(dst + qkv_e + half) = pb;
+        } else {
+          bf16_t* col = page + (size_t)rope.Hk * rope.P * rope.d +
+                        ((size_t)(qkv_head - rope.H - rope.Hk) * rope.d + qkv_e) * rope.P + slot;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            col[(size_t)r * rope.P] = float_to_bf16(sum[0][r]);
+            col[(size_t)(half + r) * rope.P] = float_to_bf16(sum[1][r]);
+          }
+        }
+      }
+      return;
     }
     float sq = 0.f;  // EMIT: x^2 over this lane's columns
     if (fin_vec) {
@@ -273,10 +356,11 @@ static bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 template <int MODE, bool PRE, bool EMIT>
 static int launch_skinny(const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M, int N,
-                         int K, SkNorm norm, hipStream_t stream) {
+                         int K, SkNorm norm, hipStream_t stream, SkRope rope = SkRope{}) {
   int nb, wpb;
-  pick_shape(N, K, MODE == SK_SWIGLU, &nb, &wpb);
+  pick_shape(MODE == SK_QKV_ROPE ? N / 2 : N, K, MODE == SK_SWIGLU || MODE == SK_QKV_ROPE, &nb, &wpb);
   const int chunks = ceil_div(K, 32), bands = ceil_div(N, 16);
+  if ((MODE == SK_SWIGLU || MODE == SK_QKV_ROPE) && wpb > 8) wpb = 8;
   if (PRE && norm.ld_ss > 4 * 4 * wpb * SS_LOADS) return APC_ERR_UNSUPPORTED;
   // whole 16-byte (float32) or 8-byte (bfloat16) accesses to C and to the emitted row where everything is aligned
   const int elem = (MODE == SK_STORE_BF16 || MODE == SK_SWIGLU) ? 2 : 4;
@@ -285,11 +369,12 @@ static int launch_skinny(const bf16_t* A, int lda, const bf16_t* W, const bf16_t
 #define SK_LAUNCH(NB_, WPB_)                                                                                  \
   hipLaunchKernelGGL((skinny_gemm_kernel<1, MODE, NB_, WPB_, PRE, EMIT>),                                     \
                      dim3(ceil_div(bands, MODE == SK_SWIGLU ? 1 : NB_)), dim3(WPB_ * WAVE), 0, stream, A, lda, W, \
-                     W2, chunks, C, ldc, M, N, K, norm, vec_c)
-  if constexpr (MODE == SK_SWIGLU) {
+                     W2, chunks, C, ldc, M, N, K, norm, vec_c, rope)
+  if constexpr (MODE == SK_SWIGLU || MODE == SK_QKV_ROPE) {
+    // two bands a wave: with 16 waves a block the two register sets of loads would not fit the 128 registers a
+    // wave has then
     if (wpb == 4) SK_LAUNCH(2, 4);
-    else if (wpb == 8) SK_LAUNCH(2, 8);
-    else SK_LAUNCH(2, 16);
+    else SK_LAUNCH(2, 8);
   } else if (nb == 2) {
     if (wpb == 4) SK_LAUNCH(2, 4);
     else SK_LAUNCH(2, 8);
@@ -372,4 +457,30 @@ APC_EXPORT int apc_skinny_swiglu_pre_bf16(const void* A, int lda, const float* s
   const SkNorm norm{const_cast<float*>(ss), n_ss, ceil_div(n_ss, 4) * 4, eps, nullptr, nullptr, 0};
   return launch_skinny<SK_SWIGLU, true, false>((const bf16_t*)A, lda, (const bf16_t*)Wg, (const bf16_t*)Wu, C, ldc, M, F,
                                                K, norm, stream);
+}
+
+// q, k, v of M <= 16 rows in one product, q and k rotated, k and v written into the paged cache (see SkRope).
+// W: tiled layout of [(H + 2 Hk) d, K]; q_out [M, ldq] takes the rotated q heads in its first H d columns.  With ss:
+// A is a row that apc_skinny_gemm_emit_bf16 left and the sums are scaled as in apc_skinny_gemm_pre_bf16.
+APC_EXPORT int apc_skinny_qkv_rope_bf16(const void* A, int lda, const float* ss, int n_ss, float eps, const void* W,
+                                        void* q_out, int ldq, int M, int K, int H, int Hk, int d,
+                                        const float* cos_sin, const int* positions, const int* row_seg,
+                                        const int* block_table, int max_blocks, void* cache, int page_tokens,
+                                        hipStream_t stream) {
+  if (M <= 0) return 0;
+  if (H <= 0 || Hk <= 0 || d <= 0 || K <= 0 || lda < K || ldq < H * d || !cos_sin || !positions || !row_seg ||
+      !block_table || max_blocks <= 0 || !cache || page_tokens <= 0 || (ss && n_ss <= 0))
+    return APC_ERR_BAD_ARG;
+  if (!operands_ok(A, lda, W, M, K) || d % 32 || ldq % 4 || ((uintptr_t)q_out & 7u) || !aligned16(cos_sin) ||
+      ((uintptr_t)cache & 7u) || (ss && !aligned16(ss)))
+    return APC_ERR_UNSUPPORTED;
+  const SkRope rope{cos_sin, positions, row_seg, block_table, max_blocks, (bf16_t*)cache, page_tokens, H, Hk, d};
+  const int N = (H + 2 * Hk) * d;
+  if (ss) {
+    const SkNorm norm{const_cast<float*>(ss), n_ss, ceil_div(n_ss, 4) * 4, eps, nullptr, nullptr, 0};
+    return launch_skinny<SK_QKV_ROPE, true, false>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, q_out, ldq, M, N, K,
+                                                   norm, stream, rope);
+  }
+  return launch_skinny<SK_QKV_ROPE, false, false>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, q_out, ldq, M, N, K,
+                                                  SkNorm{}, stream, rope);
 }

@@ -296,6 +296,19 @@ def linear_pre(raw: torch.Tensor, ss: torch.Tensor, eps: float, w, out: torch.Te
     return False
 
 
+def qkv_rope_write(a: torch.Tensor, pre, w, q_out: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
+                   cos_sin: torch.Tensor, positions: torch.Tensor, row_seg: torch.Tensor, block_table: torch.Tensor,
+                   cache: torch.Tensor, page_tokens: int) -> bool:
+    """The product for q, k and v, the rotation of whole q and k heads and the write of k and v into the pages in
+    one kernel (few rows; `pre` = (ss, eps) if `a` is a row that `linear(..., emit=...)` left, else None).  False if
+    there is no such kernel for these sizes (nothing is done then)."""
+    if isinstance(w, PackedWeight) and not FORCE_PLAIN:
+        from . import tuned
+        return tuned.qkv_rope_bf16(a, pre, w, q_out, n_heads, n_kv_heads, head_dim, cos_sin, positions, row_seg,
+                                   block_table, cache, page_tokens)
+    return False
+
+
 def swiglu_pre(raw: torch.Tensor, ss: torch.Tensor, eps: float, w_gate_up, out: torch.Tensor) -> bool:
     if isinstance(w_gate_up, tuple) and not FORCE_PLAIN:
         from . import tuned

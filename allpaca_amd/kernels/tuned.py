@@ -163,6 +163,42 @@ def gemm_pre_bf16(raw: torch.Tensor, ss: torch.Tensor, eps: float, w: PackedWeig
     return True
 
 
+def qkv_rope_bf16(a: torch.Tensor, pre, w: PackedWeight, q_out: torch.Tensor, n_heads: int, n_kv_heads: int,
+                  head_dim: int, cos_sin: torch.Tensor, positions: torch.Tensor, row_seg: torch.Tensor,
+                  block_table: torch.Tensor, cache: torch.Tensor, page_tokens: int) -> bool:
+    """q, k, v of up to 16 rows in one product that also rotates q and k (whole heads) and writes k and v into the
+    pages; rotated q goes to the first n_heads * head_dim columns of q_out.  `a`: the normalised rows, or with
+    `pre` = (ss, eps) the row that `gemm_emit_bf16` left.  False, with nothing done, for sizes the kernel does not
+    take."""
+    _ops._gpu(a, w.data, q_out, cos_sin, positions, row_seg, block_table, cache)
+    M, K = a.shape
+    H, Hk, d = n_heads, n_kv_heads, head_dim
+    if not (M <= SKINNY_MAX_ROWS and _act_ok(a) and d % 32 == 0 and q_out.dtype == torch.bfloat16
+            and cache.dtype == torch.bfloat16 and q_out.stride(0) % 4 == 0 and q_out.data_ptr() % 8 == 0):
+        return False
+    ss, eps, n_ss = None, 0.0, 0
+    if pre is not None:
+        ss, eps = pre
+        if not _pre_ok(a, ss, K):
+            return False
+        n_ss = -(-K // 16)
+    _ops._need(w.K == K and w.N == (H + 2 * Hk) * d and q_out.shape[0] == M and q_out.shape[1] >= H * d,
+               f"qkv: a [{M}, {K}], w {w.shape}, {H}+2*{Hk} heads of {d}, q_out {tuple(q_out.shape)}")
+    _ops._need(cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and tuple(cos_sin.shape[1:]) == (2, d // 2),
+               "cos/sin table must be float32 [positions, 2, head_dim/2]")
+    _ops._need(cache.dim() == 5 and cache.is_contiguous() and tuple(cache.shape[1:]) == (2, Hk, page_tokens, d),
+               f"cache must be [pages, 2, {Hk}, {page_tokens}, {d}], got {tuple(cache.shape)}")
+    _ops._need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
+               "block table must be contiguous int32 [segments, blocks]")
+    L = _lib.load("tuned")
+    _lib.check(L.apc_skinny_qkv_rope_bf16(
+        a.data_ptr(), _ops._rows(a, "a"), ss.data_ptr() if ss is not None else 0, n_ss, float(eps), w.data.data_ptr(),
+        q_out.data_ptr(), _ops._rows(q_out, "q_out"), M, K, H, Hk, d, cos_sin.data_ptr(),
+        _ops._i32(positions, M, "positions"), _ops._i32(row_seg, M, "row_seg"), block_table.data_ptr(),
+        block_table.shape[1], cache.data_ptr(), page_tokens, _ops._stream()), "skinny_qkv_rope_bf16")
+    return True
+
+
 def swiglu_pre_bf16(raw: torch.Tensor, ss: torch.Tensor, eps: float, wg: PackedWeight, wu: PackedWeight,
                     out: torch.Tensor) -> bool:
     """SwiGLU of the normalised row, from what `gemm_emit_bf16` left (see `gemm_pre_bf16`)."""

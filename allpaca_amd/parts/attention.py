@@ -59,18 +59,22 @@ class Attention(Mixer):
         h = as_normed(h)
         T = h.shape[0]
         qkv = torch.empty((T, self.qkv_width), dtype=self.rt.dtype, device=h.device)
-        h.linear(self.w_qkv, qkv)
-        rot, table = (0, None)
-        if self.position is not None:
-            fused = self.position.fused()
-            if fused is None:
-                self.position.apply(qkv, self.q_off, self.k_off, self.H, self.Hk, self.d, step.positions)
-            else:
-                rot, table = fused
+        fused = self.position.fused() if self.position is not None else None
+        rot, table = fused if fused is not None else (0, None)
         kv = cache.kv if cache.writes else None
-        if kv is not None or rot:
-            ops.rope_kv_write(qkv, self.q_off, self.k_off, self.v_off, self.H, self.Hk, self.d, rot, table,
-                              step.positions, step.row_seg, cache.block_table, kv, cache.page_tokens)
+        # few rows, whole heads rotated, an own cache: one kernel gives q, k, v, rotates and fills the pages
+        if (kv is not None and rot == self.d and h.product(
+                lambda a, pre: ops.qkv_rope_write(a, pre, self.w_qkv, qkv, self.H, self.Hk, self.d, table,
+                                                  step.positions, step.row_seg, cache.block_table, kv,
+                                                  cache.page_tokens))):
+            pass
+        else:
+            h.linear(self.w_qkv, qkv)
+            if self.position is not None and fused is None:
+                self.position.apply(qkv, self.q_off, self.k_off, self.H, self.Hk, self.d, step.positions)
+            if kv is not None or rot:
+                ops.rope_kv_write(qkv, self.q_off, self.k_off, self.v_off, self.H, self.Hk, self.d, rot, table,
+                                  step.positions, step.row_seg, cache.block_table, kv, cache.page_tokens)
         attn = torch.empty((T, self.H * self.d), dtype=self.rt.dtype, device=h.device)
         ops.paged_attention(qkv, self.q_off, attn, self.H, self.Hk, self.d, cache.kv, cache.page_tokens,
                             cache.block_table, step, window=self.window or 0, scale=self.scale)

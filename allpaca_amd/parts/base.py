@@ -129,6 +129,15 @@ class NormedInput:
         if p is None or self._h is not None or not ops.linear_pre(p.raw, p.ss, p.eps, w, out):
             ops.linear(self.tensor(), w, out)
 
+    def product(self, op) -> bool:
+        """For a part with a fused first product of its own: `op(a, pre)` is called with the row that the product
+        before the norm left and pre = (ss, eps) if there is one, otherwise with the normalised tensor and
+        pre = None.  `op` returns False if it has done nothing; the part then goes through `linear`."""
+        p = self.pre
+        if p is not None and self._h is None:
+            return bool(op(p.raw, (p.ss, p.eps)))
+        return bool(op(self.tensor(), None))
+
     def swiglu(self, w_gate_up, out: torch.Tensor) -> None:
         from ..kernels import ops
         p = self.pre

@@ -316,6 +316,84 @@ def test_rotation_and_cache_write_16_bytes_a_lane_equals_the_plain_kernel(H, Hk,
         assert (results[0][1] != 0).any()
 
 
+@pytest.mark.parametrize("M,H,Hk,d,K,P_,pre", [(8, 32, 8, 128, 4096, 16, True), (5, 6, 2, 64, 328, 8, True),
+                                               (16, 3, 3, 32, 72, 24, False), (1, 5, 1, 96, 200, 16, True),
+                                               (3, 4, 2, 256, 264, 32, False)])
+def test_product_for_q_k_v_that_rotates_and_fills_the_pages_equals_the_kernels_one_after_the_other(M, H, Hk, d, K, P_, pre):
+    """One kernel for q, k, v of few rows, the rotation and the cache write gives what the product followed by
+    `rope_kv_write` gives: the same rotated q, the same pages (sums rounded to bfloat16 before the rotation in
+    both)."""
+    from allpaca_amd.kernels import ops
+    t = tuned()
+    rng = np.random.default_rng(M * 1000 + d)
+    N = (H + 2 * Hk) * d
+    w = pack(gen(N, K, seed=3, dtype=BF).to(DEV))
+    a = gen(M, K, seed=1, dtype=BF, scale=2.0).to(DEV)
+    eps = 2e-5
+    ss = None
+    if pre:
+        bands = -(-K // 16)
+        ss = torch.zeros(16, -(-bands // 4) * 4, device=DEV)
+        ss[:M, :bands] = torch.from_numpy(rng.uniform(0.5, 40.0, (M, bands)).astype(np.float32)).to(DEV)
+    max_pos = 5 * P_
+    # rows of three segments at scattered positions, among them a page's first and last slot
+    pos_list = [int(x) for x in rng.integers(0, max_pos, M)]
+    pos_list[0] = P_ - 1
+    if M > 1:
+        pos_list[1] = 2 * P_
+    seg_list = [r % 3 for r in range(M)]
+    while len({(s_, p_) for s_, p_ in zip(seg_list, pos_list)}) < M:        # no two rows on one place of the cache
+        pos_list = [(p_ + r) % max_pos for r, p_ in enumerate(pos_list)]
+    pos = torch.tensor(pos_list, dtype=torch.int32, device=DEV)
+    seg = torch.tensor(seg_list, dtype=torch.int32, device=DEV)
+    max_blocks = 5
+    bt = torch.from_numpy(rng.permutation(3 * max_blocks).reshape(3, max_blocks).astype(np.int32)).to(DEV)
+    ang = np.arange(max_pos)[:, None] * (1.0 / 300.0 ** (np.arange(d // 2) / (d // 2)))[None, :]
+    table = torch.from_numpy(np.stack([np.cos(ang), np.sin(ang)], 1).astype(np.float32)).to(DEV)
+    results = []
+    for fused in (True, False):
+        qkv = torch.full((M, N), 3.0, dtype=BF, device=DEV)
+        cache = torch.zeros(3 * max_blocks, 2, Hk, P_, d, dtype=BF, device=DEV)
+        if fused:
+            assert ops.qkv_rope_write(a, (ss, eps) if pre else None, w, qkv, H, Hk, d, table, pos, seg, bt, cache, P_)
+        else:
+            if pre:
+                assert t.gemm_pre_bf16(a, ss, eps, w, qkv)
+            else:
+                ops.linear(a, w, qkv)
+            ops.rope_kv_write(qkv, 0, H * d, (H + Hk) * d, H, Hk, d, d, table, pos, seg, bt, cache, P_)
+        c64 = f64(cache)
+        results.append((f64(qkv)[:, :H * d].reshape(M, H, 2, d // 2), c64[:, 0].reshape(-1, Hk, P_, 2, d // 2), c64[:, 1]))
+    # The two ways add the waves' partial sums in different orders, so now and then a sum falls on the other side
+    # of a rounding to bfloat16: one unit of one element of a pair, which the rotation spreads over the pair
+    # (its length is what the rotation keeps), and one unit of the result.
+    for which, (got, want) in enumerate(zip(results[0], results[1])):
+        diff = np.abs(got - want)
+        pair = np.sqrt((want ** 2).sum(axis=-2, keepdims=True)) if which < 2 else 0.0
+        assert (diff <= 2.0 ** -7 * np.abs(want) + 2.0 ** -7 * pair + 1e-30).all() and (diff > 0).mean() < 0.02
+    assert (results[0][1] != 0).sum() + (results[0][2] != 0).sum() == M * 2 * Hk * d   # every row wrote its k and v, once
+
+
+def test_product_for_q_k_v_that_rotates_declines_what_it_does_not_take():
+    from allpaca_amd.kernels import ops
+    H, Hk, d, K, P_ = 2, 1, 48, 64, 16                                          # head size no multiple of 32
+    w = pack(gen((H + 2 * Hk) * d, K, seed=3, dtype=BF).to(DEV))
+    table = torch.zeros(32, 2, d // 2, device=DEV)
+    z = torch.zeros(4, dtype=torch.int32, device=DEV)
+    bt = torch.zeros(1, 2, dtype=torch.int32, device=DEV)
+    cache = torch.zeros(2, 2, Hk, P_, d, dtype=BF, device=DEV)
+    qkv = torch.zeros(4, (H + 2 * Hk) * d, dtype=BF, device=DEV)
+    a = gen(4, K, seed=1, dtype=BF).to(DEV)
+    assert not ops.qkv_rope_write(a, None, w, qkv, H, Hk, d, table, z, z, bt, cache, P_)
+    assert not cache.any() and not qkv.any()
+    a17 = gen(17, K, seed=1, dtype=BF).to(DEV)                                   # more rows than the kernel takes
+    w2 = pack(gen(4 * 64, K, seed=3, dtype=BF).to(DEV))
+    cache2 = torch.zeros(2, 2, 1, P_, 64, dtype=BF, device=DEV)
+    assert not ops.qkv_rope_write(a17, None, w2, torch.zeros(17, 256, dtype=BF, device=DEV), 2, 1, 64,
+                                  torch.zeros(32, 2, 32, device=DEV), torch.zeros(17, dtype=torch.int32, device=DEV),
+                                  torch.zeros(17, dtype=torch.int32, device=DEV), bt, cache2, P_)
+
+
 def run_attention(H, Hk, d, P_, lens, rows_per_seg, window=0, seed=0):
     """Sequences of `lens` keys in the cache; the last `rows_per_seg[s]` positions of sequence s are the step's rows."""
     from allpaca_amd.engine.batch import Entry, pack_step
