@@ -65,6 +65,11 @@ class Engine:
         return cls(folder, config, **options)
 
     # ---- requests ------------------------------------------------------------
+    def warm_up(self, max_context: Optional[int] = None) -> int:
+        """Captures the decode graphs of every batch size up to `max_active_requests` and every context bucket up to
+        `max_context` (default: the longest the run allows) before serving starts; returns their number."""
+        return self.runner.capture_decode_graphs(self.config.max_active_requests, max_context)
+
     def add_request(self, prompt_token_ids: Sequence[int], params: Optional[GenerationParams] = None) -> int:
         params = params or GenerationParams()
         prompt = [int(t) for t in prompt_token_ids]

@@ -126,18 +126,45 @@ class ModelRunner:
         g.fill(seqs)
         return self._launch(g, [e.tokens[0] for e in entries])
 
-    def _graph_for(self, seqs: Sequence[Hashable]) -> "DecodeGraph":
-        n = len(seqs)
+    def _bucket(self, n: int, longest: int) -> tuple:
+        """(rows, span) of the graph for n requests of which the longest will hold `longest` tokens."""
         rows = 1 << max(0, (n - 1).bit_length())
-        longest = max(self.cache.length(s) for s in seqs) + 1
         span = max(256, 1 << (longest - 1).bit_length())
         span = min(span, -(-self.rt.max_positions // self.cache.page_tokens) * self.cache.page_tokens)
-        span = max(span, longest)
-        key = (rows, span)
+        return rows, max(span, longest)
+
+    def _graph_for(self, seqs: Sequence[Hashable]) -> "DecodeGraph":
+        key = self._bucket(len(seqs), max(self.cache.length(s) for s in seqs) + 1)
         g = self.graphs.get(key)
         if g is None:
-            g = self.graphs[key] = DecodeGraph(self, rows, span)
+            g = self.graphs[key] = DecodeGraph(self, *key)
         return g
+
+    def capture_decode_graphs(self, max_rows: int, max_context: Optional[int] = None) -> int:
+        """Captures now, instead of at its first use (some tens of milliseconds in the middle of serving), the
+        graph of every bucket that decode steps of up to `max_rows` requests and `max_context` tokens (default:
+        the run's limit) can ask for.  Returns how many graphs were captured."""
+        if not self.use_graphs:
+            return 0
+        top = min(max_context or self.rt.max_positions, self.rt.max_positions)
+        keys = set()
+        n = 1
+        while True:
+            longest = 1
+            while True:
+                keys.add(self._bucket(min(n, max_rows), min(longest, top)))
+                if longest >= top:
+                    break
+                longest *= 2
+            if n >= max_rows:
+                break
+            n *= 2
+        made = 0
+        for key in sorted(keys):
+            if key not in self.graphs:
+                self.graphs[key] = DecodeGraph(self, *key)
+                made += 1
+        return made
 
     def _launch(self, g: "DecodeGraph", tokens: Sequence[int]) -> torch.Tensor:
         g.set_tokens(tokens)

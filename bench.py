@@ -25,7 +25,8 @@ HBM_PEAK_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 
-def build_engine(cfg_json, dtype, batch, context, extra_tokens, layers, seed=0, use_graphs=True, max_context=0):
+def build_engine(cfg_json, dtype, batch, context, extra_tokens, layers, seed=0, use_graphs=True, max_context=0,
+                 chunk_tokens=2048, pool_tokens=0):
     """An engine on random weights made directly on the GPU (no model folder is written for 16 GB)."""
     import torch
 
@@ -47,8 +48,8 @@ def build_engine(cfg_json, dtype, batch, context, extra_tokens, layers, seed=0, 
     # every sequence may grow to `max_context` tokens (positions, block table, pages of the pool)
     per_seq = -(-max(context + extra_tokens, max_context) // page) * page
     ec = EngineConfig(dtype="bfloat16" if dtype == "bf16" else "float32", page_tokens=page,
-                      num_pages=batch * per_seq // page + 8, max_active_requests=max(batch, 1),
-                      max_batch_tokens=2048, chunk_tokens=2048, use_graphs=use_graphs)
+                      num_pages=(pool_tokens or batch * per_seq) // page + 8, max_active_requests=max(batch, 1),
+                      max_batch_tokens=2048, chunk_tokens=chunk_tokens, use_graphs=use_graphs)
     rt = Runtime(torch.device("cuda:0"), tdt, per_seq)
     # weights tensor by tensor on the GPU: nothing of 16 GB passes through host memory
     specs = model.param_specs()
@@ -155,6 +156,35 @@ def prefill_run(eng, cfg, tokens, repeats=3):
     return best
 
 
+def requests_run(eng, cfg, n_requests, min_prompt, max_prompt, new_tokens, seed=0):
+    """`n_requests` requests with prompts of random length arrive at once and run to `new_tokens` tokens each
+    through the scheduler: portions of prompts beside decoding rows.  Returns a dict of totals and mean times."""
+    import numpy as np
+    import torch
+
+    from allpaca_amd.sampling import GenerationParams
+    rng = np.random.default_rng(seed)
+    lengths = [int(x) for x in rng.integers(min_prompt, max_prompt + 1, size=n_requests)]
+    gp = GenerationParams(max_tokens=new_tokens, temperature=0.0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ids = [eng.add_request(rng.integers(0, cfg.vocab_size, size=n).tolist(), gp) for n in lengths]
+    reqs = [eng.requests[i] for i in ids]
+    steps = 0
+    while eng.has_unfinished():
+        eng.step()
+        steps += 1
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    times = [r.timing() for r in reqs]
+    out_tokens = sum(len(r.output) for r in reqs)
+    assert out_tokens == n_requests * new_tokens, f"{out_tokens} tokens from {n_requests} requests"
+    return {"seconds": dt, "steps": steps, "prompt_tokens": sum(lengths), "output_tokens": out_tokens,
+            "ttft_ms": 1e3 * float(np.mean([t["ttft"] for t in times])),
+            "itl_ms": 1e3 * float(np.mean([t["itl"] for t in times])),
+            "preemptions": eng.scheduler.preemption_count}
+
+
 def prefill_flops(cfg, layers, T):
     D, F, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
     H, Hk, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
@@ -177,6 +207,13 @@ def main() -> int:
     ap.add_argument("--preset", default="llama-3.1-8b")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points and the prefill")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--requests", type=int, default=0,
+                    help="instead of the decode steps: this many requests with prompts of --min-prompt..--max-prompt "
+                         "tokens arrive at once and decode --new-tokens tokens each under chunked prefill")
+    ap.add_argument("--min-prompt", type=int, default=128)
+    ap.add_argument("--max-prompt", type=int, default=4096)
+    ap.add_argument("--new-tokens", type=int, default=256)
+    ap.add_argument("--chunk", type=int, default=512, help="largest portion of a prompt in a step (with --requests)")
     ap.add_argument("--only", choices=["decode", "prefill"], default=None,
                     help="for profiling: only the decode steps at --batch (as --no-points), or only the 2,048-token "
                          "prefill (prints its figures as the line's value)")
@@ -195,6 +232,28 @@ def main() -> int:
     klib.load("plain")
     klib.load("tuned")
 
+    if args.requests:
+        n = args.requests
+        top = args.max_prompt + args.new_tokens
+        cfg, eng = build_engine(cfg_json, args.dtype, n, top, 0, layers, use_graphs=not args.no_graphs,
+                                max_context=top, chunk_tokens=args.chunk, pool_tokens=n * (top + 16))
+        t0 = time.perf_counter()
+        captured = eng.warm_up()                                                                    # decode graphs
+        requests_run(eng, cfg, min(n, 4), args.min_prompt, min(args.max_prompt, 512), 8, seed=1)   # first launches
+        warm = time.perf_counter() - t0
+        r = requests_run(eng, cfg, n, args.min_prompt, args.max_prompt, args.new_tokens)
+        print(json.dumps({
+            "metric": f"output tok/s, {n} requests at once, prompts {args.min_prompt}-{args.max_prompt}, "
+                      f"{args.new_tokens} new tokens each, chunked prefill",
+            "value": round(r["output_tokens"] / r["seconds"], 1), "unit": "tok/s", "n_gpus": 1,
+            "seconds": round(r["seconds"], 3), "steps": r["steps"], "prompt_tokens": r["prompt_tokens"],
+            "output_tokens": r["output_tokens"], "all_tokens_per_s": round((r["prompt_tokens"] + r["output_tokens"]) / r["seconds"], 1),
+            "mean_ttft_ms": round(r["ttft_ms"], 1), "mean_itl_ms": round(r["itl_ms"], 2), "preemptions": r["preemptions"],
+            "graphs_captured_before": captured, "warm_up_seconds": round(warm, 2),
+            "dtype": args.dtype, "data": "synthetic: random N(0, 0.02) weights, uniform random token ids",
+            "config": {"model": args.preset, "layers": layers, "layers_of_configuration": full_layers,
+                       "chunk_tokens": args.chunk, "max_batch_tokens": 2048, "page_tokens": 16}}), flush=True)
+        return 0
     if args.only == "decode":
         args.no_points = True
     if args.only == "prefill":
@@ -240,8 +299,7 @@ def main() -> int:
 
     sec = ms[args.batch] / 1e3
     out = {
-        "metric": "decode tok/s @ batch 8, context 2048 (Llama-3.1-8B shapes)" if (args.batch, args.context) == (8, 2048)
-        else f"decode tok/s @ batch {args.batch}, context {args.context}",
+        "metric": f"decode tok/s @ batch {args.batch}, context {args.context} ({args.preset} shapes)",
         "value": round(args.batch / sec, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms[args.batch], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic: random N(0, 0.02) weights, uniform random token ids",

@@ -259,6 +259,23 @@ def test_generation_with_graphs_equals_the_plain_implementation():
     assert eng.runner.graph_replays > 0
 
 
+def test_graphs_captured_before_serving_are_the_ones_generation_asks_for():
+    """`warm_up` captures every (rows, context) bucket; generation afterwards captures none and gives the plain
+    implementation's tokens."""
+    folder = H.model_folder("B", "float32", True)
+    cfg, w = H.oracle(folder)
+    prompts = [H.random_tokens(cfg["vocab_size"], n, seed=n) for n in (2, 7, 20, 3, 11)]
+    want = [P.greedy_generate(cfg, w, p, 12) for p in prompts]
+    eng = engine_for(folder, use_graphs=True, max_active_requests=5, max_tokens=2048)
+    made = eng.warm_up()
+    assert made == len(eng.runner.graphs) and made >= 4 and eng.warm_up() == 0
+    assert {k[0] for k in eng.runner.graphs} == {1, 2, 4, 8}
+    outs = eng.generate(prompts, params(max_tokens=12, temperature=0.0))
+    assert [o.token_ids for o in outs] == want
+    assert len(eng.runner.graphs) == made and eng.runner.graph_replays > 0
+    assert engine_for(folder, use_graphs=False).warm_up() == 0
+
+
 def test_steps_prepared_ahead_give_the_same_tokens_when_requests_stop_arrive_and_are_aborted():
     """With graphs on, the engine sets up the next decode step while the GPU works on the current one.  A stop token,
     a request that arrives between two steps and an abort each cancel what was set up; the tokens are those of the
