@@ -25,7 +25,8 @@ def _code(t: torch.Tensor) -> int:
 
 
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """The current HIP stream's handle (the raw call: `torch.cuda.current_stream()` builds an object each time)."""
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
 
 
 def _need(cond: bool, msg: str) -> None:
@@ -41,15 +42,18 @@ def _gpu(*ts: Optional[torch.Tensor]) -> None:
 
 def _rows(t: torch.Tensor, what: str) -> int:
     """A [rows, cols] view with unit column stride; returns its row stride."""
-    _need(t.dim() == 2, f"{what}: expected 2 dimensions, got shape {tuple(t.shape)}")
-    _need(t.shape[1] == 0 or t.stride(1) == 1, f"{what}: columns must be contiguous")
+    if not (t.dim() == 2):
+        raise ValueError(f"{what}: expected 2 dimensions, got shape {tuple(t.shape)}")
+    if not (t.shape[1] == 0 or t.stride(1) == 1):
+        raise ValueError(f"{what}: columns must be contiguous")
     return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
 
 
 def _i32(t: Optional[torch.Tensor], n: int, what: str) -> int:
     if t is None:
         return 0
-    _need(t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n, f"{what}: need >= {n} contiguous int32")
+    if not (t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n):
+        raise ValueError(f"{what}: need >= {n} contiguous int32")
     return t.data_ptr()
 
 
@@ -89,8 +93,8 @@ def rmsnorm_rows(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.T
     ldx, ldo = _rows(x, "rmsnorm x"), _rows(out, "rmsnorm out")
     R = out.shape[0]
     D = x.shape[1]
-    _need(weight.dtype == torch.float32 and weight.is_contiguous() and weight.numel() == D,
-          f"rmsnorm weight must be float32 [{D}]")
+    if not (weight.dtype == torch.float32 and weight.is_contiguous() and weight.numel() == D):
+        raise ValueError(f"rmsnorm weight must be float32 [{D}]")
     _need(out.shape[1] == D, "rmsnorm out width differs from x")
     _need(rows is not None or x.shape[0] == R, "rmsnorm: out rows differ from x rows")
     L = _lib.load("plain")
@@ -146,9 +150,10 @@ def rope_kv_write(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads
     max_blocks = 0
     if cache is not None:
         _need(block_table is not None and row_seg is not None, "cache write needs a block table and row segments")
-        _need(cache.dim() == 5 and cache.is_contiguous() and cache.shape[1] == 2 and cache.shape[2] == n_kv_heads
-              and cache.shape[3] == page_tokens and cache.shape[4] == head_dim,
-              f"cache must be [pages, 2, {n_kv_heads}, {page_tokens}, {head_dim}], got {tuple(cache.shape)}")
+        if not (cache.dim() == 5 and cache.is_contiguous()
+                and tuple(cache.shape[1:]) == (2, n_kv_heads, page_tokens, head_dim)):
+            raise ValueError(f"cache must be [pages, 2, {n_kv_heads}, {page_tokens}, {head_dim}], "
+                             f"got {tuple(cache.shape)}")
         _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
               "block table must be contiguous int32 [segments, blocks]")
         max_blocks = block_table.shape[1]
@@ -179,8 +184,10 @@ def gemm_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: 
     lda, ldw, ldc = _rows(a, "gemm a"), _rows(w, "gemm w"), _rows(out, "gemm out")
     M, K = a.shape
     N = w.shape[0]
-    _need(w.shape[1] == K, f"gemm: a is [*, {K}] but w is {tuple(w.shape)}")
-    _need(out.shape == (M, N), f"gemm: out must be [{M}, {N}], got {tuple(out.shape)}")
+    if not (w.shape[1] == K):
+        raise ValueError(f"gemm: a is [*, {K}] but w is {tuple(w.shape)}")
+    if not (out.shape == (M, N)):
+        raise ValueError(f"gemm: out must be [{M}, {N}], got {tuple(out.shape)}")
     _need(not accumulate or out.dtype == torch.float32, "gemm: accumulation needs a float32 destination")
     L = _lib.load("plain")
     for r0 in range(0, M, 1 << 21):  # grid.y limit: 65535 tiles of 64 rows
@@ -201,8 +208,9 @@ def paged_attention_plain(q: torch.Tensor, q_off: int, out: torch.Tensor, n_head
     _need(out.shape == (T, n_heads * head_dim), "attention out must be [rows, heads*head_dim]")
     _need(n_heads % n_kv_heads == 0, "heads must be a multiple of kv heads")
     _need(head_dim <= 256, "plain attention handles head_dim <= 256")
-    _need(cache.dim() == 5 and cache.is_contiguous() and tuple(cache.shape[1:]) == (2, n_kv_heads, page_tokens, head_dim),
-          f"cache must be [pages, 2, {n_kv_heads}, {page_tokens}, {head_dim}], got {tuple(cache.shape)}")
+    if not (cache.dim() == 5 and cache.is_contiguous()
+            and tuple(cache.shape[1:]) == (2, n_kv_heads, page_tokens, head_dim)):
+        raise ValueError(f"cache must be [pages, 2, {n_kv_heads}, {page_tokens}, {head_dim}], got {tuple(cache.shape)}")
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
           "block table must be contiguous int32 [segments, blocks]")
     L = _lib.load("plain")
@@ -232,7 +240,8 @@ def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Te
     R, V = logits.shape
     _need(logits.dtype == torch.float32, "logits are float32")
     for t, name in ((temperature, "temperature"), (top_p, "top_p"), (uniform, "uniform")):
-        _need(t.dtype == torch.float32 and t.is_contiguous() and t.numel() >= R, f"{name}: float32 [{R}]")
+        if not (t.dtype == torch.float32 and t.is_contiguous() and t.numel() >= R):
+            raise ValueError(f"{name}: float32 [{R}]")
     L = _lib.load("plain")
     _lib.check(L.apc_sample_rows(logits.data_ptr(), ld, R, V, temperature.data_ptr(), _i32(top_k, R, "top_k"),
                                  top_p.data_ptr(), uniform.data_ptr(), _i32(out, R, "sample out"), _stream()),

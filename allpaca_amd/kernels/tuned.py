@@ -15,6 +15,7 @@ from . import lib as _lib
 from . import ops as _ops
 from .packing import PackedWeight
 
+MANY_ROWS_SPLIT_MAX = 1024   # up to here the tiled kernel may cut K into slices to get enough blocks
 SKINNY_MAX_ROWS = 16     # the streaming kernel: up to one 16-row tile of activations
 SPLITK_MAX_ROWS = 128    # the tiled kernel with K cut into slices: 17..128 rows
 
@@ -23,6 +24,25 @@ def _k_split(M: int, N: int, K: int) -> int:
     """Slices of K for the split kernel: enough blocks for the chip (about 512), at least 4 K-steps of 64 each."""
     blocks = -(-N // 128) * -(-M // 128)
     s = max(1, min(8, -(-512 // blocks)))
+    return max(1, min(s, K // 256))
+
+
+def _k_split_many_rows(M: int, N: int, K: int) -> int:
+    """Slices of K for 129..1024 rows: a matrix with few output columns gives the 128 x 128 tiles too few blocks
+    for 256 compute units (o_proj and down of an 8B model at 512 rows: 128), and slicing K, at the price of writing
+    and adding float32 partial sums, was measured faster up to about 200 blocks (down, 4096 x 14336, 256 rows: 150
+    us whole, 52 us in 4 slices); with more outputs than K and 150 blocks or more it was not."""
+    blocks = -(-N // 128) * -(-M // 128)
+    if blocks <= 56:
+        s = 5
+    elif blocks <= 68:
+        s = 4
+    elif blocks <= 88:
+        s = 3
+    elif blocks <= 208 and not (blocks >= 150 and N > K):
+        s = 2
+    else:
+        s = 1
     return max(1, min(s, K // 256))
 
 
@@ -39,8 +59,10 @@ def gemm_bf16(a: torch.Tensor, w: PackedWeight, out: torch.Tensor, accumulate: b
     _ops._gpu(a, w.data, out)
     M, K = a.shape
     N = w.N
-    _ops._need(w.K == K, f"gemm: a is [*, {K}] but w is {w.shape}")
-    _ops._need(out.shape == (M, N), f"gemm: out must be [{M}, {N}], got {tuple(out.shape)}")
+    if not (w.K == K):
+        raise ValueError(f"gemm: a is [*, {K}] but w is {w.shape}")
+    if not (out.shape == (M, N)):
+        raise ValueError(f"gemm: out must be [{M}, {N}], got {tuple(out.shape)}")
     _ops._need(not accumulate or out.dtype == torch.float32, "gemm: accumulation needs a float32 destination")
     _ops._need(out.dtype in (torch.bfloat16, torch.float32), "gemm: out must be bfloat16 or float32")
     _ops._need(w.data.is_contiguous() and w.data.shape[0] * 16 >= N and w.data.shape[1] * 32 >= K,
@@ -51,8 +73,8 @@ def gemm_bf16(a: torch.Tensor, w: PackedWeight, out: torch.Tensor, accumulate: b
     lda, ldc = _ops._rows(a, "a"), _ops._rows(out, "out")
     mode = 2 if accumulate else (0 if out.dtype == torch.bfloat16 else 1)
     L = _lib.load("tuned")
-    if SKINNY_MAX_ROWS < M <= SPLITK_MAX_ROWS:
-        ks = _k_split(M, N, K)
+    if SKINNY_MAX_ROWS < M <= MANY_ROWS_SPLIT_MAX:
+        ks = _k_split(M, N, K) if M <= SPLITK_MAX_ROWS else _k_split_many_rows(M, N, K)
         if ks > 1:
             ws = torch.empty(ks * M * N, dtype=torch.float32, device=a.device)
             _lib.check(L.apc_gemm_splitk_bf16(a.data_ptr(), lda, w.data.data_ptr(), 0, out.data_ptr(), ldc, M, N, K,
@@ -68,15 +90,17 @@ def swiglu_bf16(h: torch.Tensor, wg: PackedWeight, wu: PackedWeight, out: torch.
     _ops._gpu(h, wg.data, wu.data, out)
     M, K = h.shape
     F = out.shape[1]
-    _ops._need(wg.shape == (F, K) and wu.shape == (F, K), f"swiglu: weights must both be [{F}, {K}]")
+    if not (wg.shape == (F, K) and wu.shape == (F, K)):
+        raise ValueError(f"swiglu: weights must both be [{F}, {K}]")
     _ops._need(out.shape[0] == M and out.dtype == torch.bfloat16, "swiglu: out must be bfloat16 [rows, F]")
     if not _act_ok(h):
         raise ValueError("swiglu_bf16: activations must be bfloat16 rows of a width and stride that are multiples "
                          "of 8, 16-byte aligned")
     lda, ldc = _ops._rows(h, "h"), _ops._rows(out, "out")
     L = _lib.load("tuned")
-    if SKINNY_MAX_ROWS < M <= SPLITK_MAX_ROWS:
-        ks = _k_split(M, 2 * F, K)
+    ks = _k_split_many_rows(M, 2 * F, K) if SPLITK_MAX_ROWS < M <= MANY_ROWS_SPLIT_MAX else 1
+    if SKINNY_MAX_ROWS < M <= SPLITK_MAX_ROWS or ks > 1:
+        ks = _k_split(M, 2 * F, K) if M <= SPLITK_MAX_ROWS else ks
         ws = torch.empty(2 * ks * M * F, dtype=torch.float32, device=h.device)
         _lib.check(L.apc_gemm_splitk_bf16(h.data_ptr(), lda, wg.data.data_ptr(), wu.data.data_ptr(), out.data_ptr(), ldc,
                                           M, F, K, 3, ks, ws.data_ptr(), _ops._stream()), "gemm_splitk_bf16")
@@ -98,7 +122,8 @@ def gemm_emit_bf16(a: torch.Tensor, w: PackedWeight, residual: torch.Tensor, g: 
     if (M > SPLITK_MAX_ROWS or not _act_ok(a) or residual.dtype != torch.float32 or g.dtype != torch.float32
             or g.numel() != N or not g.is_contiguous()):
         return None
-    _ops._need(w.K == K and residual.shape == (M, N), f"gemm: a [{M}, {K}], w {w.shape}, residual {tuple(residual.shape)}")
+    if not (w.K == K and residual.shape == (M, N)):
+        raise ValueError(f"gemm: a [{M}, {K}], w {w.shape}, residual {tuple(residual.shape)}")
     raw = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
     if M > SKINNY_MAX_ROWS:   # the tiled kernel with K in slices: sums per row and block of 256 columns
         ks = _k_split(M, N, K)
@@ -150,7 +175,8 @@ def gemm_pre_bf16(raw: torch.Tensor, ss: torch.Tensor, eps: float, w: PackedWeig
     M, K = raw.shape
     if out.dtype not in (torch.bfloat16, torch.float32):
         return False
-    _ops._need(w.K == K and out.shape == (M, w.N), f"gemm: raw [{M}, {K}], w {w.shape}, out {tuple(out.shape)}")
+    if not (w.K == K and out.shape == (M, w.N)):
+        raise ValueError(f"gemm: raw [{M}, {K}], w {w.shape}, out {tuple(out.shape)}")
     if M > SKINNY_MAX_ROWS:
         return _pre_splitk(raw, ss, eps, w, None, out, w.N, 0 if out.dtype == torch.bfloat16 else 1)
     if not _pre_ok(raw, ss, K):
@@ -182,12 +208,12 @@ def qkv_rope_bf16(a: torch.Tensor, pre, w: PackedWeight, q_out: torch.Tensor, n_
         if not _pre_ok(a, ss, K):
             return False
         n_ss = -(-K // 16)
-    _ops._need(w.K == K and w.N == (H + 2 * Hk) * d and q_out.shape[0] == M and q_out.shape[1] >= H * d,
-               f"qkv: a [{M}, {K}], w {w.shape}, {H}+2*{Hk} heads of {d}, q_out {tuple(q_out.shape)}")
+    if not (w.K == K and w.N == (H + 2 * Hk) * d and q_out.shape[0] == M and q_out.shape[1] >= H * d):
+        raise ValueError(f"qkv: a [{M}, {K}], w {w.shape}, {H}+2*{Hk} heads of {d}, q_out {tuple(q_out.shape)}")
     _ops._need(cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and tuple(cos_sin.shape[1:]) == (2, d // 2),
                "cos/sin table must be float32 [positions, 2, head_dim/2]")
-    _ops._need(cache.dim() == 5 and cache.is_contiguous() and tuple(cache.shape[1:]) == (2, Hk, page_tokens, d),
-               f"cache must be [pages, 2, {Hk}, {page_tokens}, {d}], got {tuple(cache.shape)}")
+    if not (cache.dim() == 5 and cache.is_contiguous() and tuple(cache.shape[1:]) == (2, Hk, page_tokens, d)):
+        raise ValueError(f"cache must be [pages, 2, {Hk}, {page_tokens}, {d}], got {tuple(cache.shape)}")
     _ops._need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
                "block table must be contiguous int32 [segments, blocks]")
     L = _lib.load("tuned")
@@ -207,7 +233,8 @@ def swiglu_pre_bf16(raw: torch.Tensor, ss: torch.Tensor, eps: float, wg: PackedW
     F = out.shape[1]
     if out.dtype != torch.bfloat16:
         return False
-    _ops._need(wg.shape == (F, K) and wu.shape == (F, K) and out.shape[0] == M, f"swiglu: weights must both be [{F}, {K}]")
+    if not (wg.shape == (F, K) and wu.shape == (F, K) and out.shape[0] == M):
+        raise ValueError(f"swiglu: weights must both be [{F}, {K}]")
     if M > SKINNY_MAX_ROWS:
         return _pre_splitk(raw, ss, eps, wg, wu, out, F, 3)
     if not _pre_ok(raw, ss, K):
@@ -248,9 +275,9 @@ def attention_bf16(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int,
     _ops._need(q_off + n_heads * head_dim <= q.shape[1], "attention: q heads exceed the row")
     _ops._need(out.shape == (T, n_heads * head_dim), "attention out must be [rows, heads*head_dim]")
     _ops._need(n_heads % n_kv_heads == 0, "heads must be a multiple of kv heads")
-    _ops._need(cache.dim() == 5 and cache.is_contiguous()
-               and tuple(cache.shape[1:]) == (2, n_kv_heads, page_tokens, head_dim),
-               f"cache must be [pages, 2, {n_kv_heads}, {page_tokens}, {head_dim}], got {tuple(cache.shape)}")
+    if not (cache.dim() == 5 and cache.is_contiguous()
+            and tuple(cache.shape[1:]) == (2, n_kv_heads, page_tokens, head_dim)):
+        raise ValueError(f"cache must be [pages, 2, {n_kv_heads}, {page_tokens}, {head_dim}], got {tuple(cache.shape)}")
     _ops._need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
                "block table must be contiguous int32 [segments, blocks]")
     _ops._need(step.positions.numel() >= T and step.row_seg.numel() >= T, "step rows differ from q rows")

@@ -53,7 +53,9 @@ GEMM_SHAPES = [(1, 5, 16), (3, 100, 136), (8, 4096, 512), (16, 33, 1208), (17, 2
                (65, 64, 64), (128, 129, 72), (200, 300, 200), (300, 515, 120), (1000, 40, 1024),
                (40, 200, 1208), (64, 130, 2056), (100, 96, 520), (128, 48, 4096), (130, 200, 320), (256, 130, 192),
                # enough blocks for the 256-row tiles: a last tile of 232 rows, K a multiple of 64 and not
-               (1000, 8192, 200), (1024, 8190, 192)]
+               (1000, 8192, 200), (1024, 8190, 192),
+               # 129..1024 rows and few output columns: K in slices (5, 2 and 3 of them), a last row tile of 44 rows
+               (512, 384, 2048), (200, 4096, 520), (300, 1100, 1024)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
@@ -260,7 +262,7 @@ def test_embedding_from_the_tiled_table():
     assert torch.equal(out.cpu(), table.float().cpu()[toks.cpu().long()])
 
 
-@pytest.mark.parametrize("M,F,K", [(1, 24, 64), (8, 176, 64), (9, 200, 120), (64, 512, 192), (65, 40, 72),
+@pytest.mark.parametrize("M,F,K", [(1, 24, 64), (8, 176, 64), (9, 200, 120), (64, 512, 192), (65, 40, 72), (300, 520, 1024),
                                    (130, 200, 120), (300, 512, 192), (256, 14336 // 8, 512), (48, 176, 1032),
                                    (100, 72, 2048), (300, 200, 320), (1000, 4096, 200), (1024, 4090, 128)])
 def test_swiglu_bf16(M, F, K):
