@@ -33,13 +33,25 @@ struct GemmRegs {
   Frag a[BM / 32], w[4];
 };
 
+// PRE (storing modes): A is the row bfloat16(x * g) that a product into the residual left for the RMS norm, and
+// ss[m][parts] are its sums of x^2 per row and block of columns; the sums of this product are scaled by
+// 1 / sqrt(sum(ss[m]) / K + eps): the product of the normalised row without a kernel for the norm.
+struct TiledPre {
+  const float* ss;
+  int parts;
+  float eps;
+};
+
 // EVEN_K: K is a multiple of 64, so no load needs a bound check.  BM: rows of the block tile, 128 or 256.
-template <int MODE, bool EVEN_K, int BM>
+template <int MODE, bool EVEN_K, int BM, bool PRE = false>
 __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda,
                                                         const bf16_t* __restrict__ W,
                                                         const bf16_t* __restrict__ W2, int chunks,
                                                         void* __restrict__ C, int ldc, int M, int N, int K,
-                                                        int k_split) {
+                                                        int k_split, TiledPre pre = TiledPre{}) {
+  static_assert(!PRE || MODE == G_STORE_BF16 || MODE == G_STORE_F32 || MODE == G_SWIGLU,
+                "a product that reads a normalised row stores its result");
+  __shared__ float rstd_s[PRE ? BM : 1];
   constexpr int AP = BM / 32;          // 16-byte pieces of A per thread and K step
   constexpr int WM = BM / 64;          // 32-row accumulators of a wave along M
   constexpr int PIECES = AP + 4;       // pieces of A and W per thread and K step
@@ -67,6 +79,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
     if (nt >= NT || mt >= MT) return;
   }
   const int m0 = mt * BM, n0 = nt * NB;
+  if constexpr (PRE) {  // one row a thread, its parts added in order; read after the barriers of the K loop
+    if (tid < BM) {
+      const float* row = pre.ss + (size_t)min(m0 + tid, M - 1) * pre.parts;
+      float sum = 0.f;
+      for (int p = 0; p < pre.parts; ++p) sum += row[p];
+      rstd_s[tid] = 1.0f / sqrtf(sum / (float)K + pre.eps);
+    }
+  }
   // G_PARTIAL: blockIdx.z = which * k_split + slice; the block multiplies slice `slice` of K with matrix `which`
   // (0: W, 1: W2) and leaves its float32 sums in C[which][slice][M][N]
   const int slice = MODE == G_PARTIAL ? blockIdx.z % k_split : 0;
@@ -209,6 +229,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
     for (int r = 0; r < 16; ++r) {
       const int m = m0 + wm * (BM / 2) + a * 32 + (r / 4) * 8 + lc * 4 + (r % 4);
       if (m >= M) continue;
+      if constexpr (PRE) {
+        const float rs = rstd_s[m - m0];
+        acc[a][0][r] *= rs;
+        acc[a][1][r] *= rs;
+      }
       if (MODE == G_SWIGLU) {
         const int n = n0 + wn * 32 + li;
         if (n < N) ((bf16_t*)C)[(size_t)m * ldc + n] = float_to_bf16(silu_f(acc[a][0][r]) * acc[a][1][r]);
@@ -230,18 +255,18 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
 
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
-template <int MODE>
+template <int MODE, bool PRE = false>
 static int launch_gemm(const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M, int N,
-                       int K, hipStream_t stream) {
+                       int K, hipStream_t stream, TiledPre pre = TiledPre{}) {
   constexpr int NB = MODE == G_SWIGLU ? BN / 2 : BN;
   const long blocks = 8L * ceil_div(ceil_div(N, NB), 8) * ceil_div(M, BM_ROWS);
   if (blocks > 0x7fffffffL) return APC_ERR_BAD_ARG;
   if (K % BK == 0)
-    hipLaunchKernelGGL((gemm_bf16_kernel<MODE, true, BM_ROWS>), dim3((unsigned)blocks), dim3(256), 0, stream, A, lda, W,
-                       W2, ceil_div(K, 32), C, ldc, M, N, K, 1);
+    hipLaunchKernelGGL((gemm_bf16_kernel<MODE, true, BM_ROWS, PRE>), dim3((unsigned)blocks), dim3(256), 0, stream, A,
+                       lda, W, W2, ceil_div(K, 32), C, ldc, M, N, K, 1, pre);
   else
-    hipLaunchKernelGGL((gemm_bf16_kernel<MODE, false, BM_ROWS>), dim3((unsigned)blocks), dim3(256), 0, stream, A, lda, W,
-                       W2, ceil_div(K, 32), C, ldc, M, N, K, 1);
+    hipLaunchKernelGGL((gemm_bf16_kernel<MODE, false, BM_ROWS, PRE>), dim3((unsigned)blocks), dim3(256), 0, stream, A,
+                       lda, W, W2, ceil_div(K, 32), C, ldc, M, N, K, 1, pre);
   APC_LAUNCH_CHECK();
   return 0;
 }
@@ -317,7 +342,7 @@ static int launch_splitk(const void* A, int lda, const void* W, const void* Wu, 
 #define PARTIAL_LAUNCH(EVEN_, BM_)                                                                                  \
   hipLaunchKernelGGL((gemm_bf16_kernel<G_PARTIAL, EVEN_, BM_>), dim3(ceil_div(N, BN), ceil_div(M, BM_), k_split * n_mats), \
                      dim3(256), 0, stream, (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)Wu, ceil_div(K, 32), \
-                     workspace, N, M, N, K, k_split)
+                     workspace, N, M, N, K, k_split, TiledPre{})
   if (M <= 64) {
     if (K % BK == 0) PARTIAL_LAUNCH(true, 64);
     else PARTIAL_LAUNCH(false, 64);
@@ -390,4 +415,24 @@ APC_EXPORT int apc_gemm_swiglu_bf16(const void* A, int lda, const void* Wg, cons
   if (K <= 0 || lda < K || ldc < F) return APC_ERR_BAD_ARG;
   if (K % 8 || lda % 8 || !aligned16(A) || !aligned16(Wg) || !aligned16(Wu)) return APC_ERR_UNSUPPORTED;
   return launch_gemm<G_SWIGLU>((const bf16_t*)A, lda, (const bf16_t*)Wg, (const bf16_t*)Wu, C, ldc, M, F, K, stream);
+}
+
+// The storing products on a row that a product into the residual left for the RMS norm, K in one piece:
+// A = raw [M, K], ss = [M][ss_parts] sums of x^2; out = (A . W^T) / sqrt(sum(ss[m]) / K + eps).
+// mode 0 store bfloat16, 1 store float32, 3 SwiGLU (W = gate, Wu = up; C is [M, N] with N = the width of each).
+APC_EXPORT int apc_gemm_pre_bf16(const void* A, int lda, const float* ss, int ss_parts, float eps, const void* W,
+                                 const void* Wu, void* C, int ldc, int M, int N, int K, int mode, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || lda < K || ldc < N || !ss || ss_parts <= 0) return APC_ERR_BAD_ARG;
+  if ((mode == G_SWIGLU) != (Wu != nullptr)) return APC_ERR_BAD_ARG;
+  if (K % 8 || lda % 8 || !aligned16(A) || !aligned16(W) || (Wu && !aligned16(Wu))) return APC_ERR_UNSUPPORTED;
+  const bf16_t* a = (const bf16_t*)A;
+  const bf16_t* w = (const bf16_t*)W;
+  const TiledPre pre{ss, ss_parts, eps};
+  switch (mode) {
+    case G_STORE_BF16: return launch_gemm<G_STORE_BF16, true>(a, lda, w, nullptr, C, ldc, M, N, K, stream, pre);
+    case G_STORE_F32: return launch_gemm<G_STORE_F32, true>(a, lda, w, nullptr, C, ldc, M, N, K, stream, pre);
+    case G_SWIGLU: return launch_gemm<G_SWIGLU, true>(a, lda, w, (const bf16_t*)Wu, C, ldc, M, N, K, stream, pre);
+    default: return APC_ERR_BAD_ARG;
+  }
 }

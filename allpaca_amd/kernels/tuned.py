@@ -21,9 +21,10 @@ SPLITK_MAX_ROWS = 128    # the tiled kernel with K cut into slices: 17..128 rows
 
 
 def _k_split(M: int, N: int, K: int) -> int:
-    """Slices of K for the split kernel: enough blocks for the chip (about 512), at least 4 K-steps of 64 each."""
+    """Slices of K for the split kernel with 17..128 rows: about 240 blocks in all (measured best at the shapes of 3B
+    and 8B models: 32 column tiles in 6-8 slices, 48 in 4-5, 224 whole), at least 4 K-steps of 64 each."""
     blocks = -(-N // 128) * -(-M // 128)
-    s = max(1, min(8, -(-512 // blocks)))
+    s = max(1, min(12, round(240 / blocks)))
     return max(1, min(s, K // 256))
 
 
@@ -44,6 +45,13 @@ def _k_split_many_rows(M: int, N: int, K: int) -> int:
     else:
         s = 1
     return max(1, min(s, K // 256))
+
+
+def _tiled_k_split(M: int, N: int, K: int) -> int:
+    """Slices of K on the tiled kernel for M rows (1: K in one piece)."""
+    if M <= SPLITK_MAX_ROWS:
+        return _k_split(M, N, K)
+    return _k_split_many_rows(M, N, K) if M <= MANY_ROWS_SPLIT_MAX else 1
 
 
 def _aligned(*ts: torch.Tensor) -> bool:
@@ -74,7 +82,7 @@ def gemm_bf16(a: torch.Tensor, w: PackedWeight, out: torch.Tensor, accumulate: b
     mode = 2 if accumulate else (0 if out.dtype == torch.bfloat16 else 1)
     L = _lib.load("tuned")
     if SKINNY_MAX_ROWS < M <= MANY_ROWS_SPLIT_MAX:
-        ks = _k_split(M, N, K) if M <= SPLITK_MAX_ROWS else _k_split_many_rows(M, N, K)
+        ks = _tiled_k_split(M, N, K)
         if ks > 1:
             ws = torch.empty(ks * M * N, dtype=torch.float32, device=a.device)
             _lib.check(L.apc_gemm_splitk_bf16(a.data_ptr(), lda, w.data.data_ptr(), 0, out.data_ptr(), ldc, M, N, K,
@@ -98,9 +106,8 @@ def swiglu_bf16(h: torch.Tensor, wg: PackedWeight, wu: PackedWeight, out: torch.
                          "of 8, 16-byte aligned")
     lda, ldc = _ops._rows(h, "h"), _ops._rows(out, "out")
     L = _lib.load("tuned")
-    ks = _k_split_many_rows(M, 2 * F, K) if SPLITK_MAX_ROWS < M <= MANY_ROWS_SPLIT_MAX else 1
-    if SKINNY_MAX_ROWS < M <= SPLITK_MAX_ROWS or ks > 1:
-        ks = _k_split(M, 2 * F, K) if M <= SPLITK_MAX_ROWS else ks
+    ks = _tiled_k_split(M, 2 * F, K) if M > SKINNY_MAX_ROWS else 1
+    if ks > 1:
         ws = torch.empty(2 * ks * M * F, dtype=torch.float32, device=h.device)
         _lib.check(L.apc_gemm_splitk_bf16(h.data_ptr(), lda, wg.data.data_ptr(), wu.data.data_ptr(), out.data_ptr(), ldc,
                                           M, F, K, 3, ks, ws.data_ptr(), _ops._stream()), "gemm_splitk_bf16")
@@ -114,21 +121,21 @@ def gemm_emit_bf16(a: torch.Tensor, w: PackedWeight, residual: torch.Tensor, g: 
     """residual += a . w^T, and for the RMS norm with weight g that reads the residual next: the row
     bfloat16(residual * g) and the sums of residual^2 per band of 16 columns and row.  Returns (raw [M, N],
     ss) or None, with nothing done, for sizes no kernel takes.  ss is [16, ceil(N/16) rounded up to 4] from the
-    streaming kernel (up to 16 rows) and [M, ceil(N/256)] from the tiled kernel with K in slices (17..128 rows); the
-    products below take either."""
+    streaming kernel (up to 16 rows) and [M, ceil(N/256)] from the tiled kernel with K in slices (17..1024 rows, where
+    the matrix has so few columns that K is cut); the products below take either."""
     _ops._gpu(a, w.data, residual, g)
     M, K = a.shape
     N = w.N
-    if (M > SPLITK_MAX_ROWS or not _act_ok(a) or residual.dtype != torch.float32 or g.dtype != torch.float32
+    if (M > MANY_ROWS_SPLIT_MAX or not _act_ok(a) or residual.dtype != torch.float32 or g.dtype != torch.float32
             or g.numel() != N or not g.is_contiguous()):
         return None
     if not (w.K == K and residual.shape == (M, N)):
         raise ValueError(f"gemm: a [{M}, {K}], w {w.shape}, residual {tuple(residual.shape)}")
-    raw = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
     if M > SKINNY_MAX_ROWS:   # the tiled kernel with K in slices: sums per row and block of 256 columns
-        ks = _k_split(M, N, K)
+        ks = _tiled_k_split(M, N, K)
         if ks == 1:
             return None
+        raw = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
         ss = torch.empty((M, -(-N // 256)), dtype=torch.float32, device=a.device)
         ws = torch.empty(ks * M * N, dtype=torch.float32, device=a.device)
         L = _lib.load("tuned")
@@ -137,6 +144,7 @@ def gemm_emit_bf16(a: torch.Tensor, w: PackedWeight, residual: torch.Tensor, g: 
                                                g.data_ptr(), raw.data_ptr(), N, ss.data_ptr(), _ops._stream()),
                    "gemm_splitk_emit_bf16")
         return raw, ss
+    raw = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
     ss = torch.empty((16, -(-(-(-N // 16)) // 4) * 4), dtype=torch.float32, device=a.device)
     L = _lib.load("tuned")
     _lib.check(L.apc_skinny_gemm_emit_bf16(a.data_ptr(), _ops._rows(a, "a"), w.data.data_ptr(), residual.data_ptr(),
@@ -150,21 +158,25 @@ def _pre_ok(raw: torch.Tensor, ss: torch.Tensor, K: int) -> bool:
             and tuple(ss.shape) == (16, -(-(-(-K // 16)) // 4) * 4))
 
 
-def _pre_splitk(raw: torch.Tensor, ss: torch.Tensor, eps: float, w, wu, out: torch.Tensor, n_cols: int, mode: int) -> bool:
-    """The same on the tiled kernel with K in slices (17..128 rows): ss is [M, ceil(K / 256)]."""
+def _pre_tiled(raw: torch.Tensor, ss: torch.Tensor, eps: float, w, wu, out: torch.Tensor, n_cols: int, mode: int) -> bool:
+    """The same on the tiled kernel (17..1024 rows), K in slices or in one piece: ss is [M, ceil(K / 256)]."""
     M, K = raw.shape
-    if not (SKINNY_MAX_ROWS < M <= SPLITK_MAX_ROWS and _act_ok(raw) and ss.dtype == torch.float32
+    if not (SKINNY_MAX_ROWS < M <= MANY_ROWS_SPLIT_MAX and _act_ok(raw) and ss.dtype == torch.float32
             and ss.is_contiguous() and tuple(ss.shape) == (M, -(-K // 256)) and ss.shape[1] <= 256):
         return False
-    ks = _k_split(M, n_cols * (2 if wu is not None else 1), K)
-    if ks == 1 and wu is None:
-        return False
-    ws = torch.empty((2 if wu is not None else 1) * ks * M * n_cols, dtype=torch.float32, device=raw.device)
+    n_mats = 2 if wu is not None else 1
+    ks = _tiled_k_split(M, n_cols * n_mats, K)
     L = _lib.load("tuned")
+    wu_ptr = wu.data.data_ptr() if wu is not None else 0
+    if ks == 1:
+        _lib.check(L.apc_gemm_pre_bf16(raw.data_ptr(), _ops._rows(raw, "raw"), ss.data_ptr(), ss.shape[1], float(eps),
+                                       w.data.data_ptr(), wu_ptr, out.data_ptr(), _ops._rows(out, "out"), M, n_cols, K,
+                                       mode, _ops._stream()), "gemm_pre_bf16")
+        return True
+    ws = torch.empty(n_mats * ks * M * n_cols, dtype=torch.float32, device=raw.device)
     _lib.check(L.apc_gemm_splitk_pre_bf16(raw.data_ptr(), _ops._rows(raw, "raw"), ss.data_ptr(), ss.shape[1], float(eps),
-                                          w.data.data_ptr(), wu.data.data_ptr() if wu is not None else 0, out.data_ptr(),
-                                          _ops._rows(out, "out"), M, n_cols, K, mode, ks, ws.data_ptr(), _ops._stream()),
-               "gemm_splitk_pre_bf16")
+                                          w.data.data_ptr(), wu_ptr, out.data_ptr(), _ops._rows(out, "out"), M, n_cols,
+                                          K, mode, ks, ws.data_ptr(), _ops._stream()), "gemm_splitk_pre_bf16")
     return True
 
 
@@ -178,7 +190,7 @@ def gemm_pre_bf16(raw: torch.Tensor, ss: torch.Tensor, eps: float, w: PackedWeig
     if not (w.K == K and out.shape == (M, w.N)):
         raise ValueError(f"gemm: raw [{M}, {K}], w {w.shape}, out {tuple(out.shape)}")
     if M > SKINNY_MAX_ROWS:
-        return _pre_splitk(raw, ss, eps, w, None, out, w.N, 0 if out.dtype == torch.bfloat16 else 1)
+        return _pre_tiled(raw, ss, eps, w, None, out, w.N, 0 if out.dtype == torch.bfloat16 else 1)
     if not _pre_ok(raw, ss, K):
         return False
     L = _lib.load("tuned")
@@ -236,7 +248,7 @@ def swiglu_pre_bf16(raw: torch.Tensor, ss: torch.Tensor, eps: float, wg: PackedW
     if not (wg.shape == (F, K) and wu.shape == (F, K) and out.shape[0] == M):
         raise ValueError(f"swiglu: weights must both be [{F}, {K}]")
     if M > SKINNY_MAX_ROWS:
-        return _pre_splitk(raw, ss, eps, wg, wu, out, F, 3)
+        return _pre_tiled(raw, ss, eps, wg, wu, out, F, 3)
     if not _pre_ok(raw, ss, K):
         return False
     L = _lib.load("tuned")

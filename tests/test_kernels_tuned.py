@@ -193,8 +193,9 @@ def test_swiglu_of_the_normalised_row_from_what_was_left(M, F, K):
     check(f64(out), P.silu(raw64 @ f64(w[:F]).T * rstd) * (raw64 @ f64(w[F:]).T * rstd), BF)
 
 
-@pytest.mark.parametrize("M,D,K", [(40, 520, 1208), (64, 4096, 512), (100, 300, 2056), (17, 256, 520)])
-def test_product_into_the_residual_leaves_the_next_norms_row_with_17_to_128_rows(M, D, K):
+@pytest.mark.parametrize("M,D,K", [(40, 520, 1208), (64, 4096, 512), (100, 300, 2056), (17, 256, 520), (300, 520, 1208),
+                                   (1000, 264, 1024)])
+def test_product_into_the_residual_leaves_the_next_norms_row_with_17_to_1024_rows(M, D, K):
     """The same from the tiled kernel with K in slices: sums of squares per row and block of 256 columns."""
     t = tuned()
     a, w = gen(M, K, seed=1, dtype=BF).to(DEV), gen(D, K, seed=2, dtype=BF).to(DEV)
@@ -215,9 +216,14 @@ def test_product_into_the_residual_leaves_the_next_norms_row_with_17_to_128_rows
     assert (d <= 2.0 ** -7 * np.abs(raw_want) + 1.5e-5 * np.abs(x).max()).all() and (d > 0).mean() < 0.01
 
 
-@pytest.mark.parametrize("M,N,K", [(40, 200, 1208), (64, 6144, 4096), (100, 96, 520), (128, 130, 2048)])
-def test_product_of_the_normalised_row_from_what_was_left_with_17_to_128_rows(M, N, K):
+@pytest.mark.parametrize("M,N,K", [(40, 200, 1208), (64, 6144, 4096), (100, 96, 520), (128, 130, 2048),
+                                   # K in one piece (enough tiles without slices): 224 and 192 tiles; a last row tile of 44
+                                   (64, 28672, 520), (300, 8192, 264), (300, 2048, 1288)])
+def test_product_of_the_normalised_row_from_what_was_left_with_17_to_1024_rows(M, N, K):
+    """On the tiled kernel, with K in slices (the finishing kernel scales) or whole (the product's epilogue does)."""
     t = tuned()
+    whole = t._tiled_k_split(M, N, K) == 1
+    assert whole == ((M, N, K) in [(64, 28672, 520), (300, 8192, 264)])
     x = f64(gen(M, K, seed=1, scale=3.0))
     x[0, : K // 2] *= 40.0
     g = f64(1 + 0.2 * gen(K, seed=2))
