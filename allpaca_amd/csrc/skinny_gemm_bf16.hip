@@ -8,7 +8,7 @@
 //    range of K and reads it in steps of 4 tiles per band: every load of W is 1 KiB of consecutive bytes and a
 //    wave walks forward through one region of memory;
 //  * the activations are the other operand (row m = lane % 16, 16 bytes of k per lane), loaded once per step
-//    for all NB bands: D[n][m], so a lane ends with 4 consecutive n of one row m;
+//    for all NB bands: D[n][m], so a lane ends with 4 consecutive n of one row m (SwiGLU: steps of 2 tiles);
 //  * the loads of the next step are in flight while the current one is multiplied (two register sets that
 //    swap roles; no branch around a load in the steady state);
 //  * the waves' partial sums are added in wave order through LDS, then the epilogue runs: store (bfloat16 or
@@ -31,10 +31,10 @@ constexpr int TILE_ELEMS = 16 * 32;  // elements of a tile
 
 enum { SK_STORE_BF16 = 0, SK_STORE_F32 = 1, SK_ACC_F32 = 2, SK_SWIGLU = 3, SK_QKV_ROPE = 4 };
 
-template <int MT, int NB>
+template <int MT, int NB, int U>
 struct SkRegs {
-  Frag w[NB][SK_U];
-  Frag a[MT][SK_U];
+  Frag w[NB][U];
+  Frag a[MT][U];
 };
 
 // NB: weight bands per block (for SwiGLU: 2 = one gate band and the up band of the same outputs)
@@ -69,8 +69,15 @@ struct SkRope {
   int P, H, Hk, d;
 };
 
+// Tiles per band and step, and blocks that share a compute unit.  SwiGLU on a wide layer has more blocks than
+// compute units and each block streams 2 bands: with steps of 2 tiles a block of 8 waves needs under 128 registers
+// a lane, two blocks share a unit, and one block's first loads and final reduction hide behind the other's stream
+// (8B shapes, 8 rows: 48.0 -> 44.4 us; the bytes in flight per unit stay the same).
+constexpr int sk_step(int mode) { return mode == SK_SWIGLU ? 2 : SK_U; }
+constexpr int sk_blocks(int mode, int wpb) { return (mode == SK_SWIGLU && wpb == 8) ? 2 : 1; }
+
 template <int MT, int MODE, int NB, int WPB, bool PRE, bool EMIT>
-__global__ __launch_bounds__(WPB * 64) void skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda,
+__global__ __launch_bounds__(WPB * 64, sk_blocks(MODE, WPB)) void skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda,
                                                                const bf16_t* __restrict__ W,
                                                                const bf16_t* __restrict__ W2, int chunks,
                                                                void* __restrict__ C, int ldc, int M, int N, int K,
@@ -78,6 +85,7 @@ __global__ __launch_bounds__(WPB * 64) void skinny_gemm_kernel(const bf16_t* __r
   static_assert(MODE != SK_QKV_ROPE || NB == 2, "the two bands of a block hold the two halves of the pairs");
   static_assert(!EMIT || MODE == SK_ACC_F32, "only a product that adds into the residual emits the next norm's row");
   static_assert(!PRE || MODE != SK_ACC_F32, "a product that reads a normalised row stores its result");
+  constexpr int U = sk_step(MODE);
   static_assert(MT == 1, "written for one tile of rows (the finishing wave's early loads, the folded norm)");
   __shared__ float red[WPB * NB * MT * 256];
   __shared__ float row_ss[WPB * MT * 16];
@@ -117,18 +125,18 @@ __global__ __launch_bounds__(WPB * 64) void skinny_gemm_kernel(const bf16_t* __r
   for (int b = 0; b < NB; ++b)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[b][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
-  auto load_step = [&](SkRegs<MT, NB>& r, int ch) {  // tiles ch .. ch+3, all inside K
+  auto load_step = [&](SkRegs<MT, NB, U>& r, int ch) {  // tiles ch .. ch+3, all inside K
 #pragma unroll
-    for (int u = 0; u < SK_U; ++u) {
+    for (int u = 0; u < U; ++u) {
 #pragma unroll
       for (int b = 0; b < NB; ++b) r.w[b][u] = load_frag(wb[b] + (size_t)(ch + u) * TILE_ELEMS);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) r.a[mt][u] = load_frag(arow[mt] + (ch + u) * 32);
     }
   };
-  auto compute = [&](const SkRegs<MT, NB>& r) {
+  auto compute = [&](const SkRegs<MT, NB, U>& r) {
 #pragma unroll
-    for (int u = 0; u < SK_U; ++u)
+    for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -137,15 +145,15 @@ __global__ __launch_bounds__(WPB * 64) void skinny_gemm_kernel(const bf16_t* __r
 
   // this wave's range of tiles along K: [c_lo, c_hi); steps of 4 whole tiles, then single tiles
   const int full_chunks = K / 32;                       // tiles that lie wholly inside K (for the activations)
-  const int per_wave = ((chunks + WPB - 1) / WPB + SK_U - 1) / SK_U * SK_U;
+  const int per_wave = ((chunks + WPB - 1) / WPB + U - 1) / U * U;
   const int c_lo = min(wave * per_wave, chunks), c_hi = min(c_lo + per_wave, chunks);
   const int c_full_hi = min(c_hi, full_chunks);
-  const int nsteps = c_full_hi > c_lo ? (c_full_hi - c_lo) / SK_U : 0;
+  const int nsteps = c_full_hi > c_lo ? (c_full_hi - c_lo) / U : 0;
   // Steps are loaded two ahead (register sets r0, r1 take turns); no branch lies around a load in the steady loop,
   // so the waits for one set never wait for the other.
-  SkRegs<MT, NB> r0, r1;
+  SkRegs<MT, NB, U> r0, r1;
   if (nsteps > 0) load_step(r0, c_lo);
-  if (nsteps > 1) load_step(r1, c_lo + SK_U);
+  if (nsteps > 1) load_step(r1, c_lo + U);
   // Behind the first loads of the stream, and needed only at the end: the sums of x^2 that the emitting product
   // left (PRE; the 4 * WPB (wave, c) pairs of the block take groups of 4 bands in turn, the pieces meet in LDS with
   // the partial sums of the product), and what the finishing wave of an output band adds to (residual, EMIT: g).
@@ -191,21 +199,21 @@ __global__ __launch_bounds__(WPB * 64) void skinny_gemm_kernel(const bf16_t* __r
     int at = c_lo, done = 0;
     while (done + 3 < nsteps) {  // steps done, done+1 are loaded; done+2, done+3 exist
       compute(r0);
-      load_step(r0, at + 2 * SK_U);
+      load_step(r0, at + 2 * U);
       compute(r1);
-      load_step(r1, at + 3 * SK_U);
-      at += 2 * SK_U;
+      load_step(r1, at + 3 * U);
+      at += 2 * U;
       done += 2;
     }
     const int rem = nsteps - done;  // 1..3
     compute(r0);
-    if (rem == 3) load_step(r0, at + 2 * SK_U);
+    if (rem == 3) load_step(r0, at + 2 * U);
     if (rem >= 2) compute(r1);
     if (rem == 3) compute(r0);
   }
   // what is left of the range: single tiles; the last one may be cut by K (K is a multiple of 8, so a lane's
   // 16 bytes of activations are inside or outside as a whole; W is zero beyond K)
-  for (int ch = c_lo + nsteps * SK_U; ch < c_hi; ++ch) {
+  for (int ch = c_lo + nsteps * U; ch < c_hi; ++ch) {
     const bool in = ch * 32 + c * 8 < K;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
