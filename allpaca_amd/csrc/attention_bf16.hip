@@ -1,7 +1,10 @@
 // Attention over the paged cache in bfloat16 on MFMA, float32 softmax.
 //
-//   prefill kernel   a tile of up to 64 consecutive rows of one request x one head; keys in tiles of 64
-//                    through LDS; S = Q K^T and O += P V on v_mfma_f32_16x16x32_bf16; online softmax.
+//   prefill kernels  a tile of up to 64 consecutive rows of one request x one head; keys in tiles of 64
+//                    through LDS; online softmax.  Head sizes up to 128: v_mfma_f32_32x32x16_bf16, a wave takes
+//                    32 rows x half of each tile's keys (attn_prefill32_kernel; 98 us for 2,048 rows of 32 heads
+//                    of 128, 707 TFLOP/s at 32,768 rows).  Larger heads: v_mfma_f32_16x16x32_bf16, 16 rows a wave
+//                    (attn_prefill_kernel, which was 9 % slower at 128).
 //   decode kernel    one row x one kv head (the H/Hk query heads of the group are the 16 rows of the MFMA
 //                    tile, so keys and values are read once per group); each wave is a "part" that covers
 //                    KW consecutive keys straight from global memory; parts are merged by a second kernel
@@ -257,6 +260,238 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   }
 }
 
+// The same tile on v_mfma_f32_32x32x16_bf16, for head sizes up to 128.  The 4 waves are 2 halves of the rows x 2
+// halves of each tile's 64 keys: a wave computes S^T [32 keys x 32 rows] and O^T [d x 32 rows] for its keys only,
+// with a running maximum and sum of its own, and the two waves of a row half merge once at the end through LDS.
+// Against the 16-row kernel above an operand read from LDS feeds twice the arithmetic (LDS bandwidth was what
+// bound that kernel), P goes from the first product's result registers straight into the second product's operand
+// (a lane's 8 results of a 16-key step are keys lh*4+0..3 and 8+lh*4+0..3, lh = lane / 32; V^T lies in LDS with the
+// two middle groups of 4 keys of every 16 swapped, so that the matching 8 values of V are one 16-byte read), and a
+// row's maximum and sum take one exchange between 2 lanes instead of two between 4.
+template <int DP>  // head_dim rounded up to a multiple of 32, at most 128
+__global__ __launch_bounds__(256) void attn_prefill32_kernel(
+    const bf16_t* __restrict__ q, int ldq, int q_off, bf16_t* __restrict__ out, int ldo, int H, int Hk, int d,
+    const bf16_t* __restrict__ cache, int P, const int* __restrict__ block_table, int max_blocks,
+    const int* __restrict__ positions, const int* __restrict__ row_seg, const int* __restrict__ tile_row0,
+    const int* __restrict__ tile_rows, int n_tiles, int window, float scale) {
+  constexpr int KROW = DP + (DP % 128 == 0 ? 72 : DP % 128 == 64 ? 8 : DP % 128 == 32 ? 40 : 104);
+  constexpr int VROW = KT + KPAD;
+  constexpr int DT = DP / 32;  // 32-row tiles of O^T
+  constexpr int LDS_ELEMS = KT * KROW + DP * VROW;
+  static_assert((size_t)LDS_ELEMS * 2 >= (size_t)(2 * DT * 16 * 64 + 2 * 2 * 32) * 4, "the merge needs this much LDS");
+  __shared__ __attribute__((aligned(16))) bf16_t smem[LDS_ELEMS];
+  bf16_t* Ks = smem;
+  bf16_t* Vs = smem + KT * KROW;
+  const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+  const int li = lane % 32, lh = lane / 32;
+  const int rh = wave / 2, kh = wave % 2;  // half of the rows, half of each tile's keys
+  int tile, h;
+  {
+    const int id = blockIdx.x, G = H / Hk;
+    if (Hk % 8 == 0) {  // see attn_prefill_kernel
+      const int xcd = id % 8, slot = id / 8;
+      const int lhd = slot / n_tiles;
+      tile = n_tiles - 1 - slot % n_tiles;
+      h = (xcd + 8 * (lhd / G)) * G + lhd % G;
+    } else {
+      tile = n_tiles - 1 - id % n_tiles;
+      h = id / n_tiles;
+    }
+  }
+  const int row0 = tile_row0[tile], nrows = tile_rows[tile];
+  const int kvh = h / (H / Hk);
+  const int pos0 = positions[row0];
+  const int* bt = block_table + (size_t)row_seg[row0] * max_blocks;
+  const int last = pos0 + nrows - 1;
+  const int first = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const size_t page_stride = (size_t)2 * Hk * P * d;
+  const int dchunks = d / 8;
+
+  for (int idx = tid; idx < LDS_ELEMS; idx += 256) smem[idx] = 0;  // padding columns of K, rows of V beyond d
+
+  // this wave's 32 query rows as the second operand: row = lane % 32, 8 elements of d per lane and step of 16
+  const int my_row = rh * 32 + li;
+  Frag qf[DP / 16];
+  {
+    const bf16_t* qrow = q + (size_t)(row0 + min(my_row, nrows - 1)) * ldq + q_off + (size_t)h * d;
+#pragma unroll
+    for (int ks = 0; ks < DP / 16; ++ks) {
+      const int e = ks * 16 + lh * 8;
+      qf[ks] = (my_row < nrows && e < d) ? load_frag(qrow + e) : zero_frag();
+    }
+  }
+  const int my_pos = pos0 + my_row;
+  const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
+  const int wave_hi = pos0 + rh * 32;  // smallest position of the wave's rows
+  const int wave_top = wave_hi + 31;
+  const int wave_lo = (window > 0 && wave_top - window + 1 > 0) ? wave_top - window + 1 : 0;
+  const float sc2 = scale * LOG2E;
+  floatx16 o[DT];  // O^T: element dt*32 + (r/4)*8 + lh*4 + r%4 of row li
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const bf16_t* krd = Ks + (kh * 32 + li) * KROW + lh * 8;  // key kh*32 + li, d piece lh of a step of 16
+  const bf16_t* vrd = Vs + li * VROW + kh * 32 + lh * 8;    // value row li of a group of 32, this half's columns
+
+  // global -> registers -> LDS as in attn_prefill_kernel; the 8 keys of a group go into V^T's columns as two
+  // pieces of 4 (the column order described above)
+  constexpr int PIECES = DP / 32;
+  const int grp = tid / 32, gl = tid % 32;
+  const int last_group = (last / 8) * 8;
+  int k_ldst[PIECES], v_ldst[PIECES];
+  bool on[PIECES];
+#pragma unroll
+  for (int j = 0; j < PIECES; ++j) {
+    const int idx = gl + 32 * j;
+    on[j] = idx < d;
+    const int key = on[j] ? idx / dchunks : 0, ch = on[j] ? idx % dchunks : 0;
+    k_ldst[j] = (grp * 8 + key) * KROW + ch * 8;
+    v_ldst[j] = (on[j] ? idx : 0) * VROW + (grp / 2) * 16 + (grp % 2) * 4;
+  }
+  const bf16_t* k_head = cache + (size_t)kvh * P * d;
+  const bf16_t* v_head = cache + (size_t)(Hk + kvh) * P * d;
+  int page_next = 0;
+  auto lookup_tile = [&](int t0) { page_next = bt[min(t0 + grp * 8, last_group) / P]; };
+  Frag kreg[PIECES], vreg[PIECES];
+  auto load_tile = [&](int t0) {
+    const int tg = min(t0 + grp * 8, last_group), slot0 = tg % P;
+    const bf16_t* kp = k_head + (size_t)page_next * page_stride + (size_t)slot0 * d;
+    const bf16_t* vp = v_head + (size_t)page_next * page_stride + slot0;
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) {
+      const int idx = on[j] ? gl + 32 * j : 0;
+      kreg[j] = load_frag(kp + idx * 8);
+      vreg[j] = load_frag(vp + (size_t)idx * P);
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) {
+      if (on[j]) {
+        *reinterpret_cast<Frag*>(Ks + k_ldst[j]) = kreg[j];
+        uint2 a, b;
+        a.x = vreg[j].w[0];
+        a.y = vreg[j].w[1];
+        b.x = vreg[j].w[2];
+        b.y = vreg[j].w[3];
+        *reinterpret_cast<uint2*>(Vs + v_ldst[j]) = a;
+        *reinterpret_cast<uint2*>(Vs + v_ldst[j] + 8) = b;
+      }
+    }
+  };
+
+  const int t_begin = (first / KT) * KT;
+  lookup_tile(t_begin);
+  load_tile(t_begin);
+  lookup_tile(t_begin + KT);
+  __syncthreads();
+  store_tile();
+  __syncthreads();
+  for (int t0 = t_begin; t0 <= last; t0 += KT) {
+    load_tile(t0 + KT);
+    lookup_tile(t0 + 2 * KT);
+
+    // S^T: lane holds keys tk + (r/4)*8 + lh*4 + r%4 of row li
+    const int tk = t0 + kh * 32;
+    floatx16 s;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < DP / 16; ++ks) {
+      const Frag kf = *reinterpret_cast<const Frag*>(krd + ks * 16);
+      s = mfma32(kf, qf[ks], s);
+    }
+    float mx = -INFINITY;
+    if (tk >= wave_lo && tk + 31 <= wave_hi) {  // every row of the wave sees all 32 keys
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[r]);
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int t = tk + (r / 4) * 8 + lh * 4 + (r % 4);
+        const float v = (t >= my_lo && t <= my_pos) ? s[r] : -INFINITY;
+        s[r] = v;
+        mx = fmaxf(mx, v);
+      }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE)) * sc2;
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = exp2_neg(m_run - m_safe);
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      s[r] = exp2_neg(fmaf(s[r], sc2, -m_safe));
+      sum += s[r];
+    }
+    l_run = l_run * alpha + (sum + __shfl_xor(sum, 32, WAVE));
+    m_run = m_new;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+    }
+    // O^T += V^T P^T, two steps of 16 keys
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      Frag pf;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) pf.w[w] = bf16_pair(s[8 * j + 2 * w], s[8 * j + 2 * w + 1]);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const Frag vf = *reinterpret_cast<const Frag*>(vrd + dt * 32 * VROW + j * 16);
+        o[dt] = mfma32(vf, pf, o[dt]);
+      }
+    }
+    __syncthreads();
+    store_tile();
+    __syncthreads();
+  }
+
+  // the two key halves of a row half meet: wave kh = 1 leaves its maximum, sum and O^T in LDS, wave kh = 0 adds
+  float* mo = reinterpret_cast<float*>(smem);            // [rh][dt][r][lane]
+  float* ml = mo + 2 * DT * 16 * 64;                     // [rh][m, l][32 rows]
+  if (kh == 1) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mo[((rh * DT + dt) * 16 + r) * 64 + lane] = o[dt][r];
+    if (lh == 0) {
+      ml[(rh * 2 + 0) * 32 + li] = m_run;
+      ml[(rh * 2 + 1) * 32 + li] = l_run;
+    }
+  }
+  __syncthreads();
+  if (kh == 0 && my_row < nrows) {
+    const float m2 = ml[(rh * 2 + 0) * 32 + li], l2 = ml[(rh * 2 + 1) * 32 + li];
+    const float m = fmaxf(m_run, m2);
+    const float m_safe = m == -INFINITY ? 0.f : m;
+    const float a1 = exp2_neg(m_run - m_safe), a2 = exp2_neg(m2 - m_safe);
+    const float inv = 1.0f / (l_run * a1 + l2 * a2);
+    bf16_t* orow = out + (size_t)(row0 + my_row) * ldo + (size_t)h * d;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int e = dt * 32 + g * 8 + lh * 4;
+        if (e < d) {
+          float y[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            y[r] = (o[dt][g * 4 + r] * a1 + mo[((rh * DT + dt) * 16 + g * 4 + r) * 64 + lane] * a2) * inv;
+          uint2 pk;
+          pk.x = bf16_pair(y[0], y[1]);
+          pk.y = bf16_pair(y[2], y[3]);
+          *reinterpret_cast<uint2*>(orow + e) = pk;
+        }
+      }
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------ decode
 // parts[row][head][part][d + 2]: o[0..d), m, l
 template <int DP>
@@ -482,13 +717,18 @@ APC_EXPORT int apc_attention_prefill_bf16(const void* q, int ldq, int q_off, voi
   hipLaunchKernelGGL((attn_prefill_kernel<DP_>), grid, block, 0, stream, (const bf16_t*)q, ldq, q_off, (bf16_t*)out, \
                      ldo, H, Hk, d, (const bf16_t*)cache, page_tokens, block_table, max_blocks, positions, row_seg,  \
                      tile_row0, tile_rows, n_tiles, window, scale)
-  if (d <= 32) PF_LAUNCH(32);
-  else if (d <= 64) PF_LAUNCH(64);
-  else if (d <= 96) PF_LAUNCH(96);
-  else if (d <= 128) PF_LAUNCH(128);
+#define PF32_LAUNCH(DP_)                                                                                             \
+  hipLaunchKernelGGL((attn_prefill32_kernel<DP_>), grid, block, 0, stream, (const bf16_t*)q, ldq, q_off, (bf16_t*)out, \
+                     ldo, H, Hk, d, (const bf16_t*)cache, page_tokens, block_table, max_blocks, positions, row_seg,    \
+                     tile_row0, tile_rows, n_tiles, window, scale)
+  if (d <= 32) PF32_LAUNCH(32);
+  else if (d <= 64) PF32_LAUNCH(64);
+  else if (d <= 96) PF32_LAUNCH(96);
+  else if (d <= 128) PF32_LAUNCH(128);
   else if (d <= 192) PF_LAUNCH(192);
   else PF_LAUNCH(256);
 #undef PF_LAUNCH
+#undef PF32_LAUNCH
   APC_LAUNCH_CHECK();
   return 0;
 }

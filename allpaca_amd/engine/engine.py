@@ -4,7 +4,7 @@ the scheduler and the sampler, and offers the reference's calls
 crates/allpaca-core/src/engine.rs:2895, 3002, 3167, 3650, 3661)."""
 from __future__ import annotations
 
-import os
+import shutil
 import tempfile
 import time
 from typing import Dict, Iterator, List, Mapping, Optional, Sequence
@@ -40,13 +40,15 @@ class Engine:
         cfg.validate()
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU is visible; the engine has no CPU path")
-        self.config = cfg
-        dtype = _DTYPES[cfg.dtype]
         num_pages = cfg.num_pages or -(-cfg.max_tokens // cfg.page_tokens)
-        self.model_config, self.model = load_model(model, dtype, cfg.device,
-                                                   max_positions=num_pages * cfg.page_tokens)
-        self.runner = ModelRunner(self.model, cfg.page_tokens, num_pages, cfg.max_active_requests,
-                                  use_graphs=cfg.use_graphs)
+        model_config, bound = load_model(model, _DTYPES[cfg.dtype], cfg.device, max_positions=num_pages * cfg.page_tokens)
+        self._assemble(model_config, bound, cfg)
+
+    def _assemble(self, model_config, model, cfg: EngineConfig) -> None:
+        """Runner, scheduler and sampler around a model that is bound to its weights."""
+        self.config, self.model_config, self.model = cfg, model_config, model
+        num_pages = cfg.num_pages or -(-cfg.max_tokens // cfg.page_tokens)
+        self.runner = ModelRunner(model, cfg.page_tokens, num_pages, cfg.max_active_requests, use_graphs=cfg.use_graphs)
         self.scheduler = Scheduler(self.runner.cache, cfg.max_active_requests, cfg.max_batch_tokens, cfg.chunk_tokens)
         self.sampler = Sampler(self.runner.rt.device, cfg.seed)
         self.requests: Dict[int, Request] = {}
@@ -55,14 +57,26 @@ class Engine:
         self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0}
 
     @classmethod
+    def from_model(cls, model_config, model, config: EngineConfig) -> "Engine":
+        """An engine around a `DecoderModel` that the caller has built and bound to weights on the GPU (weights made
+        in place, without a model folder)."""
+        config.validate()
+        eng = cls.__new__(cls)
+        eng._assemble(model_config, model, config)
+        return eng
+
+    @classmethod
     def synthetic(cls, config_json: Mapping, seed: int = 0, config: Optional[EngineConfig] = None, **options) -> "Engine":
-        """An engine on random weights: the model folder is written to a temporary place first
-        (the reference's `--synthetic`, crates/allpaca-core/src/engine.rs:1577-1586)."""
+        """An engine on random weights: the model folder is written to a temporary place first and removed once
+        the weights are on the GPU (the reference's `--synthetic`, crates/allpaca-core/src/engine.rs:1577-1586)."""
         from ..weights import write_model_folder
         dtype = _DTYPES[(config.dtype if config else options.get("dtype", EngineConfig().dtype))]
         folder = tempfile.mkdtemp(prefix="allpaca_amd_synthetic_")
-        write_model_folder(folder, config_json, seed, dtype)
-        return cls(folder, config, **options)
+        try:
+            write_model_folder(folder, config_json, seed, dtype)
+            return cls(folder, config, **options)
+        finally:
+            shutil.rmtree(folder, ignore_errors=True)
 
     # ---- requests ------------------------------------------------------------
     def warm_up(self, max_context: Optional[int] = None) -> int:

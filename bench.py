@@ -30,14 +30,10 @@ def build_engine(cfg_json, dtype, batch, context, extra_tokens, layers, seed=0, 
     """An engine on random weights made directly on the GPU (no model folder is written for 16 GB)."""
     import torch
 
-    from allpaca_amd.cache import CacheManager  # noqa: F401
     from allpaca_amd.config import EngineConfig
     from allpaca_amd.engine.engine import Engine
-    from allpaca_amd.engine.runner import ModelRunner
-    from allpaca_amd.engine.scheduler import Scheduler
     from allpaca_amd.models import DecoderModel, describe_model
     from allpaca_amd.parts import Runtime
-    from allpaca_amd.sampling.sampler import Sampler
     from allpaca_amd.weights import random_tensors
 
     cfg_json = dict(cfg_json, num_hidden_layers=layers)
@@ -58,13 +54,7 @@ def build_engine(cfg_json, dtype, batch, context, extra_tokens, layers, seed=0, 
         tensors.update(random_tensors({name: ps}, seed, tdt, 0.02, 0.0, device="cuda:0"))
     model.bind(tensors, rt)
     del tensors
-    eng = Engine.__new__(Engine)
-    eng.config, eng.model_config, eng.model = ec, cfg, model
-    eng.runner = ModelRunner(model, ec.page_tokens, ec.num_pages, ec.max_active_requests, use_graphs=use_graphs)
-    eng.scheduler = Scheduler(eng.runner.cache, ec.max_active_requests, ec.max_batch_tokens, ec.chunk_tokens)
-    eng.sampler = Sampler(rt.device, ec.seed)
-    eng.requests, eng._next_id, eng._prepared = {}, 0, None
-    eng.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0}
+    eng = Engine.from_model(cfg, model, ec)
     return cfg, eng
 
 
