@@ -10,8 +10,12 @@ Every step, under a budget of `max_batch_tokens`:
 A portion may have any size >= 1.  When a decoding request cannot get the page
 its next token needs, the most recently admitted running request is preempted:
 its pages go back, and it returns to the front of the waiting queue to be
-recomputed from its prompt and the tokens it has generated.  A request that
-could never fit the pool is refused when it is added.
+recomputed from its prompt and the tokens it has generated.  The same happens
+when no running request can advance at all (every one is in its prompt and waits
+for a page that only another one's end would free): the most recently admitted
+gives way until someone can go on, so some request advances in every step, the
+one admitted first never loses what it has computed, and the engine cannot stall.  A request that could never fit the pool
+is refused when it is added.
 
 The reference advances one request per tick (`pick_runnable`, longest wait first,
 crates/allpaca-core/src/scheduler.rs:607-664) by `prefill.chunk_tokens`
@@ -155,7 +159,17 @@ class Scheduler:
         plan.preempted.append(victim)
 
     def plan(self) -> Plan:
-        plan = Plan()
+        plan = self._plan_once(Plan())
+        while not plan.scheduled and len(self.running) > 1:
+            # Nobody can advance: the requests in their prompts hold all pages between them.  The newest gives its
+            # pages back (it is not admitted again in this step), until the oldest can go on.
+            self._preempt(max(self.running, key=lambda r: r.order), plan)
+            plan = self._plan_once(plan)
+        return plan
+
+    def _plan_once(self, plan: Plan) -> Plan:
+        """Fills `plan.scheduled` (from nothing); what `plan` lists as preempted and admitted so far stays."""
+        plan.scheduled = []
         budget = self.budget
         promised = [0] * len(self.cache.paged_groups)
         # 1. decodes, oldest admission first.  If a page is missing, the newest running request that is not

@@ -300,6 +300,58 @@ def test_the_newest_request_preempts_itself():
     assert [r.id for r in p.preempted] == [1] and [e.request.id for e in p.scheduled] == [0]
 
 
+def test_prompts_that_hold_all_pages_between_them_do_not_stall():
+    """Two requests in their prompts hold the whole pool and each waits for a page: the newest gives way."""
+    cm, s = sched(num_pages=4, page_tokens=4, max_active=4, budget=8, chunk=4)
+    a, b = req(0, 12, max_tokens=2), req(1, 12, max_tokens=2)
+    s.add(a)
+    s.add(b)
+    run_step(cm, s)
+    p = run_step(cm, s)
+    assert [(e.request.id, e.count) for e in p.scheduled] == [(0, 4), (1, 4)] and cm.free_pages() == 0
+    p = run_step(cm, s)                  # neither can take a third page
+    assert [r.id for r in p.preempted] == [1] and [(e.request.id, e.count) for e in p.scheduled] == [(0, 4)]
+    assert b.status == "waiting" and b.computed == 0 and s.waiting[0] is b
+    for _ in range(40):
+        if not s.has_work():
+            break
+        run_step(cm, s)
+    assert a.finish_reason == b.finish_reason == "length" and len(a.output) == len(b.output) == 2
+    assert cm.free_pages() == 4
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_streams_of_requests_always_finish(seed):
+    """Whatever the pool, the budget and the order of arrival: some request advances in every step, the one
+    admitted first is never the one that gives way, so every request ends, with all its tokens, and every page comes
+    back."""
+    rng = np.random.default_rng(seed)
+    page = int(rng.choice([4, 8, 16]))
+    n_req = int(rng.integers(2, 10))
+    prompts = [int(rng.integers(1, 50)) for _ in range(n_req)]
+    new = [int(rng.integers(1, 20)) for _ in range(n_req)]
+    biggest = max(p + n for p, n in zip(prompts, new))
+    num_pages = -(-biggest // page) + int(rng.integers(0, 4)) * int(rng.integers(1, 4))
+    max_active = int(rng.integers(1, 7))
+    cm = CacheManager([FULL], page, num_pages, max_requests=max_active)
+    s = Scheduler(cm, max_active, int(rng.integers(4, 65)), int(rng.integers(2, 33)))
+    arrive = sorted(int(rng.integers(0, 25)) for _ in range(n_req))
+    reqs, steps = [], 0
+    while len(reqs) < n_req or s.has_work():
+        while len(reqs) < n_req and arrive[len(reqs)] <= steps:
+            reqs.append(req(len(reqs), prompts[len(reqs)], max_tokens=new[len(reqs)]))
+            s.add(reqs[-1])
+        had_work = s.has_work()
+        oldest = min(s.running, key=lambda r: r.order) if len(s.running) > 1 else None
+        plan = run_step(cm, s)
+        assert plan.scheduled or not had_work, "a step in which nobody advanced"
+        assert oldest not in plan.preempted
+        steps += 1
+        assert steps < 2000
+    assert all(len(r.output) == n and r.finish_reason == "length" for r, n in zip(reqs, new))
+    assert cm.free_pages() == num_pages and not cm.live()
+
+
 def test_a_request_larger_than_the_pool_is_refused():
     cm, s = sched(num_pages=4, page_tokens=4)
     with pytest.raises(RequestTooLarge, match="whole pool"):
