@@ -184,3 +184,57 @@ def test_a_far_key_is_found(dtype):
     without = list(toks)
     without[19] = 8  # no marked token: the logits at the end are far from the ones found above
     assert np.abs(H.oracle_logits(path, without)[-1] - want[-1]).max() > 0.1
+
+
+def test_widths_of_an_8b_model_in_bfloat16_against_the_32_bit_path():
+    """The tiny configurations do not reach the code paths that sizes choose (bands per block, waves per block,
+    K in slices or whole, the fused product for q, k, v with d = 128): two layers at the widths of an 8B model
+    (hidden 4096, 32 heads over 8 of 128, feed-forward 14336; a small vocabulary), weights made on the GPU, the
+    same bfloat16 values in both runs.  A whole portion, a mixed step, decode steps (replayed graphs) and a portion
+    behind them: every row's logits are within the storage noise of two layers of the 32-bit path's, and no path
+    is further off than the others."""
+    from allpaca_amd.config import preset
+    from allpaca_amd.engine.batch import Entry
+    from allpaca_amd.engine.runner import ModelRunner
+    from allpaca_amd.models import DecoderModel, describe_model
+    from allpaca_amd.parts import Runtime
+    from allpaca_amd.weights import random_tensors
+    V = 8200
+    cfg_json = dict(preset("llama-3.1-8b"), num_hidden_layers=2, vocab_size=V)
+    sharpen = (3.0 / (0.02 ** 2 * cfg_json["hidden_size"])) ** 0.5      # scores of deviation ~3, as in helpers.model_folder
+
+    def runner(dtype):
+        _, _, spec = describe_model(cfg_json)
+        model = DecoderModel(spec)
+        tensors = {}
+        for name, ps in model.param_specs().items():
+            for k, v in random_tensors({name: ps}, 0, torch.bfloat16, 0.02, 0.0, device="cuda:0").items():
+                if k.endswith("q_proj.weight") or k.endswith("k_proj.weight"):
+                    v = (v.float() * sharpen).to(torch.bfloat16)
+                tensors[k] = v if dtype == torch.bfloat16 else v.float()
+        model.bind(tensors, Runtime(torch.device("cuda:0"), dtype, 1024))
+        return ModelRunner(model, 16, 128, 8, use_graphs=True)
+
+    toks = H.random_tokens(V, 420, seed=5)
+    rows = {}
+    for dtype in (torch.float32, torch.bfloat16):
+        r = runner(dtype)
+        r.admit("a")
+        r.admit("b")
+        out = [("whole portion", r.step([Entry("a", toks[:300], list(range(300)))]))]
+        out.append(("mixed step", r.step([Entry("a", toks[300:340], list(range(40))), Entry("b", toks[:17], list(range(17)))])))
+        for j in range(6):
+            out.append(("decode step", r.step([Entry("a", [toks[340 + j]], [0]), Entry("b", [toks[17 + j]], [0])])))
+        out.append(("portion behind", r.step([Entry("a", toks[346:400], [0, 53]), Entry("b", toks[23:24], [0])])))
+        assert r.graph_replays == 6
+        rows[dtype] = [(what, lg.float().cpu().numpy().astype(np.float64)) for what, lg in out]
+        del r
+        torch.cuda.empty_cache()
+    errs = []
+    for (what, a), (_, b) in zip(rows[torch.float32], rows[torch.bfloat16]):
+        e = np.sqrt(((a - b) ** 2).mean(axis=1)) / np.sqrt((a ** 2).mean(axis=1))
+        errs.append((what, float(e.max()), float(e.mean())))
+    # measured: 0.016 on average, 0.021 at most, the same on every path
+    worst = max(e for _, e, _ in errs)
+    mean = float(np.mean([m for _, _, m in errs]))
+    assert worst < 0.03 and worst < 2.0 * mean, errs
