@@ -21,8 +21,8 @@
 #include "mfma.h"
 
 constexpr int BN = 128, BK = 64;
-// Rows of the block tile.  The kernel also builds with 256 (4 x 2 accumulators a wave, one block a compute unit);
-// on the shapes of an 8B model with 2,048 rows that was no faster than two 128-row blocks sharing a unit.
+// Rows of the block tile (the split path also uses 64).  256 rows (4 x 2 accumulators a wave, one block a compute
+// unit) were tried on the shapes of an 8B model with 2,048 rows: no faster than two 128-row blocks sharing a unit.
 constexpr int BM_ROWS = 128;
 constexpr int LDS_ROW = BK + 8;  // bfloat16 elements per LDS row (144 bytes)
 
@@ -42,7 +42,7 @@ struct TiledPre {
   float eps;
 };
 
-// EVEN_K: K is a multiple of 64, so no load needs a bound check.  BM: rows of the block tile, 128 or 256.
+// EVEN_K: K is a multiple of 64, so no load needs a bound check.  BM: rows of the block tile, 64 or 128.
 template <int MODE, bool EVEN_K, int BM, bool PRE = false>
 __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda,
                                                         const bf16_t* __restrict__ W,
