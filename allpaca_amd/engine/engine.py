@@ -22,11 +22,13 @@ from .scheduler import FINISHED, RUNNING, Request, Scheduled, Scheduler
 _DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
 
-class _PreparedStep:
-    """A decode step whose plan and batch description are ready; the tokens are still being sampled."""
+class _AheadStep:
+    """A decode step that already runs on the GPU, model and sampling, fed with the tokens of the step before on the
+    GPU itself; the host has not seen either step's tokens yet.  `dead`: requests that ended (a stop token, an
+    abort) after it was queued: their rows are ignored."""
 
-    def __init__(self, handle, scheduled):
-        self.handle, self.scheduled = handle, scheduled
+    def __init__(self, scheduled, pending):
+        self.scheduled, self.pending, self.dead = scheduled, pending, set()
 
 
 class Engine:
@@ -52,7 +54,7 @@ class Engine:
         self.scheduler = Scheduler(self.runner.cache, cfg.max_active_requests, cfg.max_batch_tokens, cfg.chunk_tokens)
         self.sampler = Sampler(self.runner.rt.device, cfg.seed)
         self.requests: Dict[int, Request] = {}
-        self._prepared: Optional[_PreparedStep] = None
+        self._ahead: Optional[_AheadStep] = None
         self._next_id = 0
         self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0}
 
@@ -103,7 +105,8 @@ class Engine:
     begin_request = add_request
 
     def abort(self, request_id: int) -> None:
-        self._prepared = None
+        if self._ahead is not None:
+            self._ahead.dead.add(request_id)
         req = self.requests.pop(request_id, None)
         if req is not None and req.status != FINISHED:
             self.scheduler.abort(req)
@@ -113,14 +116,14 @@ class Engine:
 
     # ---- one tick ---------------------------------------------------------------
     def step(self) -> List[TokenEvent]:
-        """One batch through the model: every decoding request advances by a token, prompts by a portion."""
-        prepared, self._prepared = self._prepared, None
-        if prepared is not None and self.scheduler.waiting:
-            prepared = None     # a request arrived: the scheduler decides (what was reserved stays with its requests)
-        if prepared is not None:
-            # the step was planned and set up while the GPU worked on the one before: only the tokens were missing
-            scheduled = prepared.scheduled
-            logits = self.runner.run_prepared(prepared.handle, [s.request.token_slice(s.start, 1)[0] for s in scheduled])
+        """One batch through the model: every decoding request advances by a token, prompts by a portion.
+        While nothing but decoding goes on, the step after this one is queued on the GPU before this one's tokens
+        have reached the host (`_launch_ahead`): the GPU goes from step to step without waiting for the host, and
+        the host reads each step's tokens while the next one runs."""
+        ahead, self._ahead = self._ahead, None
+        if ahead is not None:
+            scheduled = [s for s in ahead.scheduled if s.request.id not in ahead.dead]
+            sampled_all, pending = ahead.scheduled, ahead.pending
         else:
             plan = self.scheduler.plan()
             self.stats["preemptions"] += len(plan.preempted)
@@ -137,43 +140,61 @@ class Engine:
                 toks = s.request.token_slice(s.start, s.count)
                 entries.append(Entry(s.request.id, toks, [s.count - 1] if s.samples else []))
             logits = self.runner.step(entries)
-        sampled = [s for s in scheduled if s.samples]
+            sampled_all = [s for s in scheduled if s.samples]
+            pending = self._launch_sampling(logits, sampled_all, 0) if sampled_all else None
         for s in scheduled:
             self.scheduler.advance(s)
             self.stats["decode_tokens" if s.request.output and s.count == 1 else "prefill_tokens"] += s.count
         self.stats["steps"] += 1
         events: List[TokenEvent] = []
-        if sampled:
-            pending = self.sampler.launch(logits, [s.request.params for s in sampled],
-                                          [len(s.request.output) for s in sampled])
-            self._prepared = self._prepare_next(scheduled)   # host work for the next step while the GPU runs this one
+        if pending is not None:
+            if ahead is None or not ahead.dead:
+                self._ahead = self._launch_ahead(scheduled, sampled_all, pending)
             tokens = pending.wait()
             now = time.perf_counter()       # the token ids are on the host: the step is over
-            for s, tok in zip(sampled, tokens):
+            for s, tok in zip(sampled_all, tokens):
+                if ahead is not None and s.request.id in ahead.dead:
+                    continue
                 s.request.t_tokens.append(now)
                 reason = self.scheduler.append_token(s.request, tok)
                 events.append(TokenEvent(s.request.id, int(tok), reason, len(s.request.prompt)))
                 if reason is not None:
                     self.scheduler.finish(s.request, reason)
-                    self._prepared = None   # the next step is not the one that was prepared
+                    if self._ahead is not None:
+                        self._ahead.dead.add(s.request.id)    # its row of the queued step counts for nothing
+            if self._ahead is not None and all(s.request.id in self._ahead.dead for s in self._ahead.scheduled):
+                self._ahead = None
         return events
 
-    def _prepare_next(self, scheduled) -> Optional["_PreparedStep"]:
-        """If the next step is sure to be one more token for exactly the requests that run now (nothing waits, every
-        running request samples a token in this step and none reaches its `max_tokens` with it), its plan and the
-        runner's first half of it are made now.  A stop token or an abort cancels it."""
+    def _launch_sampling(self, logits, sampled, extra: int):
+        """Queues the choice of a token for every row; `extra`: tokens of each request that are on their way and
+        not appended yet (they count for the index of the random number)."""
+        return self.sampler.launch(logits, [s.request.params for s in sampled],
+                                   [len(s.request.output) + extra for s in sampled])
+
+    def _launch_ahead(self, scheduled, sampled, pending) -> Optional["_AheadStep"]:
+        """If the next step is sure to be one more token for exactly the requests of this one (nothing waits, every
+        running request samples a token in this step, in the order decode steps have, and none reaches its
+        `max_tokens` with it), it is queued now: pages reserved, positions and tables filled in, the tokens copied
+        from this step's sampling result on the GPU, model and sampling launched.  A request that ends with this
+        step's token (a stop id) has a row in the queued step that is ignored; its pages go back as always, and
+        whatever later gets them is queued behind that row's write."""
         sch = self.scheduler
-        if sch.waiting or len(scheduled) != len(sch.running):
+        if sch.waiting or len(scheduled) != len(sch.running) or len(sampled) != len(scheduled):
             return None
         for s in scheduled:
             r = s.request
             if not s.samples or r.status != RUNNING or len(r.output) + 1 >= r.params.max_tokens:
                 return None
         order = sorted((s.request for s in scheduled), key=lambda r: r.order)   # as the scheduler orders decodes
+        if [r.id for r in order] != [s.request.id for s in sampled]:
+            return None     # the sampled rows lie in another order (a prompt ended in this step): the next step will do
         handle = self.runner.prepare_decode([r.id for r in order])
         if handle is None:
             return None
-        return _PreparedStep(handle, [Scheduled(r, r.computed, 1, True) for r in order])
+        logits = self.runner.run_fed(handle, pending.device)
+        nxt = [Scheduled(r, r.computed, 1, True) for r in order]
+        return _AheadStep(nxt, self._launch_sampling(logits, nxt, 1))
 
     poll = step
 

@@ -211,6 +211,23 @@ class ModelRunner:
         return logits
 
 
+    def run_fed(self, prepared: "PreparedDecode", device_tokens: torch.Tensor) -> torch.Tensor:
+        """The second half with tokens that are still on the GPU (int32, one per request, in the order of the
+        prepared requests: what the sampling kernel of the step before wrote).  They are copied into the step's
+        description on the GPU, so the step can be queued before the host has seen them."""
+        g, n = prepared.graph, len(prepared.seqs)
+        if device_tokens.dtype != torch.int32 or device_tokens.numel() < n or device_tokens.device != g.dev.device:
+            raise StepError("tokens fed on the GPU must be int32, one per prepared request, on the engine's device")
+        g.upload()
+        g.dev[:n].copy_(device_tokens[:n])      # the tokens' place in the description (`DecodeGraph._part(0)`)
+        g.replay()
+        self.graph_replays += 1
+        for s in prepared.seqs:
+            self.cache.commit(s, 1)
+        self.steps += 1
+        return g.logits[:n]
+
+
 class PreparedDecode:
     def __init__(self, graph: "DecodeGraph", seqs: List[Hashable]):
         self.graph, self.seqs = graph, seqs

@@ -37,7 +37,8 @@ class Sampler:
     def __init__(self, device: torch.device, default_seed: int):
         self.device = device
         self.default_seed = default_seed
-        self._pinned = None   # token ids come back through pinned memory (one copy in flight at a time)
+        self._pinned = [None, None]   # token ids come back through pinned memory; two results may be under way
+        self._turn = 0
 
     def sample(self, logits: torch.Tensor, params: Sequence[GenerationParams], indices: Sequence[int]) -> List[int]:
         """logits: float32 [R, V] on the GPU; params[r] and indices[r] (how many tokens row r's request
@@ -62,19 +63,21 @@ class Sampler:
             f = torch.from_numpy(host).to(self.device)
             k = torch.from_numpy(ks).to(self.device)
             ops.sample_rows(logits, f[0], k, f[1], f[2], out)
-        if self._pinned is None or self._pinned.numel() < R:
-            self._pinned = torch.empty(max(R, 64), dtype=torch.int32).pin_memory()
-        self._pinned[:R].copy_(out, non_blocking=True)
+        self._turn ^= 1
+        if self._pinned[self._turn] is None or self._pinned[self._turn].numel() < R:
+            self._pinned[self._turn] = torch.empty(max(R, 64), dtype=torch.int32).pin_memory()
+        pinned = self._pinned[self._turn]
+        pinned[:R].copy_(out, non_blocking=True)
         done = torch.cuda.Event()
         done.record()
-        return Pending(self._pinned, R, done)
+        return Pending(pinned, R, done, out)
 
 
 class Pending:
-    """Token ids on their way to the host."""
+    """Token ids on their way to the host; `device` holds them on the GPU (int32 [n])."""
 
-    def __init__(self, pinned: torch.Tensor, n: int, done: torch.cuda.Event):
-        self.pinned, self.n, self.done = pinned, n, done
+    def __init__(self, pinned: torch.Tensor, n: int, done: torch.cuda.Event, device: torch.Tensor):
+        self.pinned, self.n, self.done, self.device = pinned, n, done, device
 
     def wait(self) -> List[int]:
         self.done.synchronize()

@@ -85,6 +85,22 @@ def test_same_seed_same_tokens_under_any_batching_and_stop_ids():
     assert out.token_ids == solo[1][: first + 1] and out.finish_reason == "stop"   # the stop token is emitted
 
 
+def test_sampled_tokens_are_the_same_with_steps_queued_ahead():
+    """With graphs the engine queues a step before the tokens of the one before have reached the host; the index
+    of a request's random number then counts the token that is still on its way."""
+    folder = H.model_folder("B", "float32", True)
+    prompts = [H.random_tokens(1000, n, seed=90 + n) for n in (3, 40, 12, 25)]
+    pr = [params(max_tokens=20, temperature=0.9, top_k=0, top_p=1.0, seed=3),
+          params(max_tokens=14, temperature=0.0),
+          params(max_tokens=20, temperature=0.7, top_k=5, seed=11),
+          params(max_tokens=9, temperature=1.3, top_k=0, top_p=0.6, seed=5)]
+    eager = engine_for(folder).generate(prompts, pr)
+    eng = engine_for(folder, use_graphs=True)
+    queued = eng.generate(prompts, pr)
+    assert [o.token_ids for o in queued] == [o.token_ids for o in eager]
+    assert eng.runner.graph_replays > 10
+
+
 def test_preemption_gives_the_same_tokens():
     folder = H.model_folder("A", "float32", True)
     prompts = [H.random_tokens(256, n, seed=70 + n) for n in (30, 25, 28)]
@@ -276,10 +292,11 @@ def test_graphs_captured_before_serving_are_the_ones_generation_asks_for():
     assert engine_for(folder, use_graphs=False).warm_up() == 0
 
 
-def test_steps_prepared_ahead_give_the_same_tokens_when_requests_stop_arrive_and_are_aborted():
-    """With graphs on, the engine sets up the next decode step while the GPU works on the current one.  A stop token,
-    a request that arrives between two steps and an abort each cancel what was set up; the tokens are those of the
-    plain implementation all the same."""
+def test_steps_queued_ahead_give_the_same_tokens_when_requests_stop_arrive_and_are_aborted():
+    """With graphs on, the engine queues the next decode step on the GPU, fed with the sampled tokens there, before
+    the host has seen the current step's tokens.  A request that stops or is aborted leaves a row in the queued step
+    that counts for nothing, one that arrives waits for the queued step; the tokens are those of the plain
+    implementation all the same."""
     folder = H.model_folder("A", "float32", True)
     cfg, w = H.oracle(folder)
     prompts = [H.random_tokens(256, n, seed=40 + n) for n in (5, 9, 3, 12)]
@@ -291,16 +308,16 @@ def test_steps_prepared_ahead_give_the_same_tokens_when_requests_stop_arrive_and
     r0 = eng.add_request(prompts[0], params(max_tokens=24, temperature=0.0, stop_token_ids=[stop]))
     r1 = eng.add_request(prompts[1], params(max_tokens=24, temperature=0.0))
     got = {r0: [], r1: []}
-    used_prepared = 0
+    queued_ahead = 0
     steps = 0
     r2 = r3 = None
     while eng.has_unfinished():
-        used_prepared += eng._prepared is not None
+        queued_ahead += eng._ahead is not None
         for ev in eng.step():
             got.setdefault(ev.request_id, []).append(ev.token_id)
         steps += 1
-        if steps == 6:                                   # arrives while a prepared step exists
-            assert eng._prepared is not None
+        if steps == 6:                                   # arrives while a queued step exists
+            assert eng._ahead is not None
             r2 = eng.add_request(prompts[2], params(max_tokens=24, temperature=0.0))
             got[r2] = []
         if steps == 12:
@@ -308,7 +325,7 @@ def test_steps_prepared_ahead_give_the_same_tokens_when_requests_stop_arrive_and
             got[r3] = []
         if steps == 16:
             eng.abort(r3)                                # leaves mid-way
-    assert used_prepared > 10
+    assert queued_ahead > 10
     assert got[r0] == cut0 and got[r1] == full[1] and got[r2] == full[2]
     assert got[r3] == full[3][: len(got[r3])] and 0 < len(got[r3]) < 24
     assert eng.runner.cache.free_pages(0) == eng.runner.cache.paged_groups[0].pool.num_pages
