@@ -43,6 +43,7 @@ __device__ __forceinline__ uint32_t bf16_pair(float a, float b) { return pack_bf
 // 2^x for x <= 0 (or -inf): the bare instruction, without the range handling that large arguments need
 __device__ __forceinline__ float exp2_neg(float x) { return __builtin_amdgcn_exp2f(x); }
 constexpr float LOG2E = 1.4426950408889634f;
+constexpr float RISE = 8.f;  // by how much (in powers of 2) a score may exceed the running reference in attn_prefill32_kernel
 
 // ------------------------------------------------------------------------------------------ prefill
 // A block of 4 waves works on up to 64 consecutive rows of one request and one head, 16 rows a wave.
@@ -417,7 +418,10 @@ __global__ __launch_bounds__(256) void attn_prefill32_kernel(
       }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE)) * sc2;
-    const float m_new = fmaxf(m_run, mx);
+    // The running maximum is only a reference point for the exponents: it moves up when a tile's maximum exceeds it
+    // by more than RISE (then O and the sum shrink by 2^-(the move)), and stays otherwise, so that P reaches at most
+    // 2^RISE and O is rescaled on a row's first tiles only.  The result O / sum does not depend on the reference.
+    const float m_new = mx > m_run + RISE ? mx : m_run;
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
     const float alpha = exp2_neg(m_run - m_safe);
     float sum = 0.f;
