@@ -121,7 +121,8 @@ def build(name: str, force: bool = False, verbose: bool = True) -> str:
         threading.Thread(target=ticker, daemon=True).start()
 
     def compile_one(src: str) -> str:
-        obj = os.path.join(d, f"{name}_{os.path.splitext(os.path.basename(src))[0]}.o")
+        # names of this process only: two processes may build the same library into the same folder at once
+        obj = os.path.join(d, f"{name}_{os.path.splitext(os.path.basename(src))[0]}.{os.getpid()}.o")
         cmd = [hipcc, *FLAGS, "-I", CSRC, "-c", src, "-o", obj]
         p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         if p.returncode != 0:
@@ -130,6 +131,7 @@ def build(name: str, force: bool = False, verbose: bool = True) -> str:
             _say(f"compiled {os.path.basename(src)} ({time.time() - t0:.0f} s)")
         return obj
 
+    objs: List[str] = []
     try:
         workers = max(1, min(len(srcs), os.cpu_count() or 1, 8))
         with ThreadPoolExecutor(workers) as ex:
@@ -141,10 +143,16 @@ def build(name: str, force: bool = False, verbose: bool = True) -> str:
         if p.returncode != 0:
             raise KernelBuildError(f"link of {out} failed:\n{p.stdout}")
         os.replace(tmp, out)
-        with open(os.path.join(d, f"{name}.hash"), "w") as f:
+        stamp = os.path.join(d, f"{name}.hash")
+        with open(stamp + f".tmp{os.getpid()}", "w") as f:
             f.write(source_hash(name))
+        os.replace(stamp + f".tmp{os.getpid()}", stamp)
     finally:
         done.set()
+        for src in srcs:
+            obj = os.path.join(d, f"{name}_{os.path.splitext(os.path.basename(src))[0]}.{os.getpid()}.o")
+            if os.path.isfile(obj):
+                os.remove(obj)
     if verbose:
         _say(f"library '{name}' ready in {time.time() - t0:.0f} s")
     return out
