@@ -263,7 +263,7 @@ def test_a_waiting_prompt_waits_for_pages():
 def reqs_status(s):
     out = {r.id: r.status for r in s.running}
     out.update({r.id: r.status for r in s.waiting})
-    return out | {}
+    return out
 
 
 def test_preemption_when_a_decode_needs_a_page():

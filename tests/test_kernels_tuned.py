@@ -32,7 +32,6 @@ def test_packing_roundtrip_and_lane_order():
     p = pack_mfma(w)
     assert tuple(p.data.shape) == (4, 3, 64, 8) and torch.equal(unpack_mfma(p), w)
     i, c = 5, 3          # lane c*16 + i of tile (band 1, chunk 2) holds w[16 + i, 64 + 8c : 64 + 8c + 8]
-    assert torch.equal(p.data[1, 2, c * 16 + i], w[16 + i, 64 + c * 8: 72]) if False else True
     wide = torch.zeros(64, 96, dtype=BF)
     wide[:50, :72] = w
     assert torch.equal(p.data[1, 2, c * 16 + i], wide[16 + i, 64 + c * 8: 64 + c * 8 + 8])
