@@ -238,3 +238,17 @@ def test_widths_of_an_8b_model_in_bfloat16_against_the_32_bit_path():
     worst = max(e for _, e, _ in errs)
     mean = float(np.mean([m for _, _, m in errs]))
     assert worst < 0.03 and worst < 2.0 * mean, errs
+
+
+@pytest.mark.parametrize("stored,run", [("float32", "bfloat16"), ("bfloat16", "float32")])
+def test_a_model_stored_in_one_precision_runs_in_the_other(stored, run):
+    """Matrices stored in 32-bit stay so in a bfloat16 run (activations are bfloat16, the products take the plain
+    kernels); matrices stored in bfloat16 are widened for a 32-bit run.  Logits against the plain implementation on
+    the folder's own values, whole and cut."""
+    for name in ("A", "B"):
+        folder = H.model_folder(name, stored, True)
+        cfg, runner = make_runner(folder, run)
+        toks = H.random_tokens(cfg.vocab_size, 70, seed=3)
+        for cuts in (H.cut_whole(70), H.cut_tail_decoded(70), H.cut_changing(70, 2)):
+            got = run_cut(runner, "x", toks, cuts)
+            H.check_logits(got, folder, toks, run, f"{name} stored {stored}, run {run}, {cuts[:4]}")
