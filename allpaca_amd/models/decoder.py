@@ -100,13 +100,18 @@ class DecoderModel:
 
 
 def load_model(model_dir: str, dtype: torch.dtype, device: torch.device | str = "cuda:0",
-               max_positions: Optional[int] = None):
+               max_positions: Optional[int] = None, beyond_configured_positions: bool = False):
     """Model folder -> (typed configuration, bound DecoderModel).  The class of the model is
-    chosen by config.json."""
+    chosen by config.json.  `max_positions`: positions the run is set up for (position tables), at most the
+    configuration's own limit unless `beyond_configured_positions` (the formulas hold at any position, and the
+    reference does not read `max_position_embeddings`; a replay of given tokens may go past it)."""
     from . import describe_model
     arch, cfg, spec = describe_model(read_config_json(model_dir))
     model = DecoderModel(spec)
     tensors = load_tensors(model_dir, model.param_specs(), dtype, spec.forbidden)
-    rt = Runtime(torch.device(device), dtype, min(max_positions or spec.max_positions, spec.max_positions))
+    positions = max_positions or spec.max_positions
+    if not beyond_configured_positions:
+        positions = min(positions, spec.max_positions)
+    rt = Runtime(torch.device(device), dtype, positions)
     model.bind(tensors, rt)
     return cfg, model
