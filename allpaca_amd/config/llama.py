@@ -9,6 +9,9 @@ from dataclasses import dataclass, field, asdict
 from typing import Any, Mapping, Optional, Tuple
 
 
+DEFAULT_MAX_POSITIONS = 2048   # `max_position_embeddings` of a llama config.json that does not name it
+
+
 class ConfigError(ValueError):
     pass
 
@@ -36,7 +39,7 @@ class Llama3RopeScaling:
 
     @classmethod
     def from_dict(cls, d: Mapping[str, Any]) -> "Llama3RopeScaling":
-        kind = d.get("rope_type", d.get("type"))
+        kind = d.get("rope_type") or d.get("type")
         if kind != "llama3":
             raise ConfigError(f"config.json: rope_scaling.rope_type {kind!r} is not supported (known: 'llama3')")
         try:
@@ -92,7 +95,17 @@ class LlamaConfig:
         for key in ("attention_bias", "mlp_bias"):
             if d.get(key):
                 raise ConfigError(f"config.json: {key} = true is not supported (the llama decoder has no biases)")
+        # Newer config.json files carry theta and the scaling in one `rope_parameters` table
+        # (HfRopeParameters, sidecar.rs:17-29); the top-level keys win where both are there.
+        nested = d.get("rope_parameters") or {}
+        theta = d.get("rope_theta")
+        if theta is None:
+            theta = nested.get("rope_theta", 10000.0)   # sidecar.rs:217-219
         scaling = d.get("rope_scaling")
+        if not scaling and (nested.get("rope_type") or nested.get("type")) not in (None, "default"):
+            scaling = nested
+        if scaling and (scaling.get("rope_type") or scaling.get("type")) == "default":
+            scaling = None
         cfg = cls(
             vocab_size=_need(d, "vocab_size"),
             hidden_size=hidden,
@@ -102,9 +115,12 @@ class LlamaConfig:
             head_dim=int(head_dim),
             intermediate_size=_need(d, "intermediate_size"),
             rms_norm_eps=float(d.get("rms_norm_eps", 1e-5)),   # sidecar.rs:214-216
-            rope_theta=float(d.get("rope_theta", 10000.0)),    # sidecar.rs:217-219
+            rope_theta=float(theta),
             rope_scaling=Llama3RopeScaling.from_dict(scaling) if scaling else None,
-            max_position_embeddings=_need(d, "max_position_embeddings"),
+            # positions the tables are made for unless the engine is set up for fewer; the reference does not read
+            # the key (no tensor's shape hangs on it), so a file without it is taken with the published default
+            max_position_embeddings=(_need(d, "max_position_embeddings") if d.get("max_position_embeddings") is not None
+                                     else DEFAULT_MAX_POSITIONS),
             tie_word_embeddings=bool(d.get("tie_word_embeddings", False)),
             hidden_act="silu",
             architectures=tuple(d.get("architectures") or ("LlamaForCausalLM",)),

@@ -30,8 +30,27 @@ def test_config_reads_every_key_and_defaults():
     assert c.rope_scaling is None and c.tie_word_embeddings is False
 
 
+def test_config_takes_the_rope_parameters_table_and_a_file_without_a_position_limit():
+    """Newer files carry theta and the scaling under `rope_parameters` (sidecar.rs:17-29); `max_position_embeddings`
+    fixes no tensor's shape and the reference does not read it."""
+    d = dict(H.TINY_B)
+    scaling, theta = d.pop("rope_scaling"), d.pop("rope_theta")
+    d["rope_parameters"] = dict(scaling, rope_theta=theta)
+    assert LlamaConfig.from_dict(d) == LlamaConfig.from_dict(H.TINY_B)
+    d = dict(H.TINY_A, rope_parameters=dict(rope_type="default", rope_theta=12345.0))
+    d.pop("rope_theta")
+    c = LlamaConfig.from_dict(d)
+    assert c.rope_theta == 12345.0 and c.rope_scaling is None
+    assert LlamaConfig.from_dict(dict(H.TINY_A, rope_scaling=dict(rope_type="default"))).rope_scaling is None
+    assert LlamaConfig.from_dict(dict(H.TINY_B, rope_scaling=dict(H.TINY_B["rope_scaling"], rope_type=None, type="llama3"))
+                                 ).rope_scaling.factor == 8.0
+    d = dict(H.TINY_A)
+    d.pop("max_position_embeddings")
+    assert LlamaConfig.from_dict(d).max_position_embeddings == 2048
+
+
 @pytest.mark.parametrize("key", ["hidden_size", "num_hidden_layers", "num_attention_heads", "intermediate_size",
-                                 "vocab_size", "max_position_embeddings"])
+                                 "vocab_size"])
 def test_config_required_keys(key):
     d = dict(H.TINY_A)
     d.pop(key)
