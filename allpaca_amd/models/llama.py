@@ -34,9 +34,10 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
                 "ffn": PartSpec("swiglu", dict(hidden_size=cfg.hidden_size,
                                                intermediate_size=cfg.intermediate_size), "mlp."),
             }))
-    forbidden = {}
+    forbidden, copies = {}, {}
     if cfg.tie_word_embeddings:
         forbidden["lm_head.weight"] = "tie_word_embeddings is true, the head is the embedding matrix"
+        copies["lm_head.weight"] = "model.embed_tokens.weight"
     return ModelSpec(
         hidden_size=cfg.hidden_size,
         vocab_size=cfg.vocab_size,
@@ -49,6 +50,8 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
         head=PartSpec("linear", dict(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size,
                                      tied=cfg.tie_word_embeddings), "lm_head."),
         forbidden=forbidden,
+        copies=copies,
+        ignored_suffixes=(".rotary_emb.inv_freq",),   # a table of rotation frequencies that older writers stored
     )
 
 

@@ -57,6 +57,11 @@ class ModelSpec:
     head: PartSpec
     # tensors that must NOT be in the file (a tied head's own matrix): name -> reason
     forbidden: Dict[str, str] = field(default_factory=dict)
+    # ... unless they are a copy, bit for bit, of the tensor they stand for (writers that store a tied matrix twice):
+    # name -> name of the tensor it must equal
+    copies: Dict[str, str] = field(default_factory=dict)
+    # endings of tensor names that are no parameters and are passed over (buffers some writers store)
+    ignored_suffixes: tuple = ()
 
     def validate(self) -> None:
         for i, e in enumerate(self.plan):

@@ -43,9 +43,12 @@ def target_dtype(spec: ParamSpec, stored: torch.dtype, run_dtype: torch.dtype) -
 
 
 def load_tensors(model_dir: str, wanted: Mapping[str, ParamSpec], run_dtype: torch.dtype,
-                 forbidden: Optional[Mapping[str, str]] = None) -> Dict[str, torch.Tensor]:
+                 forbidden: Optional[Mapping[str, str]] = None, copies: Optional[Mapping[str, str]] = None,
+                 ignored_suffixes: tuple = ()) -> Dict[str, torch.Tensor]:
     """CPU tensors for every name in `wanted` (converted by the storage rule).
-    Raises one `WeightsError` naming all missing, unexpected and wrongly shaped tensors."""
+    Raises one `WeightsError` naming all missing, unexpected and wrongly shaped tensors.
+    `forbidden`: names that must not be there (name -> reason), except that a name in `copies` may be there if it
+    equals, bit for bit, the tensor `copies[name]`; names with an ending in `ignored_suffixes` are passed over."""
     files = open_model_files(model_dir)
     where: Dict[str, SafetensorsFile] = {}
     other: List[str] = []
@@ -73,7 +76,14 @@ def load_tensors(model_dir: str, wanted: Mapping[str, ParamSpec], run_dtype: tor
         if name in wanted:
             continue
         if name in forbidden:
-            other.append(f"tensor {name} must not be present: {forbidden[name]}")
+            twin = (copies or {}).get(name)
+            if twin in where and where[name].entries[name] == where[twin].entries[twin] and \
+                    torch.equal(where[name].tensor(name).view(torch.uint8), where[twin].tensor(twin).view(torch.uint8)):
+                continue     # the same matrix stored twice
+            other.append(f"tensor {name} must not be present: {forbidden[name]}"
+                         + (f" (it is there and differs from {twin})" if twin in where else ""))
+        elif any(name.endswith(suffix) for suffix in ignored_suffixes):
+            continue
         else:
             unexpected.append(name)
     if missing or unexpected or wrong or other:

@@ -164,6 +164,26 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
         assert piece in msg
 
 
+def test_a_tied_head_stored_twice_and_a_frequency_buffer_are_passed_over(tmp_path):
+    """Some writers store a tied matrix under both names and a table of rotation frequencies: a copy, bit for bit,
+    of the embedding is no error, a head that differs is; names ending in `.rotary_emb.inv_freq` are no parameters."""
+    from allpaca_amd.models import DecoderModel, describe_model
+    path, tensors = folder(tmp_path)
+    _, _, spec = describe_model(H.TINY_A)
+    want = DecoderModel(spec).param_specs()
+    more = dict(tensors)
+    more["lm_head.weight"] = tensors["model.embed_tokens.weight"].clone()
+    more["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.ones(8)
+    rewrite(path, more)
+    got = load_tensors(path, want, torch.float32, spec.forbidden, spec.copies, spec.ignored_suffixes)
+    assert set(got) == set(want)
+    more["lm_head.weight"][3, 5] += 1.0
+    rewrite(path, more)
+    with pytest.raises(WeightsError) as e:
+        load_tensors(path, want, torch.float32, spec.forbidden, spec.copies, spec.ignored_suffixes)
+    assert any("lm_head.weight" in m and "differs" in m for m in e.value.other) and not e.value.unexpected
+
+
 def test_untied_model_needs_its_head(tmp_path):
     path, tensors = folder(tmp_path, H.TINY_B)
     want, forbidden = specs(H.TINY_B)
