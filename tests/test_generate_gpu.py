@@ -217,12 +217,14 @@ def test_trace_run_goes_past_the_position_limit_of_config_json(tmp_path):
     reference does not read that key), as the plain implementation does."""
     folder = H.model_folder("A", "float32", True)
     t = H.random_tokens(256, 200, seed=77)
-    steps = [dict(step=0, entries=[dict(id="a", tokens=t[:150], want=[100, 149])], end=[])]
+    # wanted places in any order, one of them twice: the rows come in the order asked for
+    steps = [dict(step=0, entries=[dict(id="a", tokens=t[:150], want=[149, 100, 149])], end=[])]
     steps += [dict(step=1 + j, entries=[dict(id="a", tokens=[t[150 + j]], want=[0])], end=[]) for j in range(50)]
     out = str(tmp_path / "past")
     replay(folder, "float32", steps, 256, out)
     rows = [np.fromfile(os.path.join(out, f"{s}.f32"), dtype="<f4").reshape(-1, 256) for s in range(51)]
-    H.assert_close(np.concatenate(rows), H.oracle_logits(folder, t)[[100] + list(range(149, 200))], "float32", "past the limit")
+    H.assert_close(np.concatenate(rows), H.oracle_logits(folder, t)[[149, 100] + list(range(149, 200))], "float32",
+                   "past the limit")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
