@@ -213,7 +213,7 @@ def test_widths_of_an_8b_model_in_bfloat16_against_the_32_bit_path():
                     v = (v.float() * sharpen).to(torch.bfloat16)
                 tensors[k] = v if dtype == torch.bfloat16 else v.float()
         model.bind(tensors, Runtime(torch.device("cuda:0"), dtype, 1024))
-        return ModelRunner(model, 16, 128, 8, use_graphs=True)
+        return ModelRunner(model, 16, 192, 48, use_graphs=True)
 
     toks = H.random_tokens(V, 420, seed=5)
     rows = {}
@@ -227,6 +227,18 @@ def test_widths_of_an_8b_model_in_bfloat16_against_the_32_bit_path():
             out.append(("decode step", r.step([Entry("a", [toks[340 + j]], [0]), Entry("b", [toks[17 + j]], [0])])))
         out.append(("portion behind", r.step([Entry("a", toks[346:400], [0, 53]), Entry("b", toks[23:24], [0])])))
         assert r.graph_replays == 6
+        # 40 more requests: a mixed step of 160 rows, two decode steps of 42 rows (the tiled product with K in slices
+        # and the folded norm in its finishing kernel), and a portion of 600 rows (K in slices for the narrow matrices)
+        more = [f"m{i}" for i in range(40)]
+        for m in more:
+            r.admit(m)
+        out.append(("many short prompts", r.step([Entry(m, toks[i:i + 4], [3]) for i, m in enumerate(more)])))
+        for j in range(2):
+            out.append(("decode step of 42 rows", r.step([Entry("a", [toks[400 + j]], [0]), Entry("b", [toks[24 + j]], [0])]
+                                                          + [Entry(m, [toks[i + 4 + j]], [0]) for i, m in enumerate(more)])))
+        r.release("a")
+        r.admit("c")
+        out.append(("portion of 600 rows", r.step([Entry("c", (toks * 2)[:600], [0, 299, 599])])))
         rows[dtype] = [(what, lg.float().cpu().numpy().astype(np.float64)) for what, lg in out]
         del r
         torch.cuda.empty_cache()
