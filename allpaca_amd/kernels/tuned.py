@@ -119,37 +119,38 @@ def swiglu_bf16(h: torch.Tensor, wg: PackedWeight, wu: PackedWeight, out: torch.
 
 def gemm_emit_bf16(a: torch.Tensor, w: PackedWeight, residual: torch.Tensor, g: torch.Tensor):
     """residual += a . w^T, and for the RMS norm with weight g that reads the residual next: the row
-    bfloat16(residual * g) and the sums of residual^2 per band of 16 columns and row.  Returns (raw [M, N],
-    ss) or None, with nothing done, for sizes no kernel takes.  ss is [16, ceil(N/16) rounded up to 4] from the
-    streaming kernel (up to 16 rows) and [M, ceil(N/256)] from the tiled kernel with K in slices (17..1024 rows, where
-    the matrix has so few columns that K is cut); the products below take either."""
+    bfloat16(residual * g) and sums of residual^2 per row and group of columns.  Returns (raw [M, N], ss) or None,
+    with nothing done, for sizes no kernel takes.  ss is [16, ceil(N/16) rounded up to 4] from the streaming kernel
+    (up to 16 rows) and [M, ceil(N/256)] from the tiled kernel with K in slices; the products below take what the
+    same number of rows gives."""
     _ops._gpu(a, w.data, residual, g)
     M, K = a.shape
     N = w.N
-    if (M > MANY_ROWS_SPLIT_MAX or not _act_ok(a) or residual.dtype != torch.float32 or g.dtype != torch.float32
-            or g.numel() != N or not g.is_contiguous()):
+    if (not _act_ok(a) or residual.dtype != torch.float32 or g.dtype != torch.float32 or g.numel() != N
+            or not g.is_contiguous()):
         return None
     if not (w.K == K and residual.shape == (M, N)):
         raise ValueError(f"gemm: a [{M}, {K}], w {w.shape}, residual {tuple(residual.shape)}")
-    if M > SKINNY_MAX_ROWS:   # the tiled kernel with K in slices: sums per row and block of 256 columns
+    L = _lib.load("tuned")
+    lda, ldc = _ops._rows(a, "a"), _ops._rows(residual, "residual")
+    if M > SKINNY_MAX_ROWS:   # the tiled kernel: only where K is cut into slices (the finishing kernel leaves the row)
         ks = _tiled_k_split(M, N, K)
         if ks == 1:
+            # With K in one piece the product's own epilogue would have to do it; measured at 2,048 rows that costs
+            # 20-27 us a product, more than the norm's kernel (10 us) that it would save.
             return None
         raw = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
         ss = torch.empty((M, -(-N // 256)), dtype=torch.float32, device=a.device)
         ws = torch.empty(ks * M * N, dtype=torch.float32, device=a.device)
-        L = _lib.load("tuned")
-        _lib.check(L.apc_gemm_splitk_emit_bf16(a.data_ptr(), _ops._rows(a, "a"), w.data.data_ptr(), residual.data_ptr(),
-                                               _ops._rows(residual, "residual"), M, N, K, ks, ws.data_ptr(),
-                                               g.data_ptr(), raw.data_ptr(), N, ss.data_ptr(), _ops._stream()),
-                   "gemm_splitk_emit_bf16")
+        _lib.check(L.apc_gemm_splitk_emit_bf16(a.data_ptr(), lda, w.data.data_ptr(), residual.data_ptr(), ldc, M, N, K,
+                                               ks, ws.data_ptr(), g.data_ptr(), raw.data_ptr(), N, ss.data_ptr(),
+                                               _ops._stream()), "gemm_splitk_emit_bf16")
         return raw, ss
     raw = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
     ss = torch.empty((16, -(-(-(-N // 16)) // 4) * 4), dtype=torch.float32, device=a.device)
-    L = _lib.load("tuned")
-    _lib.check(L.apc_skinny_gemm_emit_bf16(a.data_ptr(), _ops._rows(a, "a"), w.data.data_ptr(), residual.data_ptr(),
-                                           _ops._rows(residual, "residual"), M, N, K, g.data_ptr(), raw.data_ptr(), N,
-                                           ss.data_ptr(), _ops._stream()), "skinny_gemm_emit_bf16")
+    _lib.check(L.apc_skinny_gemm_emit_bf16(a.data_ptr(), lda, w.data.data_ptr(), residual.data_ptr(), ldc, M, N, K,
+                                           g.data_ptr(), raw.data_ptr(), N, ss.data_ptr(), _ops._stream()),
+               "skinny_gemm_emit_bf16")
     return raw, ss
 
 
@@ -159,10 +160,11 @@ def _pre_ok(raw: torch.Tensor, ss: torch.Tensor, K: int) -> bool:
 
 
 def _pre_tiled(raw: torch.Tensor, ss: torch.Tensor, eps: float, w, wu, out: torch.Tensor, n_cols: int, mode: int) -> bool:
-    """The same on the tiled kernel (17..1024 rows), K in slices or in one piece: ss is [M, ceil(K / 256)]."""
+    """The same on the tiled kernel (more than 16 rows), K in slices or in one piece: ss is [M, parts] with up to
+    256 sums of squares a row (what the tiled kernels leave: a part per 256 or per 128 columns)."""
     M, K = raw.shape
-    if not (SKINNY_MAX_ROWS < M <= MANY_ROWS_SPLIT_MAX and _act_ok(raw) and ss.dtype == torch.float32
-            and ss.is_contiguous() and tuple(ss.shape) == (M, -(-K // 256)) and ss.shape[1] <= 256):
+    if not (M > SKINNY_MAX_ROWS and _act_ok(raw) and ss.dtype == torch.float32 and ss.is_contiguous()
+            and ss.dim() == 2 and ss.shape[0] == M and 1 <= ss.shape[1] <= 256):
         return False
     n_mats = 2 if wu is not None else 1
     ks = _tiled_k_split(M, n_cols * n_mats, K)
