@@ -361,12 +361,10 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const float* __restric
   }
 }
 
-static int launch_splitk(const void* A, int lda, const void* W, const void* Wu, void* C, int ldc, int M, int N, int K,
-                         int mode, int k_split, float* workspace, int pre, int emit, FinishNorm norm,
-                         hipStream_t stream) {
-  if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || lda < K || ldc < N || k_split < 1 || !workspace || M > 65535) return APC_ERR_BAD_ARG;
-  if (mode < 0 || mode > G_SWIGLU || (mode == G_SWIGLU) != (Wu != nullptr)) return APC_ERR_BAD_ARG;
+// The first half of a product with K in slices: G_PARTIAL blocks leave float32 sums in workspace[which][slice][M][N].
+static int launch_partials(const void* A, int lda, const void* W, const void* Wu, int M, int N, int K, int k_split,
+                           float* workspace, hipStream_t stream) {
+  if (K <= 0 || lda < K || k_split < 1 || !workspace || M > 65535) return APC_ERR_BAD_ARG;
   if (K % 8 || lda % 8 || !aligned16(A) || !aligned16(W) || (Wu && !aligned16(Wu))) return APC_ERR_UNSUPPORTED;
   const int n_mats = Wu ? 2 : 1;
   if (k_split * n_mats > 65535) return APC_ERR_BAD_ARG;
@@ -384,6 +382,17 @@ static int launch_splitk(const void* A, int lda, const void* W, const void* Wu, 
   }
 #undef PARTIAL_LAUNCH
   APC_LAUNCH_CHECK();
+  return 0;
+}
+
+static int launch_splitk(const void* A, int lda, const void* W, const void* Wu, void* C, int ldc, int M, int N, int K,
+                         int mode, int k_split, float* workspace, int pre, int emit, FinishNorm norm,
+                         hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (ldc < N) return APC_ERR_BAD_ARG;
+  if (mode < 0 || mode > G_SWIGLU || (mode == G_SWIGLU) != (Wu != nullptr)) return APC_ERR_BAD_ARG;
+  const int e = launch_partials(A, lda, W, Wu, M, N, K, k_split, workspace, stream);
+  if (e) return e;
   const dim3 grid(ceil_div(N, 256), M);
 #define FINISH(PRE_, EMIT_)                                                                                     \
   hipLaunchKernelGGL((gemm_finish_kernel<PRE_, EMIT_>), grid, dim3(256), 0, stream, workspace, k_split, M, N, K, mode, \
@@ -394,6 +403,64 @@ static int launch_splitk(const void* A, int lda, const void* W, const void* Wu, 
 #undef FINISH
   APC_LAUNCH_CHECK();
   return 0;
+}
+
+// Finishing kernel of the product for q, k and v (K in slices): it adds the slices, scales them if the row came from
+// a product that left the norm's row (PRE), rounds to bfloat16 as a stored result would be, rotates q and k by the
+// row's position (whole heads, pairs (e, e + d/2)) and writes k and v into the paged cache: what the product's
+// finishing kernel and the kernel for rotation and cache write would do one after the other.  A block has 256
+// columns of one row, which are whole heads (256 is a multiple of d): a value meets its partner through LDS.
+struct FinishRope {
+  const float* cos_sin;    // [positions][2][d / 2]
+  const int* positions;    // [M]
+  const int* row_seg;      // [M]
+  const int* block_table;  // [segments][max_blocks]
+  int max_blocks;
+  bf16_t* cache;           // pages of [2][Hk][P * d]: keys [kv head][slot][d], values [kv head][d][slot]
+  int P, H, Hk, d;
+};
+
+template <bool PRE>
+__global__ __launch_bounds__(256) void gemm_finish_qkv_rope_kernel(const float* __restrict__ partials, int k_split, int M,
+                                                                   int N, int K, bf16_t* __restrict__ q_out, int ldq,
+                                                                   FinishNorm norm, FinishRope rope) {
+  __shared__ float red[4];
+  __shared__ float vals[256];
+  const int n = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
+  const bool on = n < N;
+  float rstd = 1.f;
+  if constexpr (PRE) {
+    const float v = threadIdx.x < norm.pre_parts ? norm.pre_ss[(size_t)m * norm.pre_parts + threadIdx.x] : 0.f;
+    rstd = 1.0f / sqrtf(block_sum<256>(v, red) / (float)K + norm.eps);
+  }
+  const size_t plane = (size_t)M * N;
+  const float* src = partials + (size_t)m * N + (on ? n : 0);
+  float g = 0.f;
+  for (int s = 0; s < k_split; ++s) g += src[s * plane];
+  const float x = bf16_to_float(float_to_bf16(g * rstd));
+  vals[threadIdx.x] = x;
+  __syncthreads();
+  if (!on) return;
+  const int d = rope.d, half = d / 2, head = n / d, e = n % d;
+  const int pos = rope.positions[m];
+  bf16_t* page = rope.cache + (size_t)rope.block_table[(size_t)rope.row_seg[m] * rope.max_blocks + pos / rope.P] *
+                                  ((size_t)2 * rope.Hk * rope.P * d);
+  const int slot = pos % rope.P;
+  if (head < rope.H + rope.Hk) {
+    const float* cs = rope.cos_sin + (size_t)pos * d;
+    float y;
+    if (e < half) {
+      const float av = x, bv = vals[threadIdx.x + half], c = cs[e], sn = cs[half + e];
+      y = av * c - bv * sn;
+    } else {
+      const float av = vals[threadIdx.x - half], bv = x, c = cs[e - half], sn = cs[e];
+      y = av * sn + bv * c;
+    }
+    if (head < rope.H) q_out[(size_t)m * ldq + n] = float_to_bf16(y);
+    else page[((size_t)(head - rope.H) * rope.P + slot) * d + e] = float_to_bf16(y);
+  } else {
+    page[(size_t)rope.Hk * rope.P * d + ((size_t)(head - rope.H - rope.Hk) * d + e) * rope.P + slot] = float_to_bf16(x);
+  }
 }
 
 // Product for 17..128 rows: K is cut into `k_split` slices that different blocks multiply, so that matrices with
@@ -467,4 +534,34 @@ APC_EXPORT int apc_gemm_pre_bf16(const void* A, int lda, const float* ss, int ss
     case G_SWIGLU: return launch_gemm<G_SWIGLU, true>(a, lda, w, (const bf16_t*)Wu, C, ldc, M, N, K, stream, pre);
     default: return APC_ERR_BAD_ARG;
   }
+}
+
+// q, k and v of 17 or more rows with K in slices, q and k rotated, k and v written into the paged cache (see
+// gemm_finish_qkv_rope_kernel).  W: tiled layout of [(H + 2 Hk) d, K]; q_out [M, ldq] takes the rotated q heads in its
+// first H d columns; 256 must be a multiple of d.  With ss: A is a row that a product into the residual left and the
+// sums are scaled as in apc_gemm_splitk_pre_bf16.  workspace: k_split * M * (H + 2 Hk) d floats.
+APC_EXPORT int apc_gemm_splitk_qkv_rope_bf16(const void* A, int lda, const float* ss, int ss_parts, float eps,
+                                             const void* W, void* q_out, int ldq, int M, int K, int H, int Hk, int d,
+                                             const float* cos_sin, const int* positions, const int* row_seg,
+                                             const int* block_table, int max_blocks, void* cache, int page_tokens,
+                                             int k_split, float* workspace, hipStream_t stream) {
+  if (M <= 0) return 0;
+  if (H <= 0 || Hk <= 0 || d <= 0 || ldq < H * d || !cos_sin || !positions || !row_seg || !block_table ||
+      max_blocks <= 0 || !cache || page_tokens <= 0 || !q_out || (ss && ss_parts <= 0))
+    return APC_ERR_BAD_ARG;
+  if (d % 2 || 256 % d || (ss && ss_parts > 256)) return APC_ERR_UNSUPPORTED;
+  const int N = (H + 2 * Hk) * d;
+  const int e = launch_partials(A, lda, W, nullptr, M, N, K, k_split, workspace, stream);
+  if (e) return e;
+  const FinishNorm norm{ss, ss_parts, eps, nullptr, nullptr, 0, nullptr};
+  const FinishRope rope{cos_sin, positions, row_seg, block_table, max_blocks, (bf16_t*)cache, page_tokens, H, Hk, d};
+  const dim3 grid(ceil_div(N, 256), M);
+  if (ss)
+    hipLaunchKernelGGL((gemm_finish_qkv_rope_kernel<true>), grid, dim3(256), 0, stream, workspace, k_split, M, N, K,
+                       (bf16_t*)q_out, ldq, norm, rope);
+  else
+    hipLaunchKernelGGL((gemm_finish_qkv_rope_kernel<false>), grid, dim3(256), 0, stream, workspace, k_split, M, N, K,
+                       (bf16_t*)q_out, ldq, norm, rope);
+  APC_LAUNCH_CHECK();
+  return 0;
 }

@@ -47,6 +47,7 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_rope_kv_write_bf16": [P, I, I, I, I, I, I, I, I, I, P, P, P, P, I, P, I, P],
         "apc_gemm_splitk_emit_bf16": [P, I, P, P, I, I, I, I, I, P, P, P, I, P, P],
         "apc_gemm_pre_bf16": [P, I, P, I, F, P, P, P, I, I, I, I, I, P],
+        "apc_gemm_splitk_qkv_rope_bf16": [P, I, P, I, F, P, P, I, I, I, I, I, I, P, P, P, P, I, P, I, I, P, P],
         "apc_gemm_splitk_pre_bf16": [P, I, P, I, F, P, P, P, I, I, I, I, I, I, P, P],
         "apc_gemm_splitk_bf16": [P, I, P, P, P, I, I, I, I, I, I, P, P],
         "apc_skinny_gemm_bf16": [P, I, P, P, I, I, I, I, I, P],

@@ -206,23 +206,32 @@ def gemm_pre_bf16(raw: torch.Tensor, ss: torch.Tensor, eps: float, w: PackedWeig
 def qkv_rope_bf16(a: torch.Tensor, pre, w: PackedWeight, q_out: torch.Tensor, n_heads: int, n_kv_heads: int,
                   head_dim: int, cos_sin: torch.Tensor, positions: torch.Tensor, row_seg: torch.Tensor,
                   block_table: torch.Tensor, cache: torch.Tensor, page_tokens: int) -> bool:
-    """q, k, v of up to 16 rows in one product that also rotates q and k (whole heads) and writes k and v into the
-    pages; rotated q goes to the first n_heads * head_dim columns of q_out.  `a`: the normalised rows, or with
-    `pre` = (ss, eps) the row that `gemm_emit_bf16` left.  False, with nothing done, for sizes the kernel does not
-    take."""
+    """q, k, v in one product that also rotates q and k (whole heads) and writes k and v into the pages; rotated q
+    goes to the first n_heads * head_dim columns of q_out.  Up to 16 rows: the streaming kernel (head size a
+    multiple of 32); more rows: the tiled kernel where it cuts K into slices, in its finishing kernel (256 a
+    multiple of the head size).  `a`: the normalised rows, or with `pre` = (ss, eps) the row that
+    `gemm_emit_bf16` left.  False, with nothing done, for sizes neither takes."""
     _ops._gpu(a, w.data, q_out, cos_sin, positions, row_seg, block_table, cache)
     M, K = a.shape
     H, Hk, d = n_heads, n_kv_heads, head_dim
-    if not (M <= SKINNY_MAX_ROWS and _act_ok(a) and d % 32 == 0 and q_out.dtype == torch.bfloat16
-            and cache.dtype == torch.bfloat16 and q_out.stride(0) % 4 == 0 and q_out.data_ptr() % 8 == 0):
+    N = (H + 2 * Hk) * d
+    few = M <= SKINNY_MAX_ROWS
+    if not (_act_ok(a) and q_out.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16):
         return False
-    ss, eps, n_ss = None, 0.0, 0
+    if few and not (d % 32 == 0 and q_out.stride(0) % 4 == 0 and q_out.data_ptr() % 8 == 0):
+        return False
+    ks = 1 if few else _tiled_k_split(M, N, K)
+    if not few and (ks == 1 or 256 % d or d % 2):
+        return False
+    ss, eps = None, 0.0
     if pre is not None:
         ss, eps = pre
-        if not _pre_ok(a, ss, K):
+        if few and not _pre_ok(a, ss, K):
             return False
-        n_ss = -(-K // 16)
-    if not (w.K == K and w.N == (H + 2 * Hk) * d and q_out.shape[0] == M and q_out.shape[1] >= H * d):
+        if not few and not (ss.dtype == torch.float32 and ss.is_contiguous() and ss.dim() == 2 and ss.shape[0] == M
+                            and 1 <= ss.shape[1] <= 256):
+            return False
+    if not (w.K == K and w.N == N and q_out.shape[0] == M and q_out.shape[1] >= H * d):
         raise ValueError(f"qkv: a [{M}, {K}], w {w.shape}, {H}+2*{Hk} heads of {d}, q_out {tuple(q_out.shape)}")
     _ops._need(cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and tuple(cos_sin.shape[1:]) == (2, d // 2),
                "cos/sin table must be float32 [positions, 2, head_dim/2]")
@@ -231,11 +240,21 @@ def qkv_rope_bf16(a: torch.Tensor, pre, w: PackedWeight, q_out: torch.Tensor, n_
     _ops._need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
                "block table must be contiguous int32 [segments, blocks]")
     L = _lib.load("tuned")
-    _lib.check(L.apc_skinny_qkv_rope_bf16(
-        a.data_ptr(), _ops._rows(a, "a"), ss.data_ptr() if ss is not None else 0, n_ss, float(eps), w.data.data_ptr(),
+    ss_ptr = ss.data_ptr() if ss is not None else 0
+    if few:
+        _lib.check(L.apc_skinny_qkv_rope_bf16(
+            a.data_ptr(), _ops._rows(a, "a"), ss_ptr, -(-K // 16) if ss is not None else 0, float(eps), w.data.data_ptr(),
+            q_out.data_ptr(), _ops._rows(q_out, "q_out"), M, K, H, Hk, d, cos_sin.data_ptr(),
+            _ops._i32(positions, M, "positions"), _ops._i32(row_seg, M, "row_seg"), block_table.data_ptr(),
+            block_table.shape[1], cache.data_ptr(), page_tokens, _ops._stream()), "skinny_qkv_rope_bf16")
+        return True
+    ws = torch.empty(ks * M * N, dtype=torch.float32, device=a.device)
+    _lib.check(L.apc_gemm_splitk_qkv_rope_bf16(
+        a.data_ptr(), _ops._rows(a, "a"), ss_ptr, ss.shape[1] if ss is not None else 0, float(eps), w.data.data_ptr(),
         q_out.data_ptr(), _ops._rows(q_out, "q_out"), M, K, H, Hk, d, cos_sin.data_ptr(),
         _ops._i32(positions, M, "positions"), _ops._i32(row_seg, M, "row_seg"), block_table.data_ptr(),
-        block_table.shape[1], cache.data_ptr(), page_tokens, _ops._stream()), "skinny_qkv_rope_bf16")
+        block_table.shape[1], cache.data_ptr(), page_tokens, ks, ws.data_ptr(), _ops._stream()),
+        "gemm_splitk_qkv_rope_bf16")
     return True
 
 

@@ -338,11 +338,14 @@ def test_rotation_and_cache_write_16_bytes_a_lane_equals_the_plain_kernel(H, Hk,
 
 @pytest.mark.parametrize("M,H,Hk,d,K,P_,pre", [(8, 32, 8, 128, 4096, 16, True), (5, 6, 2, 64, 328, 8, True),
                                                (16, 3, 3, 32, 72, 24, False), (1, 5, 1, 96, 200, 16, True),
-                                               (3, 4, 2, 256, 264, 32, False)])
+                                               (3, 4, 2, 256, 264, 32, False),
+                                               # more than 16 rows: in the finishing kernel of the product with K in slices
+                                               (17, 6, 2, 64, 520, 8, True), (64, 32, 8, 128, 4096, 16, True),
+                                               (100, 3, 1, 32, 1032, 16, False), (300, 4, 2, 256, 2048, 32, True)])
 def test_product_for_q_k_v_that_rotates_and_fills_the_pages_equals_the_kernels_one_after_the_other(M, H, Hk, d, K, P_, pre):
-    """One kernel for q, k, v of few rows, the rotation and the cache write gives what the product followed by
-    `rope_kv_write` gives: the same rotated q, the same pages (sums rounded to bfloat16 before the rotation in
-    both)."""
+    """One kernel for q, k, v, the rotation and the cache write (the streaming kernel up to 16 rows, the finishing
+    kernel of the tiled product with K in slices beyond) gives what the product followed by `rope_kv_write` gives:
+    the same rotated q, the same pages (sums rounded to bfloat16 before the rotation in both)."""
     from allpaca_amd.kernels import ops
     t = tuned()
     rng = np.random.default_rng(M * 1000 + d)
@@ -351,22 +354,21 @@ def test_product_for_q_k_v_that_rotates_and_fills_the_pages_equals_the_kernels_o
     a = gen(M, K, seed=1, dtype=BF, scale=2.0).to(DEV)
     eps = 2e-5
     ss = None
-    if pre:
+    if pre and M <= 16:
         bands = -(-K // 16)
         ss = torch.zeros(16, -(-bands // 4) * 4, device=DEV)
         ss[:M, :bands] = torch.from_numpy(rng.uniform(0.5, 40.0, (M, bands)).astype(np.float32)).to(DEV)
-    max_pos = 5 * P_
-    # rows of three segments at scattered positions, among them a page's first and last slot
-    pos_list = [int(x) for x in rng.integers(0, max_pos, M)]
-    pos_list[0] = P_ - 1
-    if M > 1:
-        pos_list[1] = 2 * P_
-    seg_list = [r % 3 for r in range(M)]
-    while len({(s_, p_) for s_, p_ in zip(seg_list, pos_list)}) < M:        # no two rows on one place of the cache
-        pos_list = [(p_ + r) % max_pos for r, p_ in enumerate(pos_list)]
+    elif pre:
+        ss = torch.from_numpy(rng.uniform(0.5, 40.0, (M, -(-K // 256))).astype(np.float32)).to(DEV)
+    max_blocks = max(5, -(-M // P_) + 2)
+    max_pos = max_blocks * P_
+    # rows of three segments at scattered places of the cache (no two on one), among them a page's last and first slot
+    forced = [(0, P_ - 1), (1, 2 * P_)][:M]
+    others = [(int(v) // max_pos, int(v) % max_pos) for v in rng.permutation(3 * max_pos)]
+    places = forced + [pl for pl in others if pl not in forced][:M - len(forced)]
+    seg_list, pos_list = [pl[0] for pl in places], [pl[1] for pl in places]
     pos = torch.tensor(pos_list, dtype=torch.int32, device=DEV)
     seg = torch.tensor(seg_list, dtype=torch.int32, device=DEV)
-    max_blocks = 5
     bt = torch.from_numpy(rng.permutation(3 * max_blocks).reshape(3, max_blocks).astype(np.int32)).to(DEV)
     ang = np.arange(max_pos)[:, None] * (1.0 / 300.0 ** (np.arange(d // 2) / (d // 2)))[None, :]
     table = torch.from_numpy(np.stack([np.cos(ang), np.sin(ang)], 1).astype(np.float32)).to(DEV)
@@ -384,13 +386,15 @@ def test_product_for_q_k_v_that_rotates_and_fills_the_pages_equals_the_kernels_o
             ops.rope_kv_write(qkv, 0, H * d, (H + Hk) * d, H, Hk, d, d, table, pos, seg, bt, cache, P_)
         c64 = f64(cache)
         results.append((f64(qkv)[:, :H * d].reshape(M, H, 2, d // 2), c64[:, 0].reshape(-1, Hk, P_, 2, d // 2), c64[:, 1]))
-    # The two ways add the waves' partial sums in different orders, so now and then a sum falls on the other side
-    # of a rounding to bfloat16: one unit of one element of a pair, which the rotation spreads over the pair
-    # (its length is what the rotation keeps), and one unit of the result.
+    # The two ways add the waves' partial sums in different orders: the float32 sums differ by their summation noise
+    # (1e-5 of the largest, as `check` allows; it is all there is to a sum that cancels to almost nothing), and now
+    # and then a sum falls on the other side of a rounding to bfloat16: one unit of one element of a pair, which the
+    # rotation spreads over the pair (its length is what the rotation keeps), and one unit of the result.
     for which, (got, want) in enumerate(zip(results[0], results[1])):
         diff = np.abs(got - want)
         pair = np.sqrt((want ** 2).sum(axis=-2, keepdims=True)) if which < 2 else 0.0
-        assert (diff <= 2.0 ** -7 * np.abs(want) + 2.0 ** -7 * pair + 1e-30).all() and (diff > 0).mean() < 0.02
+        tol = 2.0 ** -7 * np.abs(want) + 2.0 ** -7 * pair + 1e-5 * np.abs(want).max()
+        assert (diff <= tol).all() and (diff > 0).mean() < 0.02
     assert (results[0][1] != 0).sum() + (results[0][2] != 0).sum() == M * 2 * Hk * d   # every row wrote its k and v, once
 
 
