@@ -659,44 +659,89 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   }
 }
 
-// merge of the parts of one (row, head), in key order: first the weights of all parts (their maxima against
-// the overall maximum), then the weighted sum of their outputs with independent loads
+// Merge of the parts of one (row, head), in key order.  A thread owns elements of the head and reads every part's
+// maximum and sum itself (all threads read the same addresses: one cache line a wave), so nothing goes through LDS
+// and the block never waits for itself: the maxima, sums and outputs of up to MERGE_CHUNK parts are asked for in one
+// go, and that is the kernel's one trip to memory when the parts are no more than that.  With more parts a first
+// pass takes the maximum, a second the weighted sums, both in chunks.
 constexpr int MERGE_NT = 128;
+constexpr int MERGE_CHUNK = 16;
 __global__ __launch_bounds__(MERGE_NT) void attn_merge_kernel(const float* __restrict__ parts, int n_parts, int KW,
                                                               int H, int d, const int* __restrict__ positions,
                                                               const int* __restrict__ rows, int window,
                                                               bf16_t* __restrict__ out, int ldo) {
-  extern __shared__ float wgt[];  // [n_parts] weights, then 1 float: 1 / l
   const int ri = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int row = rows ? rows[ri] : ri;
   const int pos = positions[row];
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int p_lo = ((first / 32) * 32) / KW, p_hi = min(pos / KW, n_parts - 1);  // parts with a visible key
   const int np = p_hi - p_lo + 1;
-  const float* base = parts + (((size_t)ri * H + h) * n_parts + p_lo) * (d + 2);
-  for (int p = tid; p < np; p += MERGE_NT) wgt[p] = base[(size_t)p * (d + 2) + d];  // the parts' maxima
-  __syncthreads();
+  const size_t stride = (size_t)d + 2;
+  const float* base = parts + (((size_t)ri * H + h) * n_parts + p_lo) * stride;
+  bf16_t* orow = out + (size_t)row * ldo + (size_t)h * d;
+  const int e0 = tid, e1 = tid + MERGE_NT;  // d <= 256: at most two elements a thread
+  const bool on0 = e0 < d, on1 = e1 < d;
+  if (np <= MERGE_CHUNK) {
+    float pm[MERGE_CHUNK], pl[MERGE_CHUNK], o0[MERGE_CHUNK], o1[MERGE_CHUNK];
+#pragma unroll
+    for (int p = 0; p < MERGE_CHUNK; ++p) {
+      const float* src = base + (size_t)min(p, np - 1) * stride;
+      pm[p] = src[d];
+      pl[p] = src[d + 1];
+      o0[p] = src[on0 ? e0 : 0];
+      o1[p] = on1 ? src[e1] : 0.f;
+    }
+    float m = -INFINITY;
+#pragma unroll
+    for (int p = 0; p < MERGE_CHUNK; ++p)
+      if (p < np) m = fmaxf(m, pm[p]);
+    float l = 0.f, a0 = 0.f, a1 = 0.f;
+#pragma unroll
+    for (int p = 0; p < MERGE_CHUNK; ++p) {
+      if (p < np) {
+        const float w = pm[p] == -INFINITY ? 0.f : exp2_neg(pm[p] - m);
+        l += pl[p] * w;
+        a0 = fmaf(o0[p], w, a0);
+        a1 = fmaf(o1[p], w, a1);
+      }
+    }
+    const float inv = 1.0f / l;
+    if (on0) orow[e0] = float_to_bf16(a0 * inv);
+    if (on1) orow[e1] = float_to_bf16(a1 * inv);
+    return;
+  }
   float m = -INFINITY;
-  for (int p = 0; p < np; ++p) m = fmaxf(m, wgt[p]);
-  __syncthreads();
-  for (int p = tid; p < np; p += MERGE_NT) {
-    const float pm = wgt[p];
-    wgt[p] = pm == -INFINITY ? 0.f : exp2_neg(pm - m);
+  for (int p0 = 0; p0 < np; p0 += MERGE_CHUNK) {
+    float pm[MERGE_CHUNK];
+#pragma unroll
+    for (int p = 0; p < MERGE_CHUNK; ++p) pm[p] = base[(size_t)min(p0 + p, np - 1) * stride + d];
+#pragma unroll
+    for (int p = 0; p < MERGE_CHUNK; ++p) m = fmaxf(m, pm[p]);  // a part read twice changes no maximum
   }
-  __syncthreads();
-  if (tid == 0) {
-    float l = 0.f;
-    for (int p = 0; p < np; ++p) l += base[(size_t)p * (d + 2) + d + 1] * wgt[p];
-    wgt[np] = 1.0f / l;
+  float l = 0.f, a0 = 0.f, a1 = 0.f;
+  for (int p0 = 0; p0 < np; p0 += MERGE_CHUNK) {
+    float pm[MERGE_CHUNK], pl[MERGE_CHUNK], o0[MERGE_CHUNK], o1[MERGE_CHUNK];
+#pragma unroll
+    for (int p = 0; p < MERGE_CHUNK; ++p) {
+      const float* src = base + (size_t)min(p0 + p, np - 1) * stride;
+      pm[p] = src[d];
+      pl[p] = src[d + 1];
+      o0[p] = src[on0 ? e0 : 0];
+      o1[p] = on1 ? src[e1] : 0.f;
+    }
+#pragma unroll
+    for (int p = 0; p < MERGE_CHUNK; ++p) {
+      if (p0 + p < np) {
+        const float w = pm[p] == -INFINITY ? 0.f : exp2_neg(pm[p] - m);
+        l += pl[p] * w;
+        a0 = fmaf(o0[p], w, a0);
+        a1 = fmaf(o1[p], w, a1);
+      }
+    }
   }
-  __syncthreads();
-  const float inv = wgt[np];
-  for (int e = tid; e < d; e += MERGE_NT) {
-    float acc = 0.f;
-#pragma unroll 8
-    for (int p = 0; p < np; ++p) acc = fmaf(base[(size_t)p * (d + 2) + e], wgt[p], acc);
-    out[(size_t)row * ldo + (size_t)h * d + e] = float_to_bf16(acc * inv);
-  }
+  const float inv = 1.0f / l;
+  if (on0) orow[e0] = float_to_bf16(a0 * inv);
+  if (on1) orow[e1] = float_to_bf16(a1 * inv);
 }
 
 // ------------------------------------------------------------------------------------------ entry points
@@ -767,7 +812,7 @@ APC_EXPORT int apc_attention_decode_bf16(const void* q, int ldq, int q_off, void
   else DC_LAUNCH(256);
 #undef DC_LAUNCH
   APC_LAUNCH_CHECK();
-  hipLaunchKernelGGL(attn_merge_kernel, dim3(n_rows, H), dim3(MERGE_NT), (n_parts + 1) * sizeof(float), stream,
+  hipLaunchKernelGGL(attn_merge_kernel, dim3(n_rows, H), dim3(MERGE_NT), 0, stream,
                      workspace, n_parts, keys_per_part, H, d, positions, rows, window, (bf16_t*)out, ldo);
   APC_LAUNCH_CHECK();
   return 0;
