@@ -292,6 +292,23 @@ def _keys_per_part(n_rows: int, n_kv_heads: int, max_context: int, page_tokens: 
     return kw
 
 
+# From how many (row, kv head) pairs on a decode step's attention runs as one block per pair that finishes its heads
+# itself (no partial results through memory, no second kernel): the pairs alone then give every compute unit work
+# (measured at the shapes of an 8B model: 7-15 % faster from 32 rows on, slower with 16).
+WHOLE_MIN_PAIRS = 256
+WHOLE_WAVES = 4   # waves of such a block (NW in attention_bf16.hip)
+
+
+def _keys_per_wave_whole(max_context: int, page_tokens: int) -> int:
+    """Keys of a range in the kernel that takes a (row, kv head) whole: the context spread over the block's waves,
+    64 to 512 keys, and no more pages than a wave keeps ids for (one per lane)."""
+    kw = -(-max_context // WHOLE_WAVES)
+    kw = min(512, max(64, -(-kw // 32) * 32))
+    while kw > 32 and kw // page_tokens + 2 > 64:
+        kw -= 32
+    return kw
+
+
 def attention_bf16(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
                    cache: torch.Tensor, page_tokens: int, block_table: torch.Tensor, step, window: int = 0,
                    scale: Optional[float] = None) -> bool:
@@ -326,10 +343,18 @@ def attention_bf16(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int,
     if step.n_decode_rows:
         n = step.n_decode_rows
         span = min(step.max_decode_context, window) if window else step.max_decode_context
+        rows = step.decode_rows.data_ptr() if step.decode_rows is not None else 0
+        if (n * n_kv_heads * -(-(n_heads // n_kv_heads) // 16) >= WHOLE_MIN_PAIRS
+                and L.apc_attention_decode_whole_fits(n_heads, n_kv_heads, head_dim)):
+            kw = _keys_per_wave_whole(span, page_tokens)
+            _lib.check(L.apc_attention_decode_bf16(
+                q.data_ptr(), ldq, q_off, out.data_ptr(), ldo, n, n_heads, n_kv_heads, head_dim, cache.data_ptr(),
+                page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
+                step.row_seg.data_ptr(), rows, int(window), sc, kw, 0, 0, stream), "attention_decode_bf16 (whole)")
+            return True
         kw = _keys_per_part(n, n_kv_heads, span, page_tokens)
         n_parts = -(-step.max_decode_context // kw)
         ws = torch.empty(n * n_heads * n_parts * (head_dim + 2), dtype=torch.float32, device=q.device)
-        rows = step.decode_rows.data_ptr() if step.decode_rows is not None else 0
         _lib.check(L.apc_attention_decode_bf16(
             q.data_ptr(), ldq, q_off, out.data_ptr(), ldo, n, n_heads, n_kv_heads, head_dim, cache.data_ptr(),
             page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),

@@ -473,11 +473,36 @@ def test_attention_long_context_decode_and_portion_over_history():
     run_attention(H=8, Hk=8, d=128, P_=16, lens=[5000] + [40] * 7, rows_per_seg=[1] * 8, seed=2)
 
 
-def test_attention_finds_a_far_key_in_every_path():
+@pytest.mark.parametrize("H,Hk,d,P_,lens,rows,window", [
+    (32, 8, 128, 16, [2048, 1, 17, 700, 2047], [1, 1, 1, 1, 1], 0),
+    (4, 2, 64, 16, [3000, 5000, 40, 2049], [1, 1, 1, 1], 0),          # several ranges of keys a wave
+    (6, 2, 48, 8, [300, 129, 64, 1], [1, 1, 1, 1], 0),
+    (20, 1, 32, 24, [100, 260, 64], [1, 1, 1], 0),                     # a group wider than one 16-row tile
+    (34, 2, 80, 16, [100, 260], [1, 1], 0),
+    (16, 1, 256, 32, [500, 90], [1, 1], 0),                            # the meeting place does not fit: parts and merge
+    (4, 2, 32, 16, [300, 200, 90, 2500], [1, 1, 1, 1], 100),
+    (4, 4, 16, 16, [300, 200, 90, 1200], [1, 1, 1, 1], 1000),
+    (8, 2, 128, 16, [900, 133, 400], [1, 40, 1], 5),                    # decode rows beside a portion
+])
+def test_attention_decode_by_one_block_a_row_and_kv_head(monkeypatch, H, Hk, d, P_, lens, rows, window):
+    """The decode kernel in which the waves of one block take all keys of a (row, kv head) and finish its heads
+    themselves (chosen from 256 such pairs on; forced here) against the plain attention."""
+    monkeypatch.setattr(tuned(), "WHOLE_MIN_PAIRS", 1)
+    run_attention(H=H, Hk=Hk, d=d, P_=P_, lens=lens, rows_per_seg=rows, window=window, seed=H + d)
+
+
+def test_attention_decode_of_many_rows_takes_the_one_block_kernel_by_itself():
+    # 40 rows x 8 kv heads: above the threshold without forcing; contexts from 1 to 2,100 keys
+    lens = [1 + (i * 211) % 2100 for i in range(40)]
+    run_attention(H=16, Hk=8, d=64, P_=16, lens=lens, rows_per_seg=[1] * 40, seed=3)
+
+
+def test_attention_finds_a_far_key_in_every_path(monkeypatch):
     t = tuned()
     from allpaca_amd.engine.batch import Entry, pack_step
     H, Hk, d, P_, n = 4, 2, 64, 16, 900
-    for rows in (1, 40):
+    for rows, whole in ((1, False), (40, False), (1, True)):
+        monkeypatch.setattr(t, "WHOLE_MIN_PAIRS", 1 if whole else 1 << 30)
         cache, bt, ks, vs = make_cache([n], Hk, d, P_, BF, seed=9)
         key = 17
         page, slot = int(bt[0, key // P_]), key % P_
