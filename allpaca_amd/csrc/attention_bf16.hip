@@ -702,18 +702,18 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(
   }
 }
 
-// Merge of the parts of one (row, head), in key order.  A thread owns elements of the head and reads every part's
-// maximum and sum itself (all threads read the same addresses: one cache line a wave), so nothing goes through LDS
-// and the block never waits for itself: the maxima, sums and outputs of up to MERGE_CHUNK parts are asked for in one
-// go, and that is the kernel's one trip to memory when the parts are no more than that.  With more parts a first
-// pass takes the maximum, a second the weighted sums, both in chunks.
+// Merge of the parts of one (row, head).  Lane p of every wave reads part p's maximum and sum (64 parts a pass), a
+// thread owns elements of the head and asks for its elements of the first MERGE_CHUNK parts at the same time: with up
+// to that many parts the kernel makes one trip to memory, and nothing goes through LDS.  The parts' weights
+// 2^(maximum - overall maximum) are computed once per lane and handed round the wave; sums over parts are taken in a
+// fixed order (over the lanes of a wave as `wave_sum` adds them, over a thread's elements in part order).
 constexpr int MERGE_NT = 128;
 constexpr int MERGE_CHUNK = 16;
 __global__ __launch_bounds__(MERGE_NT) void attn_merge_kernel(const float* __restrict__ parts, int n_parts, int KW,
                                                               int H, int d, const int* __restrict__ positions,
                                                               const int* __restrict__ rows, int window,
                                                               bf16_t* __restrict__ out, int ldo) {
-  const int ri = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int ri = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid % WAVE;
   const int row = rows ? rows[ri] : ri;
   const int pos = positions[row];
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
@@ -724,61 +724,35 @@ __global__ __launch_bounds__(MERGE_NT) void attn_merge_kernel(const float* __res
   bf16_t* orow = out + (size_t)row * ldo + (size_t)h * d;
   const int e0 = tid, e1 = tid + MERGE_NT;  // d <= 256: at most two elements a thread
   const bool on0 = e0 < d, on1 = e1 < d;
-  if (np <= MERGE_CHUNK) {
-    float pm[MERGE_CHUNK], pl[MERGE_CHUNK], o0[MERGE_CHUNK], o1[MERGE_CHUNK];
+  float o0[MERGE_CHUNK], o1[MERGE_CHUNK];
+  auto load_outputs = [&](int q0) {  // this thread's elements of parts q0 .. q0 + MERGE_CHUNK - 1 (the last part again beyond)
 #pragma unroll
     for (int p = 0; p < MERGE_CHUNK; ++p) {
-      const float* src = base + (size_t)min(p, np - 1) * stride;
-      pm[p] = src[d];
-      pl[p] = src[d + 1];
+      const float* src = base + (size_t)min(q0 + p, np - 1) * stride;
       o0[p] = src[on0 ? e0 : 0];
       o1[p] = on1 ? src[e1] : 0.f;
     }
-    float m = -INFINITY;
-#pragma unroll
-    for (int p = 0; p < MERGE_CHUNK; ++p)
-      if (p < np) m = fmaxf(m, pm[p]);
-    float l = 0.f, a0 = 0.f, a1 = 0.f;
-#pragma unroll
-    for (int p = 0; p < MERGE_CHUNK; ++p) {
-      if (p < np) {
-        const float w = pm[p] == -INFINITY ? 0.f : exp2_neg(pm[p] - m);
-        l += pl[p] * w;
-        a0 = fmaf(o0[p], w, a0);
-        a1 = fmaf(o1[p], w, a1);
-      }
-    }
-    const float inv = 1.0f / l;
-    if (on0) orow[e0] = float_to_bf16(a0 * inv);
-    if (on1) orow[e1] = float_to_bf16(a1 * inv);
-    return;
-  }
-  float m = -INFINITY;
-  for (int p0 = 0; p0 < np; p0 += MERGE_CHUNK) {
-    float pm[MERGE_CHUNK];
-#pragma unroll
-    for (int p = 0; p < MERGE_CHUNK; ++p) pm[p] = base[(size_t)min(p0 + p, np - 1) * stride + d];
-#pragma unroll
-    for (int p = 0; p < MERGE_CHUNK; ++p) m = fmaxf(m, pm[p]);  // a part read twice changes no maximum
-  }
+  };
+  auto load_max = [&](int c0) { return c0 + lane < np ? base[(size_t)(c0 + lane) * stride + d] : -INFINITY; };
+  auto load_sum = [&](int c0) { return c0 + lane < np ? base[(size_t)(c0 + lane) * stride + d + 1] : 0.f; };
+  const float pm_first = load_max(0), pl_first = load_sum(0);
+  load_outputs(0);
+  float m = wave_max(pm_first);
+  for (int c0 = WAVE; c0 < np; c0 += WAVE) m = fmaxf(m, wave_max(load_max(c0)));
   float l = 0.f, a0 = 0.f, a1 = 0.f;
-  for (int p0 = 0; p0 < np; p0 += MERGE_CHUNK) {
-    float pm[MERGE_CHUNK], pl[MERGE_CHUNK], o0[MERGE_CHUNK], o1[MERGE_CHUNK];
+  for (int c0 = 0; c0 < np; c0 += WAVE) {
+    const float pm = c0 == 0 ? pm_first : load_max(c0), pl = c0 == 0 ? pl_first : load_sum(c0);
+    const float w = pm == -INFINITY ? 0.f : exp2_neg(pm - m);
+    l += wave_sum(pl * w);
+    for (int q0 = c0; q0 < min(np, c0 + WAVE); q0 += MERGE_CHUNK) {
+      if (q0 > 0) load_outputs(q0);
 #pragma unroll
-    for (int p = 0; p < MERGE_CHUNK; ++p) {
-      const float* src = base + (size_t)min(p0 + p, np - 1) * stride;
-      pm[p] = src[d];
-      pl[p] = src[d + 1];
-      o0[p] = src[on0 ? e0 : 0];
-      o1[p] = on1 ? src[e1] : 0.f;
-    }
-#pragma unroll
-    for (int p = 0; p < MERGE_CHUNK; ++p) {
-      if (p0 + p < np) {
-        const float w = pm[p] == -INFINITY ? 0.f : exp2_neg(pm[p] - m);
-        l += pl[p] * w;
-        a0 = fmaf(o0[p], w, a0);
-        a1 = fmaf(o1[p], w, a1);
+      for (int p = 0; p < MERGE_CHUNK; ++p) {
+        if (q0 + p < np) {
+          const float wp = __shfl(w, q0 + p - c0, WAVE);
+          a0 = fmaf(o0[p], wp, a0);
+          a1 = fmaf(o1[p], wp, a1);
+        }
       }
     }
   }
