@@ -1,5 +1,5 @@
 from .pages import (FREED, CacheError, CacheManager, OutOfPages, OutOfSlots, PagePool, SlotPool, group_needs)
-from .storage import CacheStorage, PagedView, StateView
+from .storage import CacheStorage, CacheTooLarge, PagedView, StateView
 
 __all__ = ["FREED", "CacheError", "CacheManager", "OutOfPages", "OutOfSlots", "PagePool", "SlotPool", "group_needs",
-           "CacheStorage", "PagedView", "StateView"]
+           "CacheStorage", "CacheTooLarge", "PagedView", "StateView"]

@@ -7,12 +7,13 @@ elements); the extra last page is never handed out (rows that pad a replayed
 graph write there).  A state group's tensor is [layers of the group, slots + 1, *shape]."""
 from __future__ import annotations
 
+import math
 from dataclasses import dataclass
 from typing import List, Optional
 
 import torch
 
-from .pages import CacheManager
+from .pages import CacheError, CacheManager
 
 _DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
 
@@ -38,19 +39,34 @@ class StateView:
     slots_host: Optional[List[int]] = None
 
 
+class CacheTooLarge(CacheError):
+    pass
+
+
 class CacheStorage:
     def __init__(self, manager: CacheManager, kv_dtype: torch.dtype, device: torch.device):
         self.manager = manager
         self.device = device
         P = manager.page_tokens
-        self.paged: List[torch.Tensor] = []
-        for g in manager.paged_groups:
-            shape = (len(g.entries), g.pool.num_pages + 1, 2, g.need.kv_heads, P, g.need.head_dim)
-            self.paged.append(torch.zeros(shape, dtype=kv_dtype, device=device))
-        self.state: List[torch.Tensor] = []
-        for g in manager.state_groups:
-            shape = (len(g.entries), manager.max_requests + 1, *g.need.shape)
-            self.state.append(torch.zeros(shape, dtype=_DTYPES[g.need.dtype], device=device))
+        elem = torch.empty((), dtype=kv_dtype).element_size()
+        paged_shapes = [(len(g.entries), g.pool.num_pages + 1, 2, g.need.kv_heads, P, g.need.head_dim)
+                        for g in manager.paged_groups]
+        state_shapes = [(len(g.entries), manager.max_requests + 1, *g.need.shape) for g in manager.state_groups]
+        need = sum(math.prod(sh) * elem for sh in paged_shapes)
+        need += sum(math.prod(sh) * torch.empty((), dtype=_DTYPES[g.need.dtype]).element_size()
+                    for sh, g in zip(state_shapes, manager.state_groups))
+        if device.type == "cuda":
+            free, _ = torch.cuda.mem_get_info(device)
+            free += torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)  # held by torch, unused
+            if need > free:
+                per_page = sum(math.prod(sh) // sh[1] * elem for sh in paged_shapes)
+                raise CacheTooLarge(
+                    f"the cache needs {need / 2**30:.1f} GiB ({[sh[1] - 1 for sh in paged_shapes]} pages of {P} tokens, "
+                    f"{per_page / 2**20:.2f} MiB a page over all layers) but {free / 2**30:.1f} GiB of device memory "
+                    f"are free: ask for fewer pages (max_tokens / num_pages)")
+        self.paged: List[torch.Tensor] = [torch.zeros(sh, dtype=kv_dtype, device=device) for sh in paged_shapes]
+        self.state: List[torch.Tensor] = [torch.zeros(sh, dtype=_DTYPES[g.need.dtype], device=device)
+                                          for sh, g in zip(state_shapes, manager.state_groups)]
 
     def dummy_page(self, group: int) -> int:
         return self.manager.paged_groups[group].pool.num_pages

@@ -345,3 +345,11 @@ def test_steps_queued_ahead_give_the_same_tokens_when_requests_stop_arrive_and_a
     assert got[r3] == full[3][: len(got[r3])] and 0 < len(got[r3]) < 24
     assert eng.runner.cache.free_pages(0) == eng.runner.cache.paged_groups[0].pool.num_pages
     eng.runner.cache.check()
+
+
+def test_a_cache_larger_than_device_memory_is_refused_with_its_size():
+    from allpaca_amd.cache import CacheTooLarge
+    from allpaca_amd.engine import Engine
+    folder = H.model_folder("A", "float32", True)
+    with pytest.raises(CacheTooLarge, match="GiB"):
+        Engine(folder, dtype="float32", page_tokens=16, max_tokens=1 << 34)
