@@ -196,23 +196,9 @@ class ModelRunner:
         g.fill(seqs)
         return PreparedDecode(g, list(seqs))
 
-    def run_prepared(self, prepared: "PreparedDecode", tokens: Sequence[int]) -> torch.Tensor:
-        """The second half: the tokens go in, the step runs.  Nothing may have happened to the requests since
-        `prepare_decode`."""
-        if len(tokens) != len(prepared.seqs):
-            raise StepError("a prepared step needs one token for each of its requests")
-        for t in tokens:
-            if not (0 <= int(t) < self.vocab_size):
-                raise StepError(f"token {t} is outside the vocabulary of {self.vocab_size}")
-        logits = self._launch(prepared.graph, tokens)
-        for s in prepared.seqs:
-            self.cache.commit(s, 1)
-        self.steps += 1
-        return logits
-
-
     def run_fed(self, prepared: "PreparedDecode", device_tokens: torch.Tensor) -> torch.Tensor:
-        """The second half with tokens that are still on the GPU (int32, one per request, in the order of the
+        """The second half: the tokens go in, the step runs; nothing may have happened to the requests since
+        `prepare_decode`.  The tokens are still on the GPU (int32, one per request, in the order of the
         prepared requests: what the sampling kernel of the step before wrote).  They are copied into the step's
         description on the GPU, so the step can be queued before the host has seen them."""
         g, n = prepared.graph, len(prepared.seqs)
