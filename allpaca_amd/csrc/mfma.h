@@ -24,6 +24,17 @@ __device__ __forceinline__ bf16x8_t as_bf16x8(const Frag& f) { return __builtin_
 __device__ __forceinline__ Frag load_frag(const bf16_t* p) { return *reinterpret_cast<const Frag*>(p); }
 __device__ __forceinline__ Frag zero_frag() { Frag f; f.w[0] = f.w[1] = f.w[2] = f.w[3] = 0u; return f; }
 
+// A buffer descriptor over global memory from `base` on (raw, no stride, no bound that matters): a load then takes the
+// descriptor and a scalar byte offset from scalar registers and one 32-bit byte offset per lane.
+typedef __amdgpu_buffer_rsrc_t BufferRsrc;
+__device__ __forceinline__ BufferRsrc make_rsrc(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000);
+}
+__device__ __forceinline__ Frag load_frag_buffer(BufferRsrc rsrc, int lane_bytes, int scalar_bytes) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  return __builtin_bit_cast(Frag, (u32x4)__builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_bytes, scalar_bytes, 0));
+}
+
 // One wave writes LDS and then reads what its other lanes wrote.  The LDS serves a wave's accesses in the order
 // it issues them, so all that is needed is that the compiler keeps that order: a wave barrier (no wait on
 // outstanding global loads, unlike a fence, so loads issued ahead stay in flight).

@@ -229,12 +229,14 @@ def test_product_into_the_residual_leaves_the_next_norms_row_with_more_than_16_r
 
 @pytest.mark.parametrize("M,N,K", [(40, 200, 1208), (64, 6144, 4096), (100, 96, 520), (128, 130, 2048),
                                    # K in one piece (enough tiles without slices): 224 and 192 tiles; a last row tile of 44
-                                   (64, 28672, 520), (300, 8192, 264), (300, 2048, 1288)])
+                                   (64, 28672, 520), (300, 8192, 264), (300, 2048, 1288),
+                                   # SwiGLU on the 256-row tile with the norm's scale in its epilogue
+                                   (1024, 2 * 16640, 128)])
 def test_product_of_the_normalised_row_from_what_was_left_with_17_to_1024_rows(M, N, K):
     """On the tiled kernel, with K in slices (the finishing kernel scales) or whole (the product's epilogue does)."""
     t = tuned()
     whole = t._tiled_k_split(M, N, K) == 1
-    assert whole == ((M, N, K) in [(64, 28672, 520), (300, 8192, 264)])
+    assert whole == ((M, N, K) in [(64, 28672, 520), (300, 8192, 264), (1024, 2 * 16640, 128)])
     x = f64(gen(M, K, seed=1, scale=3.0))
     x[0, : K // 2] *= 40.0
     g = f64(1 + 0.2 * gen(K, seed=2))
@@ -282,7 +284,10 @@ def test_embedding_from_the_tiled_table():
 
 @pytest.mark.parametrize("M,F,K", [(1, 24, 64), (8, 176, 64), (9, 200, 120), (64, 512, 192), (65, 40, 72), (300, 520, 1024),
                                    (130, 200, 120), (300, 512, 192), (256, 14336 // 8, 512), (48, 176, 1032),
-                                   (100, 72, 2048), (300, 200, 320), (1000, 4096, 200), (1024, 4090, 128)])
+                                   (100, 72, 2048), (300, 200, 320), (1000, 4096, 200), (1024, 4090, 128),
+                                   # the 256-row tile (1,024 rows or more, K a multiple of 64, 512 tiles or more): last
+                                   # row tile of 76 rows, last column tile of 16 columns; one and three K steps
+                                   (2048, 8192, 128), (1100, 13200, 192), (1024, 16640, 64)])
 def test_swiglu_bf16(M, F, K):
     t = tuned()
     h = gen(M, K, seed=1, dtype=BF).to(DEV)
