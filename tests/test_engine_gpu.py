@@ -212,7 +212,7 @@ def test_widths_of_an_8b_model_in_bfloat16_against_the_32_bit_path():
                 if k.endswith("q_proj.weight") or k.endswith("k_proj.weight"):
                     v = (v.float() * sharpen).to(torch.bfloat16)
                 tensors[k] = v if dtype == torch.bfloat16 else v.float()
-        model.bind(tensors, Runtime(torch.device("cuda:0"), dtype, 1024))
+        model.bind(tensors, Runtime(torch.device("cuda:0"), dtype, 1280))
         return ModelRunner(model, 16, 192, 48, use_graphs=True)
 
     toks = H.random_tokens(V, 420, seed=5)
@@ -239,6 +239,10 @@ def test_widths_of_an_8b_model_in_bfloat16_against_the_32_bit_path():
         r.release("a")
         r.admit("c")
         out.append(("portion of 600 rows", r.step([Entry("c", (toks * 2)[:600], [0, 299, 599])])))
+        # 1,100 rows: SwiGLU on the tile of 256 rows for most of its columns and on the tile of 128 rows for the rest
+        r.release("c")
+        r.admit("d")
+        out.append(("portion of 1,100 rows", r.step([Entry("d", (toks * 3)[:1100], [0, 550, 1099])])))
         rows[dtype] = [(what, lg.float().cpu().numpy().astype(np.float64)) for what, lg in out]
         del r
         torch.cuda.empty_cache()
