@@ -18,6 +18,7 @@
 // Reference counterpart: gemm_nt_bf16_tiled_kernel, hip/src/kernels.cpp:634 (no matrix cores there).
 #include <type_traits>
 
+#include "gemm_wide.h"
 #include "mfma.h"
 
 constexpr int BN = 128, BK = 64;
@@ -285,174 +286,6 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
   }
 }
 
-// SwiGLU of many rows on a tile of 256 rows x (128 gate + 128 up) columns: 8 waves (2 along the rows x 4 along the
-// columns), a wave computes gate and up of 128 rows x 32 outputs as 4 x 2 accumulators.  Against the 128 x 128 tile
-// above an operand read from LDS feeds a third more arithmetic (6 reads for 8 MFMAs instead of 4 for 4), a tile of
-// the weights is stored into LDS once for 256 rows instead of 128, and the block's barrier comes after twice the
-// arithmetic: LDS traffic per MFMA falls from 1.5 KiB to 1 KiB, and LDS bandwidth is what bounds the smaller tile.
-// One block a compute unit (144 KiB of LDS), two waves a SIMD.  K must be a multiple of 64; the same loads two K
-// steps ahead, spread between the groups of MFMAs, as in gemm_bf16_kernel.
-constexpr int BIG_M = 256, BIG_THREADS = 512;
-#ifndef BIG_LOAD_GROUPS
-#define BIG_LOAD_GROUPS 2
-#endif
-#ifndef BIG_STORE_GROUPS
-#define BIG_STORE_GROUPS 2
-#endif
-template <bool PRE>
-__global__ __launch_bounds__(BIG_THREADS) void gemm_swiglu_big_kernel(const bf16_t* __restrict__ A, int lda,
-                                                                       const bf16_t* __restrict__ Wg,
-                                                                       const bf16_t* __restrict__ Wu, int chunks,
-                                                                       bf16_t* __restrict__ C, int ldc, int M, int F, int K,
-                                                                       TiledPre pre) {
-  __shared__ float rstd_s[PRE ? BIG_M : 1];
-  __shared__ __attribute__((aligned(16))) bf16_t As[2][BIG_M * LDS_ROW];
-  __shared__ __attribute__((aligned(16))) bf16_t Ws[2][256 * LDS_ROW];  // 128 gate rows, then the 128 up rows
-  constexpr int PIECES = 8;  // 4 pieces of A and 4 of W per thread and K step
-  const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
-  const int wm = wave / 4, wn = wave % 4;
-  int mt, nt;
-  {
-    // block order as in gemm_bf16_kernel: XCD x takes the column tiles x, x + 8, ..; groups of up to 8 row tiles
-    const int MT = ceil_div(M, BIG_M), NT = ceil_div(F, 128), NL = ceil_div(NT, 8);
-    constexpr int GM = 8;
-    const int xcd = blockIdx.x % 8, j = blockIdx.x / 8;
-    const int first_m = j / (GM * NL) * GM, gsz = min(MT - first_m, GM), jj = j % (GM * NL);
-    mt = first_m + jj % gsz;
-    nt = jj / gsz * 8 + xcd;
-    if (nt >= NT || mt >= MT) return;
-  }
-  const int m0 = mt * BIG_M, n0 = nt * 128;
-  const int lrow = tid / 8, lchunk = tid % 8;                                   // A: 64 rows a pass
-  const int wi = tid % 16, wc = (tid / 16) % 4, wkc = (tid / 64) % 2, wbl = tid / 128;  // W: 4 bands a pass
-  const int bands = (F + 15) / 16, band0 = n0 / 16;
-  // Loads go through buffer descriptors (the tile's base in scalar registers, a byte offset per thread that never
-  // changes, the K step as a scalar offset): no address arithmetic in vector registers.  Offsets stay far below 2 GiB
-  // (256 rows of A, 8 bands of W; checked by the host).
-  const BufferRsrc abuf = make_rsrc(A + (size_t)m0 * lda);
-  const BufferRsrc gbuf = make_rsrc(Wg + (size_t)band0 * chunks * 512);
-  const BufferRsrc ubuf = make_rsrc(Wu + (size_t)band0 * chunks * 512);
-  int aoff[4], woff[4];  // bytes
-#pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    aoff[p] = ((min(m0 + p * 64 + lrow, M - 1) - m0) * lda + lchunk * 8) * 2;
-    const int rel = (p % 2) * 4 + wbl;  // band of the 8 gate (passes 0, 1) or up (passes 2, 3) bands of the tile
-    woff[p] = ((min(band0 + rel, bands - 1) - band0) * chunks * 512 + wkc * 512 + (wc * 16 + wi) * 8) * 2;
-  }
-  floatx16 acc[4][2];
-#pragma unroll
-  for (int a = 0; a < 4; ++a)
-#pragma unroll
-    for (int b = 0; b < 2; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
-  auto load_piece = [&](GemmRegs<128>& g, int kt, int j) {
-    if (j < 4) g.a[j] = load_frag_buffer(abuf, aoff[j], kt * (BK * 2));
-    else g.w[j - 4] = load_frag_buffer(j - 4 < 2 ? gbuf : ubuf, woff[j - 4], kt * 2048);
-  };
-  auto store_piece = [&](const GemmRegs<128>& g, int buf, int j) {
-    if (j < 4) {
-      *reinterpret_cast<Frag*>(&As[buf][(j * 64 + lrow) * LDS_ROW + lchunk * 8]) = g.a[j];
-    } else {
-      const int p = j - 4;
-      *reinterpret_cast<Frag*>(&Ws[buf][((p * 4 + wbl) * 16 + wi) * LDS_ROW + wkc * 32 + wc * 8]) = g.w[p];
-    }
-  };
-  const int li = lane % 32, lc = lane / 32;
-  // One K step out of LDS buffer `buf` in four groups of 8 MFMAs.  With NEXT the next step's tile is on its way at
-  // the same time: its 8 pieces are asked for in front of the first two groups and stored into the other LDS buffer
-  // behind the last two.  One set of registers: two sets with loads two steps ahead, as in gemm_bf16_kernel, were
-  // slower here (649 against 533 us on the SwiGLU product of an 8B model at 2,048 rows), and so was keeping the one
-  // set busy for a whole step (595 us).
-  GemmRegs<128> regs;
-  auto step = [&](auto NEXT, int buf, int kt_next) {
-#pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      if constexpr (decltype(NEXT)::value) {
-        if (kk < BIG_LOAD_GROUPS) {
-#pragma unroll
-          for (int j = kk * (8 / BIG_LOAD_GROUPS); j < (kk + 1) * (8 / BIG_LOAD_GROUPS); ++j) load_piece(regs, kt_next, j);
-        }
-      }
-      Frag fw[2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t)  // tile 0 = gate rows wn*32.., tile 1 = the up rows of the same outputs
-        fw[t] = *reinterpret_cast<const Frag*>(&Ws[buf][(t * 128 + wn * 32 + li) * LDS_ROW + kk * 16 + lc * 8]);
-#pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        const Frag fa = *reinterpret_cast<const Frag*>(&As[buf][(wm * 128 + a * 32 + li) * LDS_ROW + kk * 16 + lc * 8]);
-#pragma unroll
-        for (int b = 0; b < 2; ++b) acc[a][b] = mfma32(fa, fw[b], acc[a][b]);
-      }
-      if constexpr (decltype(NEXT)::value) {
-        if (kk >= 4 - BIG_STORE_GROUPS) {
-          constexpr int per = 8 / BIG_STORE_GROUPS;
-          const int g = kk - (4 - BIG_STORE_GROUPS);
-#pragma unroll
-          for (int j = g * per; j < (g + 1) * per; ++j) store_piece(regs, buf ^ 1, j);
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);  // keeps each group's memory work in its group
-    }
-  };
-  constexpr std::true_type yes{};
-  constexpr std::false_type no{};
-  const int ktiles = K / BK;
-  if (ktiles > 0) {
-#pragma unroll
-    for (int j = 0; j < PIECES; ++j) load_piece(regs, 0, j);
-#pragma unroll
-    for (int j = 0; j < PIECES; ++j) store_piece(regs, 0, j);
-    if constexpr (PRE) {  // one row a thread, its parts added in order, 8 loads at a time
-      if (tid < BIG_M) {
-        const float* row = pre.ss + (size_t)min(m0 + tid, M - 1) * pre.parts;
-        float sum = 0.f;
-        for (int p0 = 0; p0 < pre.parts; p0 += 8) {
-          float v[8];
-#pragma unroll
-          for (int j = 0; j < 8; ++j) v[j] = p0 + j < pre.parts ? row[p0 + j] : 0.f;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) sum += v[j];
-        }
-        rstd_s[tid] = 1.0f / sqrtf(sum / (float)K + pre.eps);
-      }
-    }
-    __syncthreads();
-    int kt = 0;
-    while (kt + 2 < ktiles) {  // two steps a round: the LDS buffers take turns
-      step(yes, 0, kt + 1);
-      __syncthreads();
-      step(yes, 1, kt + 2);
-      __syncthreads();
-      kt += 2;
-    }
-    if (kt + 1 < ktiles) {
-      step(yes, 0, kt + 1);
-      __syncthreads();
-      step(no, 1, 0);
-    } else {
-      step(no, 0, 0);
-    }
-  }
-  // D[i][j]: lane holds column j = lane % 32 and rows (r/4)*8 + (lane/32)*4 + r%4 of each 32 x 32 accumulator
-  const int n = n0 + wn * 32 + li;
-#pragma unroll
-  for (int a = 0; a < 4; ++a) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int m = m0 + wm * 128 + a * 32 + (r / 4) * 8 + lc * 4 + (r % 4);
-      if (m >= M || n >= F) continue;
-      float g = acc[a][0][r], u = acc[a][1][r];
-      if constexpr (PRE) {
-        const float rs = rstd_s[m - m0];
-        g *= rs;
-        u *= rs;
-      }
-      C[(size_t)m * ldc + n] = float_to_bf16(silu_f(g) * u);
-    }
-  }
-}
-
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 template <int MODE, bool PRE = false>
@@ -463,16 +296,14 @@ static int launch_gemm(const bf16_t* A, int lda, const bf16_t* W, const bf16_t* 
     // From 1,024 rows on the tile of 256 rows x 128 outputs takes as many columns as make whole rounds of one tile a
     // compute unit (at least two rounds), and the 128-row tile, two blocks a unit and so finer grained, the rest:
     // 2,048 rows x 14,336 outputs are 3.5 rounds of big tiles, of which 3 run as such (96 of 112 column tiles).
-    const int MT = ceil_div(M, BIG_M), NT = ceil_div(N, 128);
+    const int MT = ceil_div(M, 256), NT = ceil_div(N, 128);
     const long rounds = (long)MT * NT / 256;
-    if (M >= 1024 && K % BK == 0 && rounds >= 2 && MT <= 256) {
+    if (M >= 1024 && K % BK == 0 && rounds >= 2 && MT <= 256 && (long)256 * lda * 2 < 0x7fffffffL) {
       const int cols_big = (int)((rounds * 256 / MT < NT ? rounds * 256 / MT : NT));  // column tiles of the big kernel
       const int n_big = cols_big * 128 < N ? cols_big * 128 : N;
-      const long big = 8L * ceil_div(cols_big, 8) * MT;
-      if (big > 0x7fffffffL) return APC_ERR_BAD_ARG;
-      hipLaunchKernelGGL((gemm_swiglu_big_kernel<PRE>), dim3((unsigned)big), dim3(BIG_THREADS), 0, stream, A, lda, W, W2,
-                         ceil_div(K, 32), (bf16_t*)C, ldc, M, n_big, K, pre);
-      APC_LAUNCH_CHECK();
+      const int e = launch_swiglu_wide(A, lda, W, W2, (bf16_t*)C, ldc, M, n_big, K, PRE ? pre.ss : nullptr, pre.parts,
+                                       pre.eps, stream);
+      if (e) return e;
       if (n_big == N) return 0;
       const size_t w_skip = (size_t)(n_big / 16) * ceil_div(K, 32) * 512;  // whole bands of the tiled layout
       W += w_skip;

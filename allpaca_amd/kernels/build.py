@@ -23,9 +23,9 @@ CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
 
 LIBS: Dict[str, List[str]] = {
     "plain": ["plain_ops.hip", "plain_gemm.hip", "plain_attention.hip", "sampling.hip"],
-    "tuned": ["gemm_bf16.hip", "skinny_gemm_bf16.hip", "attention_bf16.hip", "rope_bf16.hip"],
+    "tuned": ["gemm_bf16.hip", "gemm_wide_bf16.hip", "skinny_gemm_bf16.hip", "attention_bf16.hip", "rope_bf16.hip"],
 }
-HEADERS = ["common.h", "mfma.h"]
+HEADERS = ["common.h", "mfma.h", "gemm_wide.h"]
 
 ARCH = "gfx950"
 # -packed-fp32-ops is switched off for device code: some packed forms have given wrong results on this hardware.
@@ -35,6 +35,24 @@ ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-mllvm", "-amdgpu-mfma-vgpr-form=1",
          "-Wno-unused-result"]
+# Sources whose MFMA accumulators go into the accumulation registers (the compiler's default): a kernel there keeps 256
+# of them a wave, beside 256 vector registers for everything else.
+ACC_REGISTER_SOURCES = {"gemm_wide_bf16.hip"}
+VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
+
+
+def flags_for(src: str) -> List[str]:
+    if os.path.basename(src) not in ACC_REGISTER_SOURCES:
+        return list(FLAGS)
+    out, skip = [], 0
+    for i, f in enumerate(FLAGS):
+        if skip:
+            skip -= 1
+        elif FLAGS[i:i + 2] == VGPR_FORM:
+            skip = 1
+        else:
+            out.append(f)
+    return out
 
 
 class KernelBuildError(RuntimeError):
@@ -71,6 +89,7 @@ def _sources(name: str) -> List[str]:
 def source_hash(name: str) -> str:
     h = hashlib.sha256()
     h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(sorted(ACC_REGISTER_SOURCES)).encode())
     for path in _sources(name) + [os.path.join(CSRC, f) for f in HEADERS]:
         if os.path.isfile(path):
             h.update(os.path.basename(path).encode())
@@ -123,7 +142,7 @@ def build(name: str, force: bool = False, verbose: bool = True) -> str:
     def compile_one(src: str) -> str:
         # names of this process only: two processes may build the same library into the same folder at once
         obj = os.path.join(d, f"{name}_{os.path.splitext(os.path.basename(src))[0]}.{os.getpid()}.o")
-        cmd = [hipcc, *FLAGS, "-I", CSRC, "-c", src, "-o", obj]
+        cmd = [hipcc, *flags_for(src), "-I", CSRC, "-c", src, "-o", obj]
         p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         if p.returncode != 0:
             raise KernelBuildError(f"hipcc failed on {src}:\n{p.stdout}")
