@@ -114,13 +114,18 @@ def decode_run(eng, cfg, batch, context, steps, warmup):
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     n = 0
+    produced = {}
     for _ in range(steps):
-        n += len(eng.step())
+        events = eng.step()
+        n += len(events)
+        for ev in events:
+            produced.setdefault(ev.request_id, []).append(ev.token_id)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     assert n == batch * steps, f"{n} tokens from {steps} steps of batch {batch}"
     for rid in list(eng.requests):
         eng.abort(rid)
+    decode_run.ids_hash = ids_hash([produced[k] for k in sorted(produced)])   # of the timed steps' tokens
     return dt / steps
 
 
@@ -146,6 +151,15 @@ def prefill_run(eng, cfg, tokens, repeats=3):
     return best
 
 
+def ids_hash(token_lists):
+    """A short hash of produced token ids (requests in order): the same run gives the same hash."""
+    import hashlib
+    h = hashlib.sha256()
+    for toks in token_lists:
+        h.update((",".join(str(int(t)) for t in toks) + ";").encode())
+    return h.hexdigest()[:16]
+
+
 def requests_run(eng, cfg, n_requests, min_prompt, max_prompt, new_tokens, seed=0):
     """`n_requests` requests with prompts of random length arrive at once and run to `new_tokens` tokens each
     through the scheduler: portions of prompts beside decoding rows.  Returns a dict of totals and mean times."""
@@ -169,9 +183,13 @@ def requests_run(eng, cfg, n_requests, min_prompt, max_prompt, new_tokens, seed=
     times = [r.timing() for r in reqs]
     out_tokens = sum(len(r.output) for r in reqs)
     assert out_tokens == n_requests * new_tokens, f"{out_tokens} tokens from {n_requests} requests"
+    ttft = [1e3 * t["ttft"] for t in times]
+    itl = [1e3 * t["itl"] for t in times]
     return {"seconds": dt, "steps": steps, "prompt_tokens": sum(lengths), "output_tokens": out_tokens,
-            "ttft_ms": 1e3 * float(np.mean([t["ttft"] for t in times])),
-            "itl_ms": 1e3 * float(np.mean([t["itl"] for t in times])),
+            "ttft_ms": float(np.mean(ttft)), "itl_ms": float(np.mean(itl)),
+            "ttft_p50_ms": float(np.percentile(ttft, 50)), "ttft_p95_ms": float(np.percentile(ttft, 95)),
+            "itl_p50_ms": float(np.percentile(itl, 50)), "itl_p95_ms": float(np.percentile(itl, 95)),
+            "ids_hash": ids_hash([r.output for r in reqs]),
             "preemptions": eng.scheduler.preemption_count}
 
 
@@ -238,7 +256,10 @@ def main() -> int:
             "value": round(r["output_tokens"] / r["seconds"], 1), "unit": "tok/s", "n_gpus": 1,
             "seconds": round(r["seconds"], 3), "steps": r["steps"], "prompt_tokens": r["prompt_tokens"],
             "output_tokens": r["output_tokens"], "all_tokens_per_s": round((r["prompt_tokens"] + r["output_tokens"]) / r["seconds"], 1),
-            "mean_ttft_ms": round(r["ttft_ms"], 1), "mean_itl_ms": round(r["itl_ms"], 2), "preemptions": r["preemptions"],
+            "mean_ttft_ms": round(r["ttft_ms"], 1), "mean_itl_ms": round(r["itl_ms"], 2),
+            "ttft_p50_ms": round(r["ttft_p50_ms"], 1), "ttft_p95_ms": round(r["ttft_p95_ms"], 1),
+            "itl_p50_ms": round(r["itl_p50_ms"], 2), "itl_p95_ms": round(r["itl_p95_ms"], 2),
+            "ids_hash": r["ids_hash"], "preemptions": r["preemptions"],
             "graphs_captured_before": captured, "warm_up_seconds": round(warm, 2),
             "dtype": args.dtype, "data": "synthetic: random N(0, 0.02) weights, uniform random token ids",
             "config": {"model": args.preset, "layers": layers, "layers_of_configuration": full_layers,
@@ -270,6 +291,7 @@ def main() -> int:
         sec = decode_run(eng, cfg, b, args.context, args.steps, args.warmup)
         ms[b] = sec * 1e3
         if b == args.batch:
+            main_hash = decode_run.ids_hash
             wbytes = weight_bytes(eng)
             ctx_mid = args.context + args.warmup + args.steps // 2
             total = wbytes + b * ctx_mid * kv_bytes_per_token(cfg, layers, 2 if args.dtype == "bf16" else 4)
@@ -304,6 +326,7 @@ def main() -> int:
             "graphs": not args.no_graphs,
         },
     }
+    out["ids_hash"] = main_hash      # of the tokens the timed steps produced (greedy): the same run, the same hash
     if prefill:
         out["prefill"] = prefill
     if roof:
