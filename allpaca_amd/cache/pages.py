@@ -47,6 +47,7 @@ class PagePool:
         self._free: List[int] = list(range(num_pages - 1, -1, -1))  # page 0 goes out first
         self._held = [False] * num_pages
         self.allocations = 0   # how many times a page was handed out (reuse shows as allocations > num_pages)
+        self.on_free = None    # called with the id of every page that comes back (a debugging aid: see CacheStorage)
 
     @property
     def free_count(self) -> int:
@@ -69,6 +70,8 @@ class PagePool:
             raise CacheError(f"page {page} freed twice")
         self._held[page] = False
         self._free.append(page)
+        if self.on_free is not None:
+            self.on_free(page)
 
     def held(self) -> List[int]:
         return [p for p, h in enumerate(self._held) if h]

@@ -68,6 +68,17 @@ class CacheStorage:
         self.state: List[torch.Tensor] = [torch.zeros(sh, dtype=_DTYPES[g.need.dtype], device=device)
                                           for sh, g in zip(state_shapes, manager.state_groups)]
 
+    def poison_free_pages(self, value: float = 1e30) -> None:
+        """A debugging aid against stale reads: every page that is free, now and whenever one comes back, is filled
+        with `value` (large and finite: a masked position multiplies what it reads by 0), so that a key or value
+        read from a page that the request has not written itself shows in the logits at once."""
+        for t, g in zip(self.paged, self.manager.paged_groups):
+            held = set(g.pool.held())
+            for page in range(g.pool.num_pages):
+                if page not in held:
+                    t[:, page].fill_(value)
+            g.pool.on_free = lambda page, t=t: t[:, page].fill_(value)
+
     def dummy_page(self, group: int) -> int:
         return self.manager.paged_groups[group].pool.num_pages
 

@@ -10,6 +10,7 @@ mixes a prompt portion with decode rows in one of them
 from __future__ import annotations
 
 import gc
+import os
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
@@ -26,13 +27,15 @@ class StepError(ValueError):
 
 class ModelRunner:
     def __init__(self, model: DecoderModel, page_tokens: int, num_pages, max_requests: int,
-                 kv_dtype: Optional[torch.dtype] = None, use_graphs: bool = False):
+                 kv_dtype: Optional[torch.dtype] = None, use_graphs: bool = False, poison_free_pages: bool = False):
         if model.rt is None:
             raise StepError("the model has no weights bound")
         self.model = model
         self.rt = model.rt
         self.cache = CacheManager(model.cache_needs(), page_tokens, num_pages, max_requests)
         self.storage = CacheStorage(self.cache, kv_dtype or self.rt.dtype, self.rt.device)
+        if poison_free_pages or os.environ.get("ALLPACA_POISON_FREE_PAGES") == "1":
+            self.storage.poison_free_pages()
         self.views = self.storage.views(model.spec.plan)
         self.pad_pages = [self.storage.dummy_page(g) for g in range(len(self.cache.paged_groups))]
         self.vocab_size = model.spec.vocab_size

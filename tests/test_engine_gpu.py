@@ -15,11 +15,11 @@ DTYPES = ["float32", "bfloat16"]
 TORCH = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
 
-def make_runner(folder, dtype, page_tokens=16, num_pages=64, max_requests=8, max_positions=None):
+def make_runner(folder, dtype, page_tokens=16, num_pages=64, max_requests=8, max_positions=None, poison=False):
     from allpaca_amd.engine.runner import ModelRunner
     from allpaca_amd.models import load_model
     cfg, model = load_model(folder, TORCH[dtype], "cuda:0", max_positions=max_positions)
-    return cfg, ModelRunner(model, page_tokens, num_pages, max_requests)
+    return cfg, ModelRunner(model, page_tokens, num_pages, max_requests, poison_free_pages=poison)
 
 
 def run_cut(runner, seq, tokens, cuts):
@@ -112,7 +112,9 @@ def test_mixed_batches_with_page_reuse(name, dtype):
     page_tokens = 16
     worst = sorted(lengths)[-4:]
     num_pages = sum(-(-n // page_tokens) for n in worst)
-    cfg, runner = make_runner(folder, dtype, page_tokens=page_tokens, num_pages=num_pages)
+    # free pages are filled with 1e30, at the start and whenever one comes back: a key or value read from a page
+    # before its new owner wrote it would show in the logits
+    cfg, runner = make_runner(folder, dtype, page_tokens=page_tokens, num_pages=num_pages, poison=True)
     toks = [H.random_tokens(cfg.vocab_size, n, seed=100 + i) for i, n in enumerate(lengths)]
     got = {i: [] for i in range(len(lengths))}
     for entries, ends in mixed_schedule(lengths, seed=7):
@@ -130,6 +132,7 @@ def test_mixed_batches_with_page_reuse(name, dtype):
             runner.release(i)
         runner.cache.check()
     assert runner.cache.paged_groups[0].pool.allocations > num_pages, "the schedule did not reuse pages"
+    assert bool((runner.storage.paged[0][:, :num_pages].float() > 1e29).all()), "pages that came back are not filled"
     for i, n in enumerate(lengths):
         H.check_logits(np.concatenate(got[i]), folder, toks[i], dtype, f"{name} mixed request {i}")
     assert runner.cache.free_pages(0) == num_pages

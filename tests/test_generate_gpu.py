@@ -153,7 +153,8 @@ def test_command_line_generate():
 
 def replay(folder, dtype, steps, max_tokens, out_dir, page_tokens=16):
     cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
-           "--out", out_dir, "--max-tokens", str(max_tokens), "--page-tokens", str(page_tokens)]
+           "--out", out_dir, "--max-tokens", str(max_tokens), "--page-tokens", str(page_tokens),
+           "--poison-free-pages"]     # free pages hold 1e30: a read of a page before its owner wrote it would show
     text = "".join(json.dumps(s) + "\n" for s in steps)
     r = subprocess.run(cmd, input=text, capture_output=True, text=True, timeout=280)
     assert r.returncode == 0, r.stderr[-3000:]
