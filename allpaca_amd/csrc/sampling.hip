@@ -11,7 +11,9 @@
 // The random number is an input, so a token depends on (seed, request, position)
 // only, never on the batch.
 #include "common.h"
+#include "no_alloc.h"
 #include <math.h>
+#include <mutex>
 
 constexpr int SNT = 256;
 constexpr int SMALL_MAX = 1024;  // survivors of top-k handled in LDS in the reference's own sequential order
@@ -232,6 +234,53 @@ APC_EXPORT int apc_argmax_rows(const float* logits, int ldl, int n_rows, int V, 
   hipLaunchKernelGGL(argmax_pieces_kernel, dim3(n_rows, pieces), dim3(SNT), 0, stream, logits, ldl, V, piece, pv, pi);
   APC_LAUNCH_CHECK();
   hipLaunchKernelGGL(argmax_final_kernel, dim3(n_rows), dim3(WAVE), 0, stream, pv, pi, pieces, out);
+  APC_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---- the variant that allocates nothing (declared in no_alloc.h) ----
+// Room for the pieces of APC_ARGMAX_NO_ALLOC_MAX_ROWS rows: values [rows][64], then indices [rows][64].  Each GPU holds
+// its own copy of the array at its own address; in host code the array's name is not that address, so the address is
+// asked for once per device (hipGetSymbolAddress, with that device current) and only the answer is handed to kernels.
+constexpr int NO_ALLOC_PIECES = 64;
+static __device__ __align__(256) unsigned char argmax_scratch[(size_t)APC_ARGMAX_NO_ALLOC_MAX_ROWS * NO_ALLOC_PIECES * 8];
+constexpr int NO_ALLOC_MAX_DEVICES = 64;
+static void* argmax_scratch_ptr[NO_ALLOC_MAX_DEVICES];  // per device, null until its first call
+static std::mutex argmax_scratch_lock;
+
+APC_EXPORT int apc_argmax_rows_no_alloc(const float* logits, int ldl, int n_rows, int V, int* out,
+                                        hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (V <= 0 || ldl < V || !logits || !out) return APC_ERR_BAD_ARG;
+  if (n_rows > APC_ARGMAX_NO_ALLOC_MAX_ROWS) return APC_ERR_TOO_LARGE;
+  if (V < 8192) {  // one block a row: no pieces, nothing beyond input and output
+    hipLaunchKernelGGL(argmax_rows_kernel, dim3(n_rows), dim3(SNT), 0, stream, logits, ldl, V, out);
+    APC_LAUNCH_CHECK();
+    return 0;
+  }
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= NO_ALLOC_MAX_DEVICES) return APC_ERR_UNSUPPORTED;
+  void* ptr;
+  {
+    std::lock_guard<std::mutex> hold(argmax_scratch_lock);
+    if (!argmax_scratch_ptr[dev]) {
+      void* p = nullptr;
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(argmax_scratch));
+      if (e != hipSuccess) return (int)e;
+      if (!p) return (int)hipErrorInvalidSymbol;
+      argmax_scratch_ptr[dev] = p;
+    }
+    ptr = argmax_scratch_ptr[dev];
+  }
+  const int piece = ceil_div(V, NO_ALLOC_PIECES);
+  float* pv = (float*)ptr;
+  int* pi = (int*)ptr + (size_t)n_rows * NO_ALLOC_PIECES;
+  hipLaunchKernelGGL(argmax_pieces_kernel, dim3(n_rows, NO_ALLOC_PIECES), dim3(SNT), 0, stream, logits, ldl, V, piece,
+                     pv, pi);
+  APC_LAUNCH_CHECK();
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(n_rows), dim3(WAVE), 0, stream, pv, pi, NO_ALLOC_PIECES, out);
   APC_LAUNCH_CHECK();
   return 0;
 }

@@ -25,7 +25,7 @@ LIBS: Dict[str, List[str]] = {
     "plain": ["plain_ops.hip", "plain_gemm.hip", "plain_attention.hip", "sampling.hip"],
     "tuned": ["gemm_bf16.hip", "gemm_wide_bf16.hip", "skinny_gemm_bf16.hip", "attention_bf16.hip", "rope_bf16.hip"],
 }
-HEADERS = ["common.h", "mfma.h", "gemm_wide.h"]
+HEADERS = ["common.h", "mfma.h", "gemm_wide.h", "no_alloc.h"]
 
 ARCH = "gfx950"
 # -packed-fp32-ops is switched off for device code: some packed forms have given wrong results on this hardware.

@@ -35,6 +35,7 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_gemm_plain": [P, I, I, P, I, I, P, I, I, I, I, I, I, P],
         "apc_paged_attention_plain": [P, I, I, I, P, I, I, I, I, I, I, P, I, I, P, I, P, P, I, F, P],
         "apc_argmax_rows": [P, I, I, I, P, P, P],
+        "apc_argmax_rows_no_alloc": [P, I, I, I, P, P],
         "apc_sample_rows": [P, I, I, I, P, P, P, P, P, P],
     },
     "tuned": {
@@ -60,7 +61,8 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 
-ERRORS = {-1: "bad argument (shape or stride the kernel does not accept)", -2: "size not supported by this kernel"}
+ERRORS = {-1: "bad argument (shape or stride the kernel does not accept)", -2: "size not supported by this kernel",
+          -3: "more rows than the entry point that allocates nothing has room for"}
 
 
 def load(name: str) -> ctypes.CDLL:
