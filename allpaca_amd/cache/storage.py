@@ -70,8 +70,9 @@ class CacheStorage:
 
     def poison_free_pages(self, value: float = 1e30) -> None:
         """A debugging aid against stale reads: every page that is free, now and whenever one comes back, is filled
-        with `value` (large and finite: a masked position multiplies what it reads by 0), so that a key or value
-        read from a page that the request has not written itself shows in the logits at once."""
+        with `value`, so that a key or value read from a page that the request has not written itself shows in the
+        logits at once.  The default is large and finite; with NaN even a stale value that is multiplied by a weight
+        of 0 shows (no kernel may let one into a product)."""
         for t, g in zip(self.paged, self.manager.paged_groups):
             held = set(g.pool.held())
             for page in range(g.pool.num_pages):

@@ -40,6 +40,18 @@ __device__ __forceinline__ float row4_sum(float v) {
   return v + __shfl_xor(v, 32, WAVE);
 }
 __device__ __forceinline__ uint32_t bf16_pair(float a, float b) { return pack_bf16x2(a, b); }
+// A value operand holds 8 consecutive positions of one element.  Positions beyond the row's last key lie in slots
+// that nobody has written since the page's last owner, positions in front of a window's first key may lie in the
+// spare page that stands in for pages given back.  Their weight in P is 0, but 0 x NaN is NaN, so all but the
+// positions lo <= p < hi of the 8 are cleared before the product sees them.
+__device__ __forceinline__ void keep_positions(Frag& v, int lo, int hi) {
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const uint32_t a = (2 * w >= lo && 2 * w < hi) ? 0x0000ffffu : 0u;
+    const uint32_t b = (2 * w + 1 >= lo && 2 * w + 1 < hi) ? 0xffff0000u : 0u;
+    v.w[w] &= a | b;
+  }
+}
 // 2^x for x <= 0 (or -inf): the bare instruction, without the range handling that large arguments need
 __device__ __forceinline__ float exp2_neg(float x) { return __builtin_amdgcn_exp2f(x); }
 constexpr float LOG2E = 1.4426950408889634f;
@@ -142,8 +154,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   int page_next = 0;  // page of this thread's group in the tile that is loaded next
   auto lookup_tile = [&](int t0) { page_next = bt[min(t0 + grp * 8, last_group) / P]; };
   Frag kreg[PIECES], vreg[PIECES];
+  int v_lo = 0, v_hi = 8;
   auto load_tile = [&](int t0) {  // uses the page found by the last lookup_tile, which was for this t0
     const int tg = min(t0 + grp * 8, last_group), slot0 = tg % P;
+    v_lo = first - tg;       // the group's positions v_lo <= p < v_hi can be seen by a row of the tile
+    v_hi = last - tg + 1;
     const bf16_t* kp = k_head + (size_t)page_next * page_stride + (size_t)slot0 * d;
     const bf16_t* vp = v_head + (size_t)page_next * page_stride + slot0;
 #pragma unroll
@@ -157,6 +172,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 #pragma unroll
     for (int j = 0; j < PIECES; ++j) {
       if (on[j]) {
+        if (v_lo > 0 || v_hi < 8) keep_positions(vreg[j], v_lo, v_hi);
         *reinterpret_cast<Frag*>(Ks + k_ldst[j]) = kreg[j];
         *reinterpret_cast<Frag*>(Vs + v_ldst[j]) = vreg[j];
       }
@@ -359,8 +375,11 @@ __global__ __launch_bounds__(256) void attn_prefill32_kernel(
   int page_next = 0;
   auto lookup_tile = [&](int t0) { page_next = bt[min(t0 + grp * 8, last_group) / P]; };
   Frag kreg[PIECES], vreg[PIECES];
+  int v_lo = 0, v_hi = 8;
   auto load_tile = [&](int t0) {
     const int tg = min(t0 + grp * 8, last_group), slot0 = tg % P;
+    v_lo = first - tg;       // the group's positions v_lo <= p < v_hi can be seen by a row of the tile
+    v_hi = last - tg + 1;
     const bf16_t* kp = k_head + (size_t)page_next * page_stride + (size_t)slot0 * d;
     const bf16_t* vp = v_head + (size_t)page_next * page_stride + slot0;
 #pragma unroll
@@ -374,6 +393,7 @@ __global__ __launch_bounds__(256) void attn_prefill32_kernel(
 #pragma unroll
     for (int j = 0; j < PIECES; ++j) {
       if (on[j]) {
+        if (v_lo > 0 || v_hi < 8) keep_positions(vreg[j], v_lo, v_hi);
         *reinterpret_cast<Frag*>(Ks + k_ldst[j]) = kreg[j];
         uint2 a, b;
         a.x = vreg[j].w[0];
@@ -581,7 +601,15 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(
 
   // lane holds keys kb + nt*16 + lc*4 + r (scores) and elements dt*16 + lc*4 + r (output) of head li of the group
   const float sc2 = scale * LOG2E;
-  auto step = [&](const KVRegs<DP>& r, int kb) {
+  auto step = [&](KVRegs<DP>& r, int kb) {
+    if (kb + 31 > pos || kb < first) {  // a step with positions the row does not see (see keep_positions)
+      const int tv = min(kb + lc * 8, (pos / 8) * 8);  // as load_kv placed this lane's 8 positions
+      const int lo = first - tv, hi = pos - tv + 1;
+      if (lo > 0 || hi < 8) {
+#pragma unroll
+        for (int dt = 0; dt < DP / 16; ++dt) keep_positions(r.v[dt], lo, hi);
+      }
+    }
     floatx4 s[2];
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {

@@ -27,14 +27,17 @@ class StepError(ValueError):
 
 class ModelRunner:
     def __init__(self, model: DecoderModel, page_tokens: int, num_pages, max_requests: int,
-                 kv_dtype: Optional[torch.dtype] = None, use_graphs: bool = False, poison_free_pages: bool = False):
+                 kv_dtype: Optional[torch.dtype] = None, use_graphs: bool = False, poison_free_pages=False):
         if model.rt is None:
             raise StepError("the model has no weights bound")
         self.model = model
         self.rt = model.rt
         self.cache = CacheManager(model.cache_needs(), page_tokens, num_pages, max_requests)
         self.storage = CacheStorage(self.cache, kv_dtype or self.rt.dtype, self.rt.device)
-        if poison_free_pages or os.environ.get("ALLPACA_POISON_FREE_PAGES") == "1":
+        # a debugging aid: True fills free pages with 1e30, a number (NaN too) with that number
+        if poison_free_pages is not False and poison_free_pages is not None and poison_free_pages != 0:
+            self.storage.poison_free_pages(1e30 if poison_free_pages is True else float(poison_free_pages))
+        elif os.environ.get("ALLPACA_POISON_FREE_PAGES") == "1":
             self.storage.poison_free_pages()
         self.views = self.storage.views(model.spec.plan)
         self.pad_pages = [self.storage.dummy_page(g) for g in range(len(self.cache.paged_groups))]

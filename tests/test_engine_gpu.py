@@ -102,9 +102,9 @@ def mixed_schedule(lengths, seed, live_max=4):
     return steps
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B", "C"])
-def test_mixed_batches_with_page_reuse(name, dtype):
+def run_mixed(name, dtype, poison):
+    """The mixed schedule of test_mixed_batches_with_page_reuse; returns the runner, the tokens and every request's
+    logits.  `poison`: what free pages are filled with, at the start and whenever one comes back (False: nothing)."""
     from allpaca_amd.engine.batch import Entry
     folder = H.model_folder(name, dtype, True)
     lengths = {"A": [33, 100, 16, 7, 64, 1, 90, 50], "B": [150, 2, 77, 40, 120, 33, 9], "C": [129, 64, 5, 200, 31, 90]}[name]
@@ -112,9 +112,7 @@ def test_mixed_batches_with_page_reuse(name, dtype):
     page_tokens = 16
     worst = sorted(lengths)[-4:]
     num_pages = sum(-(-n // page_tokens) for n in worst)
-    # free pages are filled with 1e30, at the start and whenever one comes back: a key or value read from a page
-    # before its new owner wrote it would show in the logits
-    cfg, runner = make_runner(folder, dtype, page_tokens=page_tokens, num_pages=num_pages, poison=True)
+    cfg, runner = make_runner(folder, dtype, page_tokens=page_tokens, num_pages=num_pages, poison=poison)
     toks = [H.random_tokens(cfg.vocab_size, n, seed=100 + i) for i, n in enumerate(lengths)]
     got = {i: [] for i in range(len(lengths))}
     for entries, ends in mixed_schedule(lengths, seed=7):
@@ -132,10 +130,36 @@ def test_mixed_batches_with_page_reuse(name, dtype):
             runner.release(i)
         runner.cache.check()
     assert runner.cache.paged_groups[0].pool.allocations > num_pages, "the schedule did not reuse pages"
-    assert bool((runner.storage.paged[0][:, :num_pages].float() > 1e29).all()), "pages that came back are not filled"
-    for i, n in enumerate(lengths):
-        H.check_logits(np.concatenate(got[i]), folder, toks[i], dtype, f"{name} mixed request {i}")
     assert runner.cache.free_pages(0) == num_pages
+    return folder, runner, toks, [np.concatenate(got[i]) for i in range(len(lengths))]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_batches_with_page_reuse(name, dtype):
+    # free pages are filled with 1e30, at the start and whenever one comes back: a key or value read from a page
+    # before its new owner wrote it would show in the logits
+    folder, runner, toks, got = run_mixed(name, dtype, True)
+    n = runner.cache.paged_groups[0].pool.num_pages
+    assert bool((runner.storage.paged[0][:, :n].float() > 1e29).all()), "pages that came back are not filled"
+    for i, t in enumerate(toks):
+        H.check_logits(got[i], folder, t, dtype, f"{name} mixed request {i}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_nan_in_free_pages_changes_no_bit(name, dtype):
+    """A page that comes back may hold anything, NaN too (a request whose activations blew up), and a slot beyond a
+    row's last key gets a weight of 0 in the value product: 0 x NaN would be NaN, for this request and, through
+    what it writes, for the next owner of its pages.  With NaN in every free page the logits are the same, bit for
+    bit, as with pages that hold zeros."""
+    _, _, _, clean = run_mixed(name, dtype, False)
+    _, runner, _, dirty = run_mixed(name, dtype, float("nan"))
+    n = runner.cache.paged_groups[0].pool.num_pages
+    assert bool(torch.isnan(runner.storage.paged[0][:, :n].float()).all()), "pages that came back are not filled"
+    for i, (a, b) in enumerate(zip(clean, dirty)):
+        assert np.isfinite(b).all(), f"{name} request {i}: non-finite logits with NaN in free pages"
+        assert np.array_equal(a, b), f"{name} request {i}: NaN in free pages changed the logits"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -189,13 +213,16 @@ def test_a_far_key_is_found(dtype):
     assert np.abs(H.oracle_logits(path, without)[-1] - want[-1]).max() > 0.1
 
 
-def test_widths_of_an_8b_model_in_bfloat16_against_the_32_bit_path():
+def test_widths_of_an_8b_model_against_the_plain_implementation_and_between_the_paths():
     """The tiny configurations do not reach the code paths that sizes choose (bands per block, waves per block,
-    K in slices or whole, the fused product for q, k, v with d = 128): two layers at the widths of an 8B model
-    (hidden 4096, 32 heads over 8 of 128, feed-forward 14336; a small vocabulary), weights made on the GPU, the
-    same bfloat16 values in both runs.  A whole portion, a mixed step, decode steps (replayed graphs) and a portion
-    behind them: every row's logits are within the storage noise of two layers of the 32-bit path's, and no path
-    is further off than the others."""
+    K in slices or whole, the fused product for q, k, v with d = 128, the llama3 table of a real model): two layers
+    at the widths of an 8B model (hidden 4096, 32 heads over 8 of 128, feed-forward 14336; a small vocabulary),
+    weights made on the GPU, the same bfloat16 values in both runs.  A whole portion, a mixed step, decode steps
+    (replayed graphs) and a portion behind them are compared with the plain implementation on the same values, in
+    32-bit and in bfloat16; further steps (42 decode rows, 600 and 1,100 rows) between the two paths: every row's
+    logits are within the storage noise of two layers of the 32-bit path's, and no path is further off than the
+    others."""
+    import plain_llama as P
     from allpaca_amd.config import preset
     from allpaca_amd.engine.batch import Entry
     from allpaca_amd.engine.runner import ModelRunner
@@ -205,6 +232,7 @@ def test_widths_of_an_8b_model_in_bfloat16_against_the_32_bit_path():
     V = 8200
     cfg_json = dict(preset("llama-3.1-8b"), num_hidden_layers=2, vocab_size=V)
     sharpen = (3.0 / (0.02 ** 2 * cfg_json["hidden_size"])) ** 0.5      # scores of deviation ~3, as in helpers.model_folder
+    plain_weights = {}
 
     def runner(dtype):
         _, _, spec = describe_model(cfg_json)
@@ -215,42 +243,71 @@ def test_widths_of_an_8b_model_in_bfloat16_against_the_32_bit_path():
                 if k.endswith("q_proj.weight") or k.endswith("k_proj.weight"):
                     v = (v.float() * sharpen).to(torch.bfloat16)
                 tensors[k] = v if dtype == torch.bfloat16 else v.float()
+                if k not in plain_weights:
+                    plain_weights[k] = v.float().cpu().numpy()           # the plain side widens them itself
         model.bind(tensors, Runtime(torch.device("cuda:0"), dtype, 1280))
         return ModelRunner(model, 16, 192, 48, use_graphs=True)
 
     toks = H.random_tokens(V, 420, seed=5)
     rows = {}
+    fed = {}      # request -> its tokens so far
     for dtype in (torch.float32, torch.bfloat16):
         r = runner(dtype)
+        fed.clear()
+        out = []
+
+        def step(what, entries):
+            where = []
+            for e in entries:
+                have = fed.setdefault(e.seq, [])
+                where += [(e.seq, len(have) + w) for w in e.want]
+                have += list(e.tokens)
+            out.append((what, r.step(entries).float().cpu().numpy().astype(np.float64), where))
+
         r.admit("a")
         r.admit("b")
-        out = [("whole portion", r.step([Entry("a", toks[:300], list(range(300)))]))]
-        out.append(("mixed step", r.step([Entry("a", toks[300:340], list(range(40))), Entry("b", toks[:17], list(range(17)))])))
+        step("whole portion", [Entry("a", toks[:300], list(range(300)))])
+        step("mixed step", [Entry("a", toks[300:340], list(range(40))), Entry("b", toks[:17], list(range(17)))])
         for j in range(6):
-            out.append(("decode step", r.step([Entry("a", [toks[340 + j]], [0]), Entry("b", [toks[17 + j]], [0])])))
-        out.append(("portion behind", r.step([Entry("a", toks[346:400], [0, 53]), Entry("b", toks[23:24], [0])])))
+            step("decode step", [Entry("a", [toks[340 + j]], [0]), Entry("b", [toks[17 + j]], [0])])
+        step("portion behind", [Entry("a", toks[346:400], [0, 53]), Entry("b", toks[23:24], [0])])
         assert r.graph_replays == 6
         # 40 more requests: a mixed step of 160 rows, two decode steps of 42 rows (the tiled product with K in slices
         # and the folded norm in its finishing kernel), and a portion of 600 rows (K in slices for the narrow matrices)
         more = [f"m{i}" for i in range(40)]
         for m in more:
             r.admit(m)
-        out.append(("many short prompts", r.step([Entry(m, toks[i:i + 4], [3]) for i, m in enumerate(more)])))
+        step("many short prompts", [Entry(m, toks[i:i + 4], [3]) for i, m in enumerate(more)])
         for j in range(2):
-            out.append(("decode step of 42 rows", r.step([Entry("a", [toks[400 + j]], [0]), Entry("b", [toks[24 + j]], [0])]
-                                                          + [Entry(m, [toks[i + 4 + j]], [0]) for i, m in enumerate(more)])))
+            step("decode step of 42 rows", [Entry("a", [toks[400 + j]], [0]), Entry("b", [toks[24 + j]], [0])]
+                 + [Entry(m, [toks[i + 4 + j]], [0]) for i, m in enumerate(more)])
         r.release("a")
         r.admit("c")
-        out.append(("portion of 600 rows", r.step([Entry("c", (toks * 2)[:600], [0, 299, 599])])))
+        step("portion of 600 rows", [Entry("c", (toks * 2)[:600], [0, 299, 599])])
         # 1,100 rows: SwiGLU on the tile of 256 rows for most of its columns and on the tile of 128 rows for the rest
         r.release("c")
         r.admit("d")
-        out.append(("portion of 1,100 rows", r.step([Entry("d", (toks * 3)[:1100], [0, 550, 1099])])))
-        rows[dtype] = [(what, lg.float().cpu().numpy().astype(np.float64)) for what, lg in out]
+        step("portion of 1,100 rows", [Entry("d", (toks * 3)[:1100], [0, 550, 1099])])
+        rows[dtype] = out
         del r
         torch.cuda.empty_cache()
+    # against the plain implementation: requests a and b (402 and 26 tokens), every row that was asked for
+    exact = {s: P.llama_forward(cfg_json, plain_weights, fed[s]) for s in ("a", "b")}
+    noisy = {s: P.llama_forward(cfg_json, plain_weights, fed[s], store=P.round_bf16) for s in ("a", "b")}
+    for dtype, name in ((torch.float32, "float32"), (torch.bfloat16, "bfloat16")):
+        for what, lg, where in rows[dtype]:
+            keep = [i for i, (s, _) in enumerate(where) if s in exact]
+            if not keep:
+                continue
+            want = np.stack([exact[where[i][0]][where[i][1]] for i in keep])
+            noise = np.stack([noisy[where[i][0]][where[i][1]] for i in keep])
+            if name == "float32":
+                # the bound of the tiny models (2e-5 on logits of magnitude 0.3), relative to these logits' size
+                assert np.abs(lg[keep] - want).max() <= H.F32_ATOL / 0.3 * np.abs(want).max(), what
+            else:
+                H.assert_close(lg[keep], want, name, f"8B widths, {what}", noise)
     errs = []
-    for (what, a), (_, b) in zip(rows[torch.float32], rows[torch.bfloat16]):
+    for (what, a, _), (_, b, _) in zip(rows[torch.float32], rows[torch.bfloat16]):
         e = np.sqrt(((a - b) ** 2).mean(axis=1)) / np.sqrt((a ** 2).mean(axis=1))
         errs.append((what, float(e.max()), float(e.mean())))
     # measured: 0.016 on average, 0.021 at most, the same on every path

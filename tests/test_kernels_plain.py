@@ -144,13 +144,14 @@ def test_silu_mul_and_add():
     close(f64(acc), want, atol=1e-6, rtol=1e-6)
 
 
-def make_cache(n_seq_tokens, Hk, d, P_, dtype, seed=0, shuffle=True):
-    """Random keys/values for sequences of the given lengths laid into pages in a shuffled order."""
+def make_cache(n_seq_tokens, Hk, d, P_, dtype, seed=0, shuffle=True, stale=0.0):
+    """Random keys/values for sequences of the given lengths laid into pages in a shuffled order.  `stale`: what
+    the slots beyond a sequence's last position and the three pages that belong to no sequence hold."""
     rng = np.random.default_rng(seed)
     n_blocks = [-(-n // P_) for n in n_seq_tokens]
     total = sum(n_blocks)
     ids = rng.permutation(total + 3) if shuffle else np.arange(total + 3)
-    cache = torch.zeros(total + 3, 2, Hk, P_, d, dtype=dtype)
+    cache = torch.full((total + 3, 2, Hk, P_, d), stale, dtype=dtype)
     bt = np.zeros((len(n_seq_tokens), max(n_blocks)), np.int32)
     ks, vs = [], []
     at = 0
@@ -165,7 +166,7 @@ def make_cache(n_seq_tokens, Hk, d, P_, dtype, seed=0, shuffle=True):
             bt[s, b] = page
             lo, hi = b * P_, min(n, (b + 1) * P_)
             cache[page, 0, :, : hi - lo] = k[lo:hi].permute(1, 0, 2)
-            vt = torch.zeros(Hk, d, P_, dtype=dtype)          # values lie [element][slot] inside a page
+            vt = torch.full((Hk, d, P_), stale, dtype=dtype)   # values lie [element][slot] inside a page
             vt[:, :, : hi - lo] = v[lo:hi].permute(1, 2, 0)
             cache[page, 1] = vt.reshape(Hk, P_, d)
     return cache.to(DEV), torch.from_numpy(bt).to(DEV), ks, vs

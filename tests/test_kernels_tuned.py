@@ -423,15 +423,23 @@ def test_product_for_q_k_v_that_rotates_declines_what_it_does_not_take():
                                   torch.zeros(17, dtype=torch.int32, device=DEV), bt, cache2, P_)
 
 
-def run_attention(H, Hk, d, P_, lens, rows_per_seg, window=0, seed=0):
-    """Sequences of `lens` keys in the cache; the last `rows_per_seg[s]` positions of sequence s are the step's rows."""
+def run_attention(H, Hk, d, P_, lens, rows_per_seg, window=0, seed=0, stale=0.0):
+    """Sequences of `lens` keys in the cache; the last `rows_per_seg[s]` positions of sequence s are the step's rows.
+    `stale`: what lies in the slots beyond a sequence's last key and in the spare page; with a window, the pages that
+    every row of the step has passed are marked as given back in the block table (the spare page stands in)."""
     from allpaca_amd.engine.batch import Entry, pack_step
     t = tuned()
-    cache, bt, ks, vs = make_cache(lens, Hk, d, P_, BF, seed=seed)
+    cache, bt, ks, vs = make_cache(lens, Hk, d, P_, BF, seed=seed, stale=stale)
     pos0 = [n - r for n, r in zip(lens, rows_per_seg)]
     entries = [Entry(i, [0] * r, []) for i, r in enumerate(rows_per_seg)]
     tables = [[list(bt[i, : -(-n // P_)].cpu().numpy()) for i, n in enumerate(lens)]]
-    step = pack_step(entries, pos0, [0] * len(lens), tables, torch.device(DEV), [0])
+    used = {int(p) for tb in tables[0] for p in tb}
+    spare = min(set(range(cache.shape[0])) - used)
+    if window:
+        for tb, p0 in zip(tables[0], pos0):
+            for b in range(max(0, p0 - window + 1) // P_):
+                tb[b] = -1
+    step = pack_step(entries, pos0, [0] * len(lens), tables, torch.device(DEV), [spare])
     T = sum(rows_per_seg)
     # queries scaled up: scores of deviation ~2.5, so a few keys carry each row and a wrong or missing one shows
     q = gen(T, H * d + 16, seed=seed + 7, scale=2.5, dtype=BF).to(DEV)
@@ -469,6 +477,27 @@ def test_attention_page_sizes(P_):
 @pytest.mark.parametrize("window", [1, 5, 64, 100, 1000])
 def test_attention_windows(window):
     run_attention(H=4, Hk=2, d=32, P_=16, lens=[300, 200, 90], rows_per_seg=[1, 200, 17], window=window, seed=window)
+
+
+@pytest.mark.parametrize("d,window", [(192, 100), (256, 37), (128, 70), (160, 130)])
+def test_attention_windows_with_large_heads(d, window):
+    # the 16-rows-a-wave kernel (head sizes above 128) and the 32-row one, portions longer than a tile of rows, a
+    # window that is no multiple of the key tile, pages in front of the window given back
+    run_attention(H=4, Hk=2, d=d, P_=16, lens=[400, 230, 90], rows_per_seg=[1, 150, 70], window=window, seed=d)
+    run_attention(H=2, Hk=1, d=d, P_=8, lens=[333, 77], rows_per_seg=[100, 1], window=window, seed=d + 1)
+
+
+@pytest.mark.parametrize("d", [16, 64, 128, 192, 256])
+@pytest.mark.parametrize("whole", [False, True])
+def test_attention_ignores_what_it_does_not_see(monkeypatch, d, whole):
+    """NaN in every slot beyond a sequence's last key (what a page's last owner may have left there) and in the
+    spare page that stands for pages in front of a window: those positions get a weight of 0, and 0 x NaN must
+    not reach the output."""
+    monkeypatch.setattr(tuned(), "WHOLE_MIN_PAIRS", 1 if whole else 1 << 30)
+    nan = float("nan")
+    run_attention(H=4, Hk=2, d=d, P_=16, lens=[150, 70, 33, 1, 2049], rows_per_seg=[150, 1, 5, 1, 1], seed=d, stale=nan)
+    run_attention(H=4, Hk=2, d=d, P_=8, lens=[300, 203, 90, 61], rows_per_seg=[1, 130, 17, 1], window=45, seed=d, stale=nan)
+    run_attention(H=4, Hk=1, d=d, P_=24, lens=[300, 203, 9], rows_per_seg=[1, 66, 9], window=100, seed=d, stale=nan)
 
 
 def test_attention_long_context_decode_and_portion_over_history():

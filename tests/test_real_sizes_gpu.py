@@ -1,0 +1,121 @@
+"""Kernel paths that only the sizes of real models select (a vocabulary of 128,256: the argmax in pieces, the
+streaming product with two bands a block, the sampler over a long row), each against the plain implementation or a
+float64 product.  The tiny configurations never reach them."""
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+from test_kernels_plain import DEV, f64, gen
+from test_kernels_tuned import BF, check, pack, tuned
+
+pytestmark = pytest.mark.gpu
+
+VOCAB = 128256
+
+
+def ops():
+    from allpaca_amd.kernels import ops as o
+    return o
+
+
+@pytest.mark.parametrize("V", [8192, 8193, VOCAB])
+def test_argmax_in_pieces_takes_the_first_maximum(V):
+    """From 8,192 columns on a row is cut into 64 pieces and a second kernel takes the first maximum of the pieces'
+    (crates/allpaca-core/src/sampling.rs:215-234: strict >, the lowest index among equals, token 0 when nothing is
+    above -inf)."""
+    o = ops()
+    piece = -(-V // 64)
+    R = 12
+    lg = gen(R, V, seed=V).clone()
+    top = float(lg.max()) + 1.0
+    lg[0, 5 * piece + 3] = top
+    lg[0, 40 * piece + 1] = top                  # equal maxima in two pieces: the earlier piece wins
+    lg[1, 40 * piece + 1] = top
+    lg[1, 40 * piece + 300] = top                # ... and inside one piece, in different threads
+    lg[2, :] = float("-inf")                     # nothing above -inf: token 0
+    lg[3, V - 1] = top                           # the last column (the last piece is the short one)
+    lg[4, 0] = top
+    lg[5, :] = float("nan")                      # no comparison with NaN holds: token 0
+    lg[6, 17 * piece: 18 * piece] = float("nan")
+    lg[6, 63 * piece] = top                      # first column of the last piece, behind a piece of NaN
+    lg[7, 9 * piece - 1] = top
+    lg[7, 9 * piece] = top                       # neighbours across a border between pieces
+    lg[8, 123] = float("inf")
+    lg[8, 60 * piece] = float("inf")
+    lg[9, :] = -3.0                              # all equal: index 0
+    out = torch.full((R,), -1, dtype=torch.int32, device=DEV)
+    o.argmax_rows(lg.to(DEV), out)
+    want = [P.argmax(row) for row in lg.numpy()]
+    assert out.cpu().tolist() == want
+    assert want[:10] == [5 * piece + 3, 40 * piece + 1, 0, V - 1, 0, 0, 63 * piece, 9 * piece - 1, 123, 0]
+
+
+def _columns(N, rng, n=3000):
+    """A sample of output columns that holds the first and last bands and both sides of a block's border."""
+    fixed = list(range(0, 48)) + list(range(N - 40, N)) + list(range(N // 2 - 20, N // 2 + 20))
+    return np.unique(np.concatenate([np.asarray(fixed), rng.integers(0, N, size=n)]))
+
+
+@pytest.mark.parametrize("K", [4096, 3072])
+def test_products_with_a_vocabulary_of_output_columns(K):
+    """The head of an 8B (K = 4096) and a 3B (K = 3072) model: [128256, K].  Up to 16 rows the streaming kernel
+    takes two bands a block (from 32,768 columns on); more rows go to the tiled kernel, whole or with K in slices.
+    Every path against the float64 product on a sample of columns."""
+    t = tuned()
+    N = VOCAB
+    g = torch.Generator(device=DEV).manual_seed(K)
+    w = (torch.randn((N, K), generator=g, device=DEV) * 0.05).to(BF)
+    wp = pack(w)
+    rng = np.random.default_rng(K)
+    cols = _columns(N, rng)
+    w64 = f64(w[torch.from_numpy(cols).to(DEV)])
+    for M in (1, 8, 16, 17, 64, 300):
+        a = gen(M, K, seed=M, dtype=BF).to(DEV)
+        want = f64(a) @ w64.T
+        for out_dtype in ((BF, torch.float32) if M in (8, 64) else (torch.float32,)):
+            out = torch.full((M, N), 7.0, dtype=out_dtype, device=DEV)
+            t.gemm_bf16(a, wp, out)
+            check(f64(out[:, torch.from_numpy(cols).to(DEV)]), want, out_dtype)
+            # nothing is left unwritten anywhere in the row
+            assert not bool((out == 7.0).all(dim=0).any())
+    # rows together equal each row alone, bit for bit, on the two-band kernel too
+    a = gen(16, K, seed=99, dtype=BF).to(DEV)
+    tog = torch.empty(16, N, dtype=torch.float32, device=DEV)
+    t.gemm_bf16(a, wp, tog)
+    alone = torch.empty(1, N, dtype=torch.float32, device=DEV)
+    t.gemm_bf16(a[5:6], wp, alone)
+    assert torch.equal(alone[0], tog[5])
+
+
+def test_sampler_over_a_real_vocabulary():
+    """temperature / top-k / top-p over 128,256 logits against the plain sampler (crates/allpaca-core/src/
+    sampling.rs:24-67, 215-331)."""
+    o = ops()
+    V, R = VOCAB, 14
+    rng = np.random.default_rng(5)
+    lg = gen(R, V, seed=77) * 3.0
+    lg[0, 3] = lg[0, 90000] = lg[0, V - 1] = 20.0          # ties at the top, far apart
+    lg[1, :] = float("nan")                                 # degenerate: token 0
+    lg[2, 100000:] = float("-inf")
+    temps = np.asarray([0.7, 1.0, 0.9, 0.0, 1.5, 0.8, 0.8, 0.8, 1.0, 0.3, 1.0, 2.0, 0.8, 1.0], np.float32)
+    ks = np.asarray([0, 5, 0, 0, 40, 40, 1, 2000, 0, 0, 100000, 0, 40, 0], np.int32)
+    ps = np.asarray([1.0, 1.0, 0.9, 1.0, 0.95, 0.5, 1.0, 0.95, 0.1, 1.0, 0.99, 0.0, 0.95, 0.999], np.float32)
+    us = rng.random(R).astype(np.float32)
+    us[5] = 0.0
+    us[8] = 0.99999994
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    o.sample_rows(lg.to(DEV), torch.from_numpy(temps).to(DEV), torch.from_numpy(ks).to(DEV),
+                  torch.from_numpy(ps).to(DEV), torch.from_numpy(us).to(DEV), out)
+    got = out.cpu().tolist()
+    lgn = lg.numpy()
+    bad = []
+    for r in range(R):
+        want = P.sample(lgn[r], float(temps[r]), int(ks[r]), float(ps[r]), float(us[r]))
+        if got[r] != want:
+            # a draw within rounding of the border between two candidates may fall either way (the sum over
+            # 128,256 probabilities in float32 against float64): the neighbour that a nudged draw gives is accepted
+            near = {P.sample(lgn[r], float(temps[r]), int(ks[r]), float(ps[r]), float(us[r]) + e) for e in (-2e-5, 2e-5)}
+            if got[r] not in near:
+                bad.append((r, got[r], want))
+    assert not bad, bad
