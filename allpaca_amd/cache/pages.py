@@ -20,7 +20,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
-from ..parts.base import CacheNeed, FixedState, PagedKV
+from ..parts.base import CacheNeed, need_kind
 
 FREED = -1  # block-table entry of a page that a window has passed
 
@@ -89,14 +89,14 @@ class SlotPool(PagePool):
 
 @dataclass
 class PagedGroup:
-    need: PagedKV
+    need: CacheNeed                    # kind "pages"
     entries: List[int]                 # plan entries stored in this group, in order
     pool: PagePool
 
 
 @dataclass
 class StateGroup:
-    need: FixedState
+    need: CacheNeed                    # kind "slot"
     entries: List[int]
 
 
@@ -109,16 +109,20 @@ class _Sequence:
     version: int = 0                   # changes whenever an entry of a table was taken away or replaced
 
 
-def group_needs(needs: Sequence[CacheNeed]) -> Tuple[List[Tuple[PagedKV, List[int]]], List[Tuple[FixedState, List[int]]]]:
-    paged: Dict[PagedKV, List[int]] = {}
-    state: Dict[FixedState, List[int]] = {}
+def group_needs(needs: Sequence[CacheNeed]) -> Tuple[List[Tuple[CacheNeed, List[int]]], List[Tuple[CacheNeed, List[int]]]]:
+    """Plan entries sorted by what they need: ([(need of kind "pages", entries)], [(need of kind "slot", entries)]).
+    Equal needs share a group; a need is any object with the members `parts.base` lists."""
+    paged: Dict[CacheNeed, List[int]] = {}
+    state: Dict[CacheNeed, List[int]] = {}
     for i, n in enumerate(needs):
-        if isinstance(n, PagedKV):
+        try:
+            kind = need_kind(n)
+        except TypeError as e:
+            raise TypeError(f"plan entry {i}: {e}") from None
+        if kind == "pages":
             paged.setdefault(n, []).append(i)
-        elif isinstance(n, FixedState):
+        elif kind == "slot":
             state.setdefault(n, []).append(i)
-        elif n is not None:
-            raise TypeError(f"plan entry {i}: unknown cache need {n!r}")
     return list(paged.items()), list(state.items())
 
 
@@ -173,11 +177,12 @@ class CacheManager:
     def length(self, seq) -> int:
         return self._seqs[seq].length
 
-    def _first_needed(self, need: PagedKV, next_pos: int) -> int:
-        """First position whose key a row at `next_pos` or later can still read."""
-        if need.window is None:
+    def _first_needed(self, need: CacheNeed, next_pos: int) -> int:
+        """First position whose page a row at `next_pos` or later can still read."""
+        window = getattr(need, "window", None)
+        if window is None:
             return 0
-        return max(0, next_pos - need.window + 1)
+        return max(0, next_pos - window + 1)
 
     def pages_needed(self, seq, n_new: int) -> List[int]:
         """Pages each group must still take so that positions up to length + n_new exist."""

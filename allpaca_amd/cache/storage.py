@@ -1,10 +1,11 @@
 """Device memory of the cache: one tensor per paged group and per state group,
-allocated once.  A paged group's tensor is
-[layers of the group, pages + 1, 2 (keys, values), kv_heads, page_tokens, head_dim];
-inside a page, a key's elements lie together ([page_tokens, head_dim]) and a
-value's positions lie together ([head_dim, page_tokens], the same count of
-elements); the extra last page is never handed out (rows that pad a replayed
-graph write there).  A state group's tensor is [layers of the group, slots + 1, *shape]."""
+allocated once.  A paged group's tensor is [layers of the group, pages + 1,
+*need.page_shape(page_tokens)] (for keys and values: [2, kv_heads, page_tokens,
+head_dim]; inside a page a key's elements lie together and a value's positions
+lie together, the same count of elements); the extra last page is never handed
+out (rows that pad a replayed graph write there).  A state group's tensor is
+[layers of the group, slots + 1, *need.slot_shape()].  The element type is the
+need's own, or the run's cache type where the need names none."""
 from __future__ import annotations
 
 import math
@@ -21,7 +22,7 @@ _DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.
 @dataclass
 class PagedView:
     """What an attention-like mixer gets: its layer's pages and the step's block table of its group."""
-    kv: torch.Tensor                 # [pages + 1, 2, kv_heads, page_tokens, head_dim]
+    kv: torch.Tensor                 # [pages + 1, *need.page_shape(page_tokens)]; keys and values: [.., 2, kv_heads, page_tokens, head_dim]
     page_tokens: int
     window: Optional[int]
     writes: bool                     # False for a plan entry that borrows another entry's cache
@@ -48,25 +49,34 @@ class CacheStorage:
         self.manager = manager
         self.device = device
         P = manager.page_tokens
-        elem = torch.empty((), dtype=kv_dtype).element_size()
-        paged_shapes = [(len(g.entries), g.pool.num_pages + 1, 2, g.need.kv_heads, P, g.need.head_dim)
-                        for g in manager.paged_groups]
-        state_shapes = [(len(g.entries), manager.max_requests + 1, *g.need.shape) for g in manager.state_groups]
-        need = sum(math.prod(sh) * elem for sh in paged_shapes)
-        need += sum(math.prod(sh) * torch.empty((), dtype=_DTYPES[g.need.dtype]).element_size()
-                    for sh, g in zip(state_shapes, manager.state_groups))
+
+        def dtype_of(need) -> torch.dtype:
+            name = getattr(need, "dtype", None)
+            if name is None:
+                return kv_dtype
+            if name not in _DTYPES:
+                raise CacheError(f"cache need {need!r}: element type {name!r} is not one of {sorted(_DTYPES)}")
+            return _DTYPES[name]
+
+        def nbytes(shape, dt) -> int:
+            return math.prod(shape) * torch.empty((), dtype=dt).element_size()
+
+        paged = [((len(g.entries), g.pool.num_pages + 1, *g.need.page_shape(P)), dtype_of(g.need))
+                 for g in manager.paged_groups]
+        state = [((len(g.entries), manager.max_requests + 1, *g.need.slot_shape()), dtype_of(g.need))
+                 for g in manager.state_groups]
+        need = sum(nbytes(sh, dt) for sh, dt in paged + state)
         if device.type == "cuda":
             free, _ = torch.cuda.mem_get_info(device)
             free += torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)  # held by torch, unused
             if need > free:
-                per_page = sum(math.prod(sh) // sh[1] * elem for sh in paged_shapes)
+                per_page = sum(nbytes(sh, dt) // sh[1] for sh, dt in paged)
                 raise CacheTooLarge(
-                    f"the cache needs {need / 2**30:.1f} GiB ({[sh[1] - 1 for sh in paged_shapes]} pages of {P} tokens, "
+                    f"the cache needs {need / 2**30:.1f} GiB ({[sh[1] - 1 for sh, _ in paged]} pages of {P} tokens, "
                     f"{per_page / 2**20:.2f} MiB a page over all layers) but {free / 2**30:.1f} GiB of device memory "
                     f"are free: ask for fewer pages (max_tokens / num_pages)")
-        self.paged: List[torch.Tensor] = [torch.zeros(sh, dtype=kv_dtype, device=device) for sh in paged_shapes]
-        self.state: List[torch.Tensor] = [torch.zeros(sh, dtype=_DTYPES[g.need.dtype], device=device)
-                                          for sh, g in zip(state_shapes, manager.state_groups)]
+        self.paged: List[torch.Tensor] = [torch.zeros(sh, dtype=dt, device=device) for sh, dt in paged]
+        self.state: List[torch.Tensor] = [torch.zeros(sh, dtype=dt, device=device) for sh, dt in state]
 
     def poison_free_pages(self, value: float = 1e30) -> None:
         """A debugging aid against stale reads: every page that is free, now and whenever one comes back, is filled
@@ -95,7 +105,8 @@ class CacheStorage:
             kind, gi, li = loc
             if kind == "paged":
                 need = self.manager.paged_groups[gi].need
-                out.append(PagedView(self.paged[gi][li], self.manager.page_tokens, need.window, e.cache_of is None, gi))
+                out.append(PagedView(self.paged[gi][li], self.manager.page_tokens, getattr(need, "window", None),
+                                     e.cache_of is None, gi))
             else:
                 out.append(StateView(self.state[gi][li], e.cache_of is None, gi))
         return out

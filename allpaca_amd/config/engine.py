@@ -11,8 +11,14 @@ class EngineConfig:
     671-683; `engine.max_active_requests` 386-403)."""
     dtype: str = "bfloat16"            # "bfloat16" | "float32"
     page_tokens: int = 16
-    num_pages: int = 0                 # 0: sized from max_tokens
-    max_tokens: int = 8192             # tokens the cache pool holds when num_pages is 0
+    num_pages: int = 0                 # pages of the cache pool; 0: sized from max_tokens
+    max_tokens: int = 0                # tokens the cache pool holds when num_pages is 0; 0 too: sized from memory
+    # With neither given, the pool takes `kv_bytes`, or, if that is 0, the device memory that is free once the
+    # weights are loaded minus `kv_reserve_bytes` (room for a step's activations, logits and workspaces); never more
+    # than every one of `max_active_requests` requests at the model's longest context needs
+    # (the reference's budget is `kv.vram_bytes`, crates/allpaca-core/src/engine.rs:8651-8680).
+    kv_bytes: int = 0
+    kv_reserve_bytes: int = 4 << 30
     max_active_requests: int = 64
     max_batch_tokens: int = 2048       # token budget of one step
     chunk_tokens: int = 512            # largest portion of one prompt in a step
@@ -26,3 +32,6 @@ class EngineConfig:
         for name in ("page_tokens", "max_active_requests", "max_batch_tokens", "chunk_tokens"):
             if getattr(self, name) <= 0:
                 raise ValueError(f"{name} must be positive")
+        for name in ("num_pages", "max_tokens", "kv_bytes", "kv_reserve_bytes"):
+            if getattr(self, name) < 0:
+                raise ValueError(f"{name} must not be negative")

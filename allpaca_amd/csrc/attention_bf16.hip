@@ -888,6 +888,10 @@ APC_EXPORT int apc_attention_decode_bf16(const void* q, int ldq, int q_off, void
   return 0;
 }
 
+// Rows of a tile of the prefill kernels: the caller cuts every segment of several rows into tiles of at most this many
+// consecutive rows (tile_row0, tile_rows).
+APC_EXPORT int apc_attention_prefill_tile_rows() { return QT; }
+
 // 1 if a block can take a (row, kv head) whole at these sizes (workspace = null above), else 0.
 APC_EXPORT int apc_attention_decode_whole_fits(int H, int Hk, int d) {
   if (H <= 0 || Hk <= 0 || H % Hk || d <= 0) return 0;

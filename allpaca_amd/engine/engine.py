@@ -42,14 +42,15 @@ class Engine:
         cfg.validate()
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU is visible; the engine has no CPU path")
-        num_pages = cfg.num_pages or -(-cfg.max_tokens // cfg.page_tokens)
-        model_config, bound = load_model(model, _DTYPES[cfg.dtype], cfg.device, max_positions=num_pages * cfg.page_tokens)
+        # positions the tables are made for: what the pool can hold if its size is given, else the model's own limit
+        positions = cfg.num_pages * cfg.page_tokens or cfg.max_tokens or None
+        model_config, bound = load_model(model, _DTYPES[cfg.dtype], cfg.device, max_positions=positions)
         self._assemble(model_config, bound, cfg)
 
     def _assemble(self, model_config, model, cfg: EngineConfig) -> None:
         """Runner, scheduler and sampler around a model that is bound to its weights."""
         self.config, self.model_config, self.model = cfg, model_config, model
-        num_pages = cfg.num_pages or -(-cfg.max_tokens // cfg.page_tokens)
+        num_pages = cfg.num_pages or -(-cfg.max_tokens // cfg.page_tokens) or self.pages_that_fit(model, cfg)
         self.runner = ModelRunner(model, cfg.page_tokens, num_pages, cfg.max_active_requests, use_graphs=cfg.use_graphs)
         self.scheduler = Scheduler(self.runner.cache, cfg.max_active_requests, cfg.max_batch_tokens, cfg.chunk_tokens)
         self.sampler = Sampler(self.runner.rt.device, cfg.seed)
@@ -57,6 +58,29 @@ class Engine:
         self._ahead: Optional[_AheadStep] = None
         self._next_id = 0
         self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0}
+
+    @staticmethod
+    def pages_that_fit(model, cfg: EngineConfig) -> int:
+        """Pages of the pool when neither `num_pages` nor `max_tokens` is given: floor((budget - state slots) / bytes
+        of a page over all layers), the budget being `kv_bytes` or the device memory that is free now (the weights
+        are loaded) minus `kv_reserve_bytes`; at most what `max_active_requests` requests of the longest context
+        need."""
+        from ..cache import CacheEstimate, CacheTooLarge
+        rt = model.rt
+        est = CacheEstimate.of(model.cache_needs(), cfg.page_tokens, torch.empty((), dtype=rt.dtype).element_size())
+        budget = cfg.kv_bytes
+        if not budget:
+            free, _ = torch.cuda.mem_get_info(rt.device)
+            free += torch.cuda.memory_reserved(rt.device) - torch.cuda.memory_allocated(rt.device)
+            budget = free - cfg.kv_reserve_bytes
+        pages = est.pages_for_budget(budget, cfg.max_active_requests)
+        most = cfg.max_active_requests * -(-rt.max_positions // cfg.page_tokens)
+        pages = min(pages, most)
+        if pages <= 0:
+            raise CacheTooLarge(f"no page of the cache fits: the budget is {budget / 2**30:.2f} GiB "
+                                f"(kv_bytes, or free device memory less kv_reserve_bytes), a page over all layers takes "
+                                f"{est.bytes_per_page_of_every_group / 2**20:.2f} MiB")
+        return pages
 
     @classmethod
     def from_model(cls, model_config, model, config: EngineConfig) -> "Engine":
@@ -75,7 +99,7 @@ class Engine:
         dtype = _DTYPES[(config.dtype if config else options.get("dtype", EngineConfig().dtype))]
         folder = tempfile.mkdtemp(prefix="allpaca_amd_synthetic_")
         try:
-            write_model_folder(folder, config_json, seed, dtype)
+            write_model_folder(folder, config_json, seed, dtype, keep_tensors=False)
             return cls(folder, config, **options)
         finally:
             shutil.rmtree(folder, ignore_errors=True)

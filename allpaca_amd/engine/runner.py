@@ -18,7 +18,7 @@ import torch
 
 from ..cache import CacheManager, CacheStorage, OutOfPages, PagedView, StateView
 from ..models.decoder import DecoderModel
-from .batch import Entry, StepInfo, pack_step
+from .batch import Entry, StepInfo, StepLayout, pack_step
 
 
 class StepError(ValueError):
@@ -42,8 +42,13 @@ class ModelRunner:
         self.views = self.storage.views(model.spec.plan)
         self.pad_pages = [self.storage.dummy_page(g) for g in range(len(self.cache.paged_groups))]
         self.vocab_size = model.spec.vocab_size
-        # decode-only steps are replayed as HIP graphs when every mixer of the model allows it
-        self.use_graphs = bool(use_graphs) and all(getattr(b.mixer, "graph_safe", False) for b in model.blocks)
+        # decode-only steps are replayed as HIP graphs when every part of the model allows it: a single part that
+        # plans on the host (a feed-forward that gathers rows per expert, say) would be replayed with a stale plan
+        parts = [model.embedding, model.final_norm, model.head] + [p for b in model.blocks for p in b.parts.values()]
+        self.use_graphs = bool(use_graphs) and all(getattr(p, "graph_safe", False) for p in parts)
+        from ..kernels import ops
+        self.tile_rows = ops.attention_tile_rows(self.rt.dtype)          # how the attention kernel wants longer segments cut
+        self.position_axes = int(getattr(model.spec, "position_axes", 1))
         self.graphs: Dict[Tuple[int, int], "DecodeGraph"] = {}
         self.graph_replays = 0
         self.steps = 0
@@ -97,7 +102,7 @@ class ModelRunner:
                 raise OutOfPages(f"the step needs {n} new pages in group {g}, {self.cache.free_pages(g)} are free")
         for e in entries:
             self.cache.reserve(e.seq, len(e.tokens))
-        if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+        if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] and e.positions is None for e in entries):
             logits = self.graph_step(entries)
         else:
             info = self.pack(entries)
@@ -111,7 +116,8 @@ class ModelRunner:
         pos0 = [self.cache.length(e.seq) for e in entries]
         slots = [self.cache.slot_of(e.seq) for e in entries]
         tables = [[self.cache.block_table(e.seq, g) for e in entries] for g in range(len(self.cache.paged_groups))]
-        return pack_step(entries, pos0, slots, tables, self.rt.device, self.pad_pages)
+        return pack_step(entries, pos0, slots, tables, self.rt.device, self.pad_pages, tile_rows=self.tile_rows,
+                         position_axes=self.position_axes)
 
     def bind_views(self, info: StepInfo) -> list:
         for v in self.views:
@@ -211,7 +217,7 @@ class ModelRunner:
         if device_tokens.dtype != torch.int32 or device_tokens.numel() < n or device_tokens.device != g.dev.device:
             raise StepError("tokens fed on the GPU must be int32, one per prepared request, on the engine's device")
         g.upload()
-        g.dev[:n].copy_(device_tokens[:n])      # the tokens' place in the description (`DecodeGraph._part(0)`)
+        g.layout.part(g.dev, "tokens")[:n].copy_(device_tokens[:n])
         g.replay()
         self.graph_replays += 1
         for s in prepared.seqs:
@@ -236,35 +242,26 @@ class DecodeGraph:
         self.runner, self.rows, self.span = runner, rows, span
         cache = runner.cache
         self.widths = [-(-span // cache.page_tokens) for _ in cache.paged_groups]
-        # layout of the int32 description: tokens, positions, row_seg, seg_row0, seg_rows, seg_pos0, slots,
-        # logit_rows, then one [rows, width] block table per paged group
-        sizes = [rows] * 8 + [rows * w for w in self.widths]
-        self.cuts = np.cumsum([0] + sizes)
+        # the description is laid out as every step's is (`StepLayout`): one row, one segment and one wanted row per
+        # request
+        self.layout = lay = StepLayout(rows, rows, rows, rows, 0, runner.position_axes, self.widths)
         dev = runner.rt.device
-        self.host = torch.zeros(int(self.cuts[-1]), dtype=torch.int32).pin_memory()
+        self.host = torch.zeros(lay.total, dtype=torch.int32).pin_memory()
         self.np = self.host.numpy()
-        self.dev = torch.zeros(int(self.cuts[-1]), dtype=torch.int32, device=dev)
+        self.dev = torch.zeros(lay.total, dtype=torch.int32, device=dev)
         ar = np.arange(rows, dtype=np.int32)
-        self._part(2)[:] = ar          # row_seg
-        self._part(3)[:] = ar          # seg_row0
-        self._part(4)[:] = 1           # seg_rows
-        self._part(7)[:] = ar          # logit_rows
-        v = [self.dev[self.cuts[i]: self.cuts[i + 1]] for i in range(len(sizes))]
-        self.info = StepInfo(
-            n_rows=rows, n_segs=rows, tokens=v[0], positions=v[1], row_seg=v[2], seg_row0=v[3], seg_rows=v[4],
-            seg_pos0=v[5], state_slots=v[6], logit_rows=v[7], n_logit_rows=rows,
-            block_tables=[v[8 + g].view(rows, w) for g, w in enumerate(self.widths)],
-            host_row0=list(range(rows)), host_rows=[1] * rows, host_pos0=[0] * rows, host_slots=[0] * rows,
-            max_context=span, max_rows=1, decode_only=True, decode_rows=None, n_decode_rows=rows,
-            max_decode_context=span, n_tiles=0)
+        for name, value in (("row_seg", ar), ("seg_row0", ar), ("seg_rows", 1), ("logit_rows", ar), ("decode_rows", ar)):
+            lay.part(self.np, name)[:] = value
+        self.info = lay.info(self.dev, list(range(rows)), [1] * rows, [0] * rows, [0] * rows, span, True)
+        self.info.max_context = span
         self.copied = torch.cuda.Event()
         # what the pinned block tables hold: the request of every row and how many of its pages (per group), so that
         # a step writes only what is new (`CacheManager.table_version` changes when pages were taken away)
         self.row_key: List[Optional[tuple]] = [None] * rows
         self.row_pages = [[0] * rows for _ in self.widths]
         self.rows_used = rows
-        for g, w in enumerate(self.widths):
-            self._part(8 + g)[:] = runner.pad_pages[g]
+        for g in range(len(self.widths)):
+            lay.table(self.np, g)[:] = runner.pad_pages[g]
         self.fill([])
         self.upload()
         views = runner.bind_views(self.info)
@@ -302,8 +299,8 @@ class DecodeGraph:
                 gc.enable()
         torch.cuda.synchronize(dev)
 
-    def _part(self, i: int) -> np.ndarray:
-        return self.np[self.cuts[i]: self.cuts[i + 1]]
+    def _part(self, name: str) -> np.ndarray:
+        return self.layout.part(self.np, name)
 
     def fill(self, seqs: Sequence[Hashable]) -> None:
         """Positions, state slots and block tables of the requests `seqs`, one row each (tokens: `set_tokens`)."""
@@ -311,7 +308,7 @@ class DecodeGraph:
         cache = r.cache
         n = len(seqs)
         self.copied.synchronize()      # the last upload has read the pinned buffer
-        tokens, positions, pos0, slots = self._part(0), self._part(1), self._part(5), self._part(6)
+        tokens, positions, pos0, slots = (self._part(k) for k in ("tokens", "positions", "seg_pos0", "state_slots"))
         tokens[n:] = 0
         positions[n:] = 0
         pos0[n:] = 0
@@ -319,12 +316,14 @@ class DecodeGraph:
         for i, seq in enumerate(seqs):
             positions[i] = pos0[i] = cache.length(seq)
             slots[i] = cache.slot_of(seq)
+        if self.layout.axes > 1:     # every axis carries the token's place in its request
+            self._part("position_axes").reshape(self.rows, self.layout.axes)[:] = positions[:, None]
         keys = [(seq, cache.table_version(seq)) for seq in seqs]
         used = max(n, self.rows_used)
         for g, w in enumerate(self.widths):
-            bt = self._part(8 + g).reshape(self.rows, w)
+            bt = self.layout.table(self.np, g)
             pad = r.pad_pages[g]
-            windowed = cache.paged_groups[g].need.window is not None
+            windowed = getattr(cache.paged_groups[g].need, "window", None) is not None
             if used > n:
                 bt[n:used] = pad           # rows that held a request last time and hold none now
             held = self.row_pages[g]
@@ -347,7 +346,7 @@ class DecodeGraph:
         self.rows_used = n
 
     def set_tokens(self, tokens: Sequence[int]) -> None:
-        self._part(0)[:len(tokens)] = tokens
+        self._part("tokens")[:len(tokens)] = tokens
 
     def upload(self) -> None:
         self.dev.copy_(self.host, non_blocking=True)

@@ -125,7 +125,8 @@ class Scheduler:
     def add(self, req: Request) -> None:
         need = self.cache.pages_for_tokens(len(req.prompt) + req.params.max_tokens)
         for g in self.cache.paged_groups:
-            window_pages = None if g.need.window is None else self.cache.pages_for_tokens(g.need.window) + 1
+            window = getattr(g.need, "window", None)
+            window_pages = None if window is None else self.cache.pages_for_tokens(window) + 1
             worst = need if window_pages is None else min(need, window_pages + self.cache.pages_for_tokens(self.chunk))
             if worst > g.pool.num_pages:
                 raise RequestTooLarge(

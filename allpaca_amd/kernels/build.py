@@ -23,7 +23,8 @@ CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
 
 LIBS: Dict[str, List[str]] = {
     "plain": ["plain_ops.hip", "plain_gemm.hip", "plain_attention.hip", "sampling.hip"],
-    "tuned": ["gemm_bf16.hip", "gemm_wide_bf16.hip", "skinny_gemm_bf16.hip", "attention_bf16.hip", "rope_bf16.hip"],
+    "tuned": ["gemm_bf16.hip", "gemm_wide_bf16.hip", "skinny_gemm_bf16.hip", "attention_bf16.hip", "rope_bf16.hip",
+              "probe.hip"],
 }
 HEADERS = ["common.h", "mfma.h", "gemm_wide.h", "no_alloc.h"]
 

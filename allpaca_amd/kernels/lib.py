@@ -56,6 +56,9 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_attention_prefill_bf16": [P, I, I, P, I, I, I, I, P, I, P, I, P, P, P, P, I, I, F, P],
         "apc_attention_decode_bf16": [P, I, I, P, I, I, I, I, I, P, I, P, I, P, P, P, I, F, I, I, P, P],
         "apc_attention_decode_whole_fits": [I, I, I],
+        "apc_attention_prefill_tile_rows": [],
+        "apc_probe_read": [P, Z, P, I, I, P],
+        "apc_probe_mfma": [I, P, I, P],
     },
 }
 

@@ -325,6 +325,15 @@ def swiglu_pre(raw: torch.Tensor, ss: torch.Tensor, eps: float, w_gate_up, out: 
     return False
 
 
+def attention_tile_rows(run_dtype: torch.dtype = torch.bfloat16) -> int:
+    """Rows of a tile of the attention kernel that takes segments of several rows: the step packer cuts segments into
+    such tiles (`StepInfo.tile_row0`, `tile_rows`).  The kernel's library says how many; the plain kernel, which
+    32-bit runs use, does not look at tiles."""
+    if run_dtype != torch.bfloat16 or FORCE_PLAIN:
+        return 64
+    return int(_lib.load("tuned").apc_attention_prefill_tile_rows())
+
+
 def paged_attention(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
                     cache: torch.Tensor, page_tokens: int, block_table: torch.Tensor, step, window: int = 0,
                     scale: Optional[float] = None) -> None:

@@ -108,7 +108,8 @@ def load_model(model_dir: str, dtype: torch.dtype, device: torch.device | str = 
     from . import describe_model
     arch, cfg, spec = describe_model(read_config_json(model_dir))
     model = DecoderModel(spec)
-    tensors = load_tensors(model_dir, model.param_specs(), dtype, spec.forbidden, spec.copies, spec.ignored_suffixes)
+    tensors = load_tensors(model_dir, model.param_specs(), dtype, spec.forbidden, spec.copies, spec.ignored_suffixes,
+                           spec.aliases)
     positions = max_positions or spec.max_positions
     if not beyond_configured_positions:
         positions = min(positions, spec.max_positions)

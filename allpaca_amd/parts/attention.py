@@ -31,6 +31,7 @@ class Attention(Mixer):
         self.window = int(window) if window else None
         self.scale = float(scale) if scale is not None else None
         self.position = build_part(POSITION_ENCODINGS, position) if position is not None else None
+        self.graph_safe = self.position is None or bool(self.position.graph_safe)
         self.q_off, self.k_off, self.v_off = 0, self.H * self.d, (self.H + self.Hk) * self.d
         self.qkv_width = (self.H + 2 * self.Hk) * self.d
 
@@ -71,7 +72,8 @@ class Attention(Mixer):
         else:
             h.linear(self.w_qkv, qkv)
             if self.position is not None and fused is None:
-                self.position.apply(qkv, self.q_off, self.k_off, self.H, self.Hk, self.d, step.positions)
+                self.position.apply(qkv, self.q_off, self.k_off, self.H, self.Hk, self.d,
+                                    step.positions if step.position_axes is None else step.position_axes)
             if kv is not None or rot:
                 ops.rope_kv_write(qkv, self.q_off, self.k_off, self.v_off, self.H, self.Hk, self.d, rot, table,
                                   step.positions, step.row_seg, cache.block_table, kv, cache.page_tokens)

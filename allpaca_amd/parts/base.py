@@ -34,12 +34,27 @@ HEADS: Registry = Registry("output head")
 
 
 # ---- what a mixer needs of the cache manager -------------------------------
+# A need says what it wants kept per request and in what shape; the cache manager and the cache's device memory
+# work from `kind`, `page_shape` / `slot_shape` and `dtype` alone, so a mixer may bring a need of its own (a latent
+# vector per position, keys without values, state in another element type): a frozen dataclass with these members.
+# Plan entries whose needs are equal share a group (a pool of pages of its own and one block table per request, or
+# one tensor of slots).
+#   kind = "pages":  page_shape(page_tokens) -> the shape of one page of one layer; `window` (None: every position is
+#                    kept; n: pages that the last n positions no longer reach are given back during the request);
+#                    dtype: None (the run's cache element type) or a name ("float32", "bfloat16", "int32")
+#   kind = "slot":   slot_shape() -> the shape of one request's state in one layer, zeroed at admission; dtype as above
 @dataclass(frozen=True)
 class PagedKV:
-    """Keys and values of every position (or of the last `window` positions) in pages."""
+    """Keys and values of every position (or of the last `window` positions) in pages: keys [kv_head][slot][d],
+    values [kv_head][d][slot] (the same count of elements, see the attention kernels)."""
     kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    kind = "pages"
+    dtype = None
+
+    def page_shape(self, page_tokens: int) -> Tuple[int, ...]:
+        return (2, self.kv_heads, page_tokens, self.head_dim)
 
 
 @dataclass(frozen=True)
@@ -47,9 +62,26 @@ class FixedState:
     """Per-request state of fixed size in a slot (zeroed when a request is admitted)."""
     shape: Tuple[int, ...]
     dtype: str = "float32"
+    kind = "slot"
+
+    def slot_shape(self) -> Tuple[int, ...]:
+        return tuple(self.shape)
 
 
-CacheNeed = Union[PagedKV, FixedState, None]
+CacheNeed = Any   # PagedKV, FixedState, a need of the mixer's own with the members above, or None
+
+
+def need_kind(need) -> Optional[str]:
+    """"pages", "slot" or None (no cache); raises for an object that is no cache need."""
+    if need is None:
+        return None
+    kind = getattr(need, "kind", None)
+    if kind == "pages" and callable(getattr(need, "page_shape", None)):
+        return kind
+    if kind == "slot" and callable(getattr(need, "slot_shape", None)):
+        return kind
+    raise TypeError(f"{need!r} is no cache need: it must have kind 'pages' with page_shape(page_tokens) or kind "
+                    f"'slot' with slot_shape()")
 
 
 @dataclass
@@ -66,6 +98,11 @@ class Runtime:
 
 class Part:
     """Base of every part."""
+    # True if the part only launches kernels whose arguments stay valid when the step's device buffers are refilled
+    # (nothing read back to the host, no host-side branching on the batch's content).  Decode-only steps are replayed
+    # as a HIP graph only if every part of the model says so: a part that plans on the host (rows gathered per expert
+    # from a routing result, a loop over segments) would otherwise be replayed with the first batch's plan.
+    graph_safe = False
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         return {}
@@ -167,6 +204,7 @@ class PositionEncoding(Part):
 
     def apply(self, qkv: torch.Tensor, q_off: int, k_off: int, n_heads: int, n_kv_heads: int, head_dim: int,
               positions: torch.Tensor) -> None:
+        """`positions`: int32 [rows], or [rows, axes] for a model whose spec asks for more than one position axis."""
         raise NotImplementedError
 
 
@@ -175,11 +213,6 @@ class Mixer(Part):
     takes_normed_input = False
     # True if `forward_add` takes `emit=` (a `NormEmit` or None) for its product into the residual
     emits_next_norm = False
-    # True if `forward_add` only launches kernels whose arguments stay valid when the step's device
-    # buffers are refilled (nothing read back to the host, no host-side branching on the batch): such a
-    # mixer's decode steps can be replayed as a HIP graph
-    graph_safe = False
-
     def cache_need(self) -> CacheNeed:
         return None
 

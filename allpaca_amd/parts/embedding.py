@@ -14,6 +14,8 @@ from .spec import ParamSpec
 
 @EMBEDDINGS.register("token_table")
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, vocab_size: int, hidden_size: int):
         self.V, self.D = int(vocab_size), int(hidden_size)
 
@@ -31,6 +33,7 @@ class TokenEmbedding(Part):
 @HEADS.register("linear")
 class LinearHead(Part):
     """`tied`: the head uses the embedding matrix and owns no tensor."""
+    graph_safe = True
 
     def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False):
         self.V, self.D, self.tied = int(vocab_size), int(hidden_size), bool(tied)

@@ -14,6 +14,8 @@ from .spec import ParamSpec
 
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     takes_normed_input = True
     emits_next_norm = True
 

@@ -42,6 +42,8 @@ def inverse_frequencies(rot: int, theta: float, scaling: Optional[Mapping] = Non
 
 @POSITION_ENCODINGS.register("rope")
 class RotaryEncoding(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None,
                  scaling: Optional[Mapping] = None):
         self.head_dim = int(head_dim)
@@ -68,6 +70,8 @@ class RotaryEncoding(PositionEncoding):
 
 @POSITION_ENCODINGS.register("none")
 class NoEncoding(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, **_):
         pass
 

@@ -62,6 +62,12 @@ class ModelSpec:
     copies: Dict[str, str] = field(default_factory=dict)
     # endings of tensor names that are no parameters and are passed over (buffers some writers store)
     ignored_suffixes: tuple = ()
+    # other names under which a file may hold a tensor: name -> ordered candidates (the name itself among them);
+    # the first candidate that the files hold is taken
+    aliases: Dict[str, List[str]] = field(default_factory=dict)
+    # axes of a token's position that the position encodings read: 1 (the place in the request), or more, and then a
+    # step carries int32 [rows, axes] beside the places (`StepInfo.position_axes`, given per request in `Entry.positions`)
+    position_axes: int = 1
 
     def validate(self) -> None:
         for i, e in enumerate(self.plan):

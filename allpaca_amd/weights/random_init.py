@@ -16,7 +16,7 @@ from typing import Any, Dict, Mapping, Optional
 import torch
 
 from ..parts.spec import ParamSpec
-from .safetensors_io import write_safetensors
+from .safetensors_io import write_safetensors_streamed
 
 
 def _tensor_seed(seed: int, name: str) -> int:
@@ -45,23 +45,44 @@ def random_tensors(specs: Mapping[str, ParamSpec], seed: int, dtype: torch.dtype
     return out
 
 
+def stored_dtype(ps: ParamSpec, dtype: torch.dtype) -> torch.dtype:
+    return torch.int32 if ps.store == "int32" else torch.float32 if ps.store == "float32" else dtype
+
+
 def write_model_folder(path: str, config_json: Mapping[str, Any], seed: int, dtype: torch.dtype = torch.float32,
                        std: float = 0.02, norm_std: float = 0.0,
-                       overrides: Optional[Mapping[str, torch.Tensor]] = None) -> Dict[str, torch.Tensor]:
+                       overrides: Optional[Mapping[str, torch.Tensor]] = None, keep_tensors: bool = True,
+                       device: str | torch.device = "cpu") -> Optional[Dict[str, torch.Tensor]]:
     """Writes `path/config.json` and `path/model.safetensors` for the architecture that
-    `config_json` names.  `overrides` replaces tensors by name (tests plant values with it)."""
+    `config_json` names.  `overrides` replaces tensors by name (tests plant values with it).
+    Tensors are made and written one at a time; `keep_tensors=False` returns None instead of all of them (a model
+    of many GB is then never held whole in memory); `device`: where the random numbers are drawn (a seed gives
+    other values on another kind of device)."""
     from ..models import DecoderModel, describe_model
     _, cfg, spec = describe_model(config_json)
-    model = DecoderModel(spec)
-    tensors = random_tensors(model.param_specs(), seed, dtype, std, norm_std)
-    for name, t in (overrides or {}).items():
-        if name not in tensors:
+    specs = DecoderModel(spec).param_specs()
+    overrides = dict(overrides or {})
+    for name, t in overrides.items():
+        if name not in specs:
             raise KeyError(f"override {name!r} is not a tensor of this model")
-        if tuple(t.shape) != tuple(tensors[name].shape):
-            raise ValueError(f"override {name!r} has shape {tuple(t.shape)}, needs {tuple(tensors[name].shape)}")
-        tensors[name] = t.to(tensors[name].dtype)
+        if tuple(t.shape) != tuple(specs[name].shape):
+            raise ValueError(f"override {name!r} has shape {tuple(t.shape)}, needs {tuple(specs[name].shape)}")
+    kept: Dict[str, torch.Tensor] = {}
+
+    def make(name: str) -> torch.Tensor:
+        want = stored_dtype(specs[name], dtype)
+        if name in overrides:
+            t = overrides[name].to(want)
+        else:
+            t = random_tensors({name: specs[name]}, seed, dtype, std, norm_std, device)[name]
+        if keep_tensors:
+            kept[name] = t.cpu()
+        return t
+
     os.makedirs(path, exist_ok=True)
     with open(os.path.join(path, "config.json"), "w") as f:
         json.dump(dict(config_json), f, indent=1)
-    write_safetensors(os.path.join(path, "model.safetensors"), tensors, {"format": "pt", "seed": str(seed)})
-    return tensors
+    write_safetensors_streamed(os.path.join(path, "model.safetensors"),
+                               [(name, stored_dtype(ps, dtype), tuple(ps.shape)) for name, ps in specs.items()], make,
+                               {"format": "pt", "seed": str(seed)})
+    return kept if keep_tensors else None

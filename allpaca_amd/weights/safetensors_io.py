@@ -109,24 +109,39 @@ def open_model_files(model_dir: str) -> List[SafetensorsFile]:
     raise SafetensorsError(f"{model_dir}: no model.safetensors")
 
 
-def write_safetensors(path: str, tensors: Mapping[str, torch.Tensor], metadata: Mapping[str, str] | None = None) -> None:
-    """Writes tensors (CPU or GPU) in the order given."""
+def _write_tensor(f, t: torch.Tensor) -> None:
+    """The tensor's bytes, straight from its memory (no copy of the whole tensor into a bytes object)."""
+    c = t.detach().cpu().contiguous()
+    if c.numel():
+        f.write(memoryview(c.reshape(-1).view(torch.uint8).numpy()))
+
+
+def write_safetensors_streamed(path: str, entries, make, metadata: Mapping[str, str] | None = None) -> None:
+    """Writes a file whose tensors are made one at a time: `entries` = [(name, torch dtype, shape)] in file order,
+    `make(name)` returns the tensor (CPU or GPU) when its turn comes, so a model of many GB is never held whole."""
     header: Dict[str, dict] = {}
     if metadata:
         header["__metadata__"] = dict(metadata)
     off = 0
-    for name, t in tensors.items():
-        if t.dtype not in NAMES:
-            raise SafetensorsError(f"cannot write tensor {name!r} of type {t.dtype}")
-        n = t.numel() * t.element_size()
-        header[name] = {"dtype": NAMES[t.dtype], "shape": list(t.shape), "data_offsets": [off, off + n]}
+    for name, dtype, shape in entries:
+        if dtype not in NAMES:
+            raise SafetensorsError(f"cannot write tensor {name!r} of type {dtype}")
+        n = int(np.prod(shape, dtype=np.int64)) * DTYPES[NAMES[dtype]][1] if len(shape) else DTYPES[NAMES[dtype]][1]
+        header[name] = {"dtype": NAMES[dtype], "shape": list(shape), "data_offsets": [off, off + n]}
         off += n
     blob = json.dumps(header, separators=(",", ":")).encode("utf-8")
     blob += b" " * ((8 - len(blob) % 8) % 8)
     with open(path, "wb") as f:
         f.write(struct.pack("<Q", len(blob)))
         f.write(blob)
-        for t in tensors.values():
-            c = t.detach().cpu().contiguous()
-            if c.numel():
-                f.write(c.view(torch.uint8).numpy().tobytes() if c.dim() else c.reshape(1).view(torch.uint8).numpy().tobytes())
+        for name, dtype, shape in entries:
+            t = make(name)
+            if t.dtype != dtype or tuple(t.shape) != tuple(shape):
+                raise SafetensorsError(f"tensor {name!r} came as {t.dtype} {list(t.shape)}, announced as {dtype} {list(shape)}")
+            _write_tensor(f, t)
+
+
+def write_safetensors(path: str, tensors: Mapping[str, torch.Tensor], metadata: Mapping[str, str] | None = None) -> None:
+    """Writes tensors (CPU or GPU) in the order given."""
+    write_safetensors_streamed(path, [(name, t.dtype, tuple(t.shape)) for name, t in tensors.items()],
+                               lambda name: tensors[name], metadata)

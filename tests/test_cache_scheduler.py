@@ -367,3 +367,41 @@ def test_params_defaults_follow_the_reference():
     assert GenerationParams(max_tokens=0).max_tokens == 1   # crates/allpaca-core/src/engine.rs:3194
     assert GenerationParams(temperature=1e-6).greedy and not GenerationParams(temperature=0.1).greedy
     assert FinishReason.STOP == "stop" and FinishReason.LENGTH == "length"
+
+
+def test_cache_estimate_bytes_tokens_and_pages():
+    """What a context costs and what fits a budget (the reference's KvEstimate::bytes_for / tokens_for,
+    crates/allpaca-core/src/engine.rs:8651-8680), on the sizes of an 8B model and on a model with a window and state."""
+    from allpaca_amd.cache import CacheEstimate
+    from allpaca_amd.parts import FixedState, PagedKV
+    # 32 layers of 8 kv heads of 128 in bfloat16: 128 KiB a token, 2 MiB a page of 16
+    est = CacheEstimate.of([PagedKV(8, 128)] * 32, 16, 2)
+    assert est.bytes_per_page_of_every_group == 2 << 20 and est.slot_bytes == 0
+    assert est.bytes_for(1) == 2 << 20 and est.bytes_for(16) == 2 << 20 and est.bytes_for(17) == 4 << 20
+    assert est.bytes_for(2048) == 2048 * 128 * 1024
+    assert est.tokens_for(1 << 30) == 8192 and est.tokens_for((1 << 30) - 1) == 8176 and est.tokens_for(100) == 0
+    # floor(budget / page bytes), less the spare page
+    assert est.pages_for_budget(1 << 30, 64) == 511 and est.pages_for_budget((2 << 20) - 1, 64) == 0
+    # two groups (a window of 40 positions in 3 layers, everything in 2), a layer that borrows, state in 2 layers
+    needs = [PagedKV(2, 32, 40), PagedKV(2, 32), None, FixedState((100,), "float32"), PagedKV(2, 32, 40),
+             PagedKV(2, 32), PagedKV(2, 32, 40), FixedState((100,), "float32")]
+    est = CacheEstimate.of(needs, 8, 4)
+    page = 2 * 2 * 8 * 32 * 4
+    assert sorted((g.page_bytes, g.window) for g in est.groups) == [(2 * page, None), (3 * page, 40)]
+    assert est.slot_bytes == 2 * 100 * 4
+    full = next(i for i, g in enumerate(est.groups) if g.window is None)
+    assert est.pages_of_a_request(1000, full) == 125 and est.pages_of_a_request(1000, 1 - full) == 6
+    assert est.bytes_for(1000) == 125 * 2 * page + 6 * 3 * page
+    n = est.tokens_for(50 * 5 * page)
+    assert est.bytes_for(n) <= 50 * 5 * page < est.bytes_for(n + 1)
+    assert est.pages_for_budget(10 * 800 + 7 * 5 * page + 3, 9) == 6      # 10 slots, then 7 pages of every group, one spare
+    # no paged group at all: nothing to size
+    assert CacheEstimate.of([FixedState((4,), "float32")], 8, 2).pages_for_budget(1 << 20, 4) == 0
+
+
+def test_a_cache_need_must_describe_itself():
+    from allpaca_amd.cache import CacheManager
+    class Nothing:
+        kind = "pages"
+    with pytest.raises(TypeError, match="page_shape"):
+        CacheManager([Nothing()], 8, 4, 2)

@@ -184,6 +184,55 @@ def test_a_tied_head_stored_twice_and_a_frequency_buffer_are_passed_over(tmp_pat
     assert any("lm_head.weight" in m and "differs" in m for m in e.value.other) and not e.value.unexpected
 
 
+def test_tensors_are_found_under_their_other_names(tmp_path):
+    """The reference tries an ordered list of names for every tensor: GGUF-style, HF, without the `model.` prefix,
+    a few older spellings (crates/allpaca-safetensors/src/names.rs:26-107); a missing tensor is reported with every
+    name tried (catalog.rs:117-141)."""
+    from allpaca_amd.models import DecoderModel, describe_model
+    path, tensors = folder(tmp_path, H.TINY_B)
+    _, _, spec = describe_model(H.TINY_B)
+    want = DecoderModel(spec).param_specs()
+    assert spec.aliases["model.layers.2.mlp.up_proj.weight"] == [
+        "blk.2.ffn_up.weight", "model.layers.2.mlp.up_proj.weight", "layers.2.mlp.up_proj.weight",
+        "model.layers.2.mlp.w3.weight"]
+    # every tensor under another of its names, a different one from tensor to tensor
+    renamed, used = {}, set()
+    for i, (name, t) in enumerate(tensors.items()):
+        names = spec.aliases[name]
+        renamed[names[i % len(names)]] = t
+        used.add(i % len(names))
+    assert len(used) >= 3 and ("blk.0.attn_q.weight" in renamed or "token_embd.weight" in renamed)
+    rewrite(path, renamed)
+    got = load_tensors(path, want, torch.float32, spec.forbidden, spec.copies, spec.ignored_suffixes, spec.aliases)
+    assert set(got) == set(want) and all(torch.equal(got[k], tensors[k]) for k in want)
+    # without the list, the same file is a file of unexpected tensors
+    with pytest.raises(WeightsError):
+        load_tensors(path, want, torch.float32, spec.forbidden, spec.copies, spec.ignored_suffixes)
+    # a missing tensor names every candidate; one present twice is an error; another tensor is still unexpected
+    bad = dict(tensors)
+    del bad["model.layers.1.self_attn.o_proj.weight"]
+    bad["blk.0.attn_q.weight"] = tensors["model.layers.0.self_attn.q_proj.weight"]
+    bad["blk.0.attn_q_norm.weight"] = torch.ones(32)
+    rewrite(path, bad)
+    with pytest.raises(WeightsError) as e:
+        load_tensors(path, want, torch.float32, spec.forbidden, spec.copies, spec.ignored_suffixes, spec.aliases)
+    assert e.value.missing == ["model.layers.1.self_attn.o_proj.weight (also tried: blk.1.attn_output.weight, "
+                               "layers.1.self_attn.o_proj.weight)"]
+    assert e.value.unexpected == ["blk.0.attn_q_norm.weight"]
+    assert any("more than one of its names" in m and "blk.0.attn_q.weight" in m for m in e.value.other)
+    # a tied model: the head under its GGUF-style name is as forbidden as under its own
+    path_a = str(tmp_path / "a")
+    ta = write_model_folder(path_a, H.TINY_A, 0, torch.float32)
+    _, _, spec_a = describe_model(H.TINY_A)
+    want_a = DecoderModel(spec_a).param_specs()
+    ta = dict(ta)
+    ta["output.weight"] = torch.zeros(256, 64)
+    write_safetensors(os.path.join(path_a, "model.safetensors"), ta)
+    with pytest.raises(WeightsError) as e:
+        load_tensors(path_a, want_a, torch.float32, spec_a.forbidden, spec_a.copies, spec_a.ignored_suffixes, spec_a.aliases)
+    assert any("output.weight" in m and "tie_word_embeddings" in m for m in e.value.other) and not e.value.unexpected
+
+
 def test_untied_model_needs_its_head(tmp_path):
     path, tensors = folder(tmp_path, H.TINY_B)
     want, forbidden = specs(H.TINY_B)

@@ -148,7 +148,7 @@ def test_command_line_generate():
     assert all(0 <= ln["queue_ms"] <= ln["ttft_ms"] and ln["itl_ms"] > 0 for ln in lines)   # times per request
     r = subprocess.run(cmd[:2] + ["generate", "--synthetic", "--cpu-only", "--prompt-tokens", "1"],
                        capture_output=True, text=True, timeout=120)
-    assert r.returncode == 2 and "no CPU path" in r.stderr or "not available" in r.stderr
+    assert r.returncode == 2 and ("no CPU path" in r.stderr or "not available" in r.stderr), (r.returncode, r.stderr[-500:])
 
 
 def replay(folder, dtype, steps, max_tokens, out_dir, page_tokens=16):
@@ -226,6 +226,27 @@ def test_trace_run_goes_past_the_position_limit_of_config_json(tmp_path):
     rows = [np.fromfile(os.path.join(out, f"{s}.f32"), dtype="<f4").reshape(-1, 256) for s in range(51)]
     H.assert_close(np.concatenate(rows), H.oracle_logits(folder, t)[[149, 100] + list(range(149, 200))], "float32",
                    "past the limit")
+
+
+def test_trace_run_with_large_pages_and_many_live_requests(tmp_path):
+    """Ten live requests of one to three tokens with pages of 128 positions: --max-tokens counts each request as 64
+    tokens (640), and every one of them still needs a page of its own."""
+    folder = H.model_folder("A", "float32", True)
+    toks = {f"q{i}": H.random_tokens(256, 1 + i % 3, seed=400 + i) for i in range(10)}
+    steps = [dict(step=0, entries=[dict(id=k, tokens=t[:1], want=[0]) for k, t in toks.items()], end=[]),
+             dict(step=1, entries=[dict(id=k, tokens=t[1:], want=list(range(len(t) - 1))) for k, t in toks.items()
+                                   if len(t) > 1], end=list(toks))]
+    out = str(tmp_path / "many")
+    replay(folder, "float32", steps, 640, out, page_tokens=128)
+    first = np.fromfile(os.path.join(out, "0.f32"), dtype="<f4").reshape(10, 256)
+    rest = np.fromfile(os.path.join(out, "1.f32"), dtype="<f4").reshape(-1, 256)
+    row = 0
+    for i, (k, t) in enumerate(toks.items()):
+        got = [first[i:i + 1]]
+        if len(t) > 1:
+            got.append(rest[row:row + len(t) - 1])
+            row += len(t) - 1
+        H.check_logits(np.concatenate(got), folder, t, "float32", f"trace many {k}")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

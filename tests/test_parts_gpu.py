@@ -390,3 +390,218 @@ def test_toy_architecture_registers_builds_and_steps():
     for k in toks:
         assert np.abs(np.concatenate(got[k]) - want[k]).max() < 1e-4, k
     runner.cache.check()
+
+
+# --------------------------------------------------------------------------------------------------
+# a second toy architecture: a cache need of the mixer's own (one latent vector per position, no values, 32-bit
+# whatever the run's cache type), a position encoding over two axes, and a feed-forward that plans on the host
+# beside a mixer that does not
+# --------------------------------------------------------------------------------------------------
+def register_toy2():
+    from dataclasses import dataclass
+    from typing import Optional
+
+    from allpaca_amd.models import ARCHITECTURES, Architecture
+    from allpaca_amd.parts import (MIXERS, POSITION_ENCODINGS, BlockSpec, Mixer, ModelSpec, ParamSpec, PartSpec,
+                                   PlanEntry, PositionEncoding)
+    register_toy()
+    if "toy_latent" in MIXERS:
+        return
+
+    @dataclass(frozen=True)
+    class LatentPages:
+        """One vector of `width` numbers per position, in pages, always float32."""
+        width: int
+        window: Optional[int] = None
+        kind = "pages"
+        dtype = "float32"
+
+        def page_shape(self, page_tokens):
+            return (page_tokens, self.width)
+
+    @MIXERS.register("toy_latent")
+    class LatentMixer(Mixer):
+        """c_t = h_t Wd^T is cached (nothing else); out_t = mean(c_0 .. c_t) Wu^T."""
+
+        def __init__(self, hidden_size, width):
+            self.D, self.r = hidden_size, width
+
+        def param_specs(self):
+            return {"down.weight": ParamSpec((self.r, self.D), store="float32"),
+                    "up.weight": ParamSpec((self.D, self.r), store="float32")}
+
+        def cache_need(self):
+            return LatentPages(self.r)
+
+        def bind(self, tensors, rt):
+            self.rt = rt
+            self.wd = tensors["down.weight"].to(rt.device, torch.float32)
+            self.wu = tensors["up.weight"].to(rt.device, torch.float32)
+
+        def forward(self, h, step, cache):
+            Pg = cache.page_tokens
+            assert tuple(cache.kv.shape[1:]) == (Pg, self.r) and cache.kv.dtype == torch.float32
+            out = torch.empty(h.shape[0], self.D, dtype=torch.float32, device=h.device)
+            for s, (r0, n, p0) in enumerate(zip(step.host_row0, step.host_rows, step.host_pos0)):
+                c = h[r0:r0 + n].float() @ self.wd.T
+                bt = cache.block_table[s].long()
+                pos = torch.arange(p0, p0 + n, device=h.device)
+                if cache.writes:
+                    cache.kv[bt[pos // Pg], pos % Pg] = c
+                every = torch.arange(0, p0 + n, device=h.device)
+                lat = cache.kv[bt[every // Pg], every % Pg]
+                mean = lat.cumsum(0)[p0:] / (pos + 1).unsqueeze(1).float()
+                out[r0:r0 + n] = mean @ self.wu.T
+            return out
+
+    @POSITION_ENCODINGS.register("toy_axes")
+    class TwoAxes(PositionEncoding):
+        """q and k are multiplied by 1 + gain * (a0 + 2 a1) / 100 for a token at (a0, a1)."""
+
+        def __init__(self, gain):
+            self.gain = gain
+
+        def fused(self):
+            return None
+
+        def apply(self, qkv, q_off, k_off, n_heads, n_kv_heads, head_dim, positions):
+            assert positions.dim() == 2 and positions.shape[1] == 2
+            f = (1.0 + self.gain * (positions[:, 0] + 2 * positions[:, 1]).float() / 100.0).unsqueeze(1)
+            width = (n_heads + n_kv_heads) * head_dim
+            qkv[:, q_off:q_off + width] = (qkv[:, q_off:q_off + width].float() * f).to(qkv.dtype)
+
+    def describe(c):
+        D, V = c["hidden_size"], c["vocab_size"]
+        norm = dict(size=D, eps=c["eps"])
+        attn = lambda pos: PartSpec("attention", dict(hidden_size=D, num_heads=c["heads"], num_kv_heads=c["kv_heads"],
+                                                      head_dim=c["head_dim"], position=pos), "attn.")
+        blocks = []
+        for l, kind in enumerate(c["layers"]):
+            if kind == "latent":
+                mixer = PartSpec("toy_latent", dict(hidden_size=D, width=c["latent"]), "latent.")
+                ffn = PartSpec("swiglu", dict(hidden_size=D, intermediate_size=c["ffn"]), "mlp.")
+            elif kind == "axes_attn_routed":
+                mixer = attn(PartSpec("toy_axes", dict(gain=c["gain"])))
+                ffn = PartSpec("toy_routed", dict(hidden_size=D), "moe.")
+            else:
+                mixer = attn(PartSpec("rope", dict(head_dim=c["head_dim"], theta=c["theta"])))
+                ffn = PartSpec("toy_routed", dict(hidden_size=D), "moe.")
+            blocks.append(BlockSpec("pre_norm", {"mixer_norm": PartSpec("rmsnorm", norm, "norm1."), "mixer": mixer,
+                                                 "ffn_norm": PartSpec("rmsnorm", norm, "norm2."), "ffn": ffn},
+                                    f"toy.layers.{l}."))
+        return ModelSpec(D, V, c["max_positions"], PartSpec("token_table", dict(vocab_size=V, hidden_size=D), "toy.embed."),
+                         blocks, [PlanEntry(b) for b in range(len(blocks))], PartSpec("rmsnorm", norm, "toy.norm."),
+                         PartSpec("linear", dict(vocab_size=V, hidden_size=D, tied=False), "toy.head."),
+                         position_axes=c["axes"])
+
+    ARCHITECTURES.register("Toy2ForCausalLM", Architecture("toy2", dict, describe))
+
+
+TOY2 = dict(architectures=["Toy2ForCausalLM"], vocab_size=70, hidden_size=32, heads=2, kv_heads=2, head_dim=16, ffn=40,
+            latent=5, eps=1e-5, theta=10000.0, gain=0.6, max_positions=96, axes=2, layers=["latent", "axes_attn_routed"])
+
+
+def toy2_plain(cfg, w, tokens, axis1=None):
+    """The second toy model, whole sequence, float64.  `axis1`: the tokens' places on the second axis."""
+    T = len(tokens)
+    Hh, Hk, d = cfg["heads"], cfg["kv_heads"], cfg["head_dim"]
+    x = np.asarray(w["toy.embed.weight"], np.float64)[tokens]
+    pos = np.arange(T)
+    a1 = pos if axis1 is None else np.asarray(axis1)
+    for l, kind in enumerate(cfg["layers"]):
+        p = f"toy.layers.{l}."
+        h = P.rms_norm(x, w[p + "norm1.weight"], cfg["eps"])
+        if kind == "latent":
+            c = h @ w[p + "latent.down.weight"].T
+            mean = np.cumsum(c, axis=0) / (pos + 1)[:, None]
+            x = x + mean @ w[p + "latent.up.weight"].T
+        else:
+            q = P.linear(h, w[p + "attn.q_proj.weight"]).reshape(T, Hh, d)
+            k = P.linear(h, w[p + "attn.k_proj.weight"]).reshape(T, Hk, d)
+            v = P.linear(h, w[p + "attn.v_proj.weight"]).reshape(T, Hk, d)
+            if kind == "axes_attn_routed":
+                f = (1.0 + cfg["gain"] * (pos + 2 * a1) / 100.0)[:, None, None]
+                q, k = q * f, k * f
+            else:
+                inv = P.rope_inv_freq(d, cfg["theta"])
+                q, k = P.rope_neox(q, pos, inv), P.rope_neox(k, pos, inv)
+            x = x + P.linear(P.attention(q, k, v, Hh, Hk).reshape(T, Hh * d), w[p + "attn.o_proj.weight"])
+        h = P.rms_norm(x, w[p + "norm2.weight"], cfg["eps"])
+        if kind == "latent":
+            x = x + P.swiglu(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+        else:
+            lg = h @ w[p + "moe.router.weight"].T
+            e = (lg[:, 1] > lg[:, 0]).astype(int)
+            x = x + np.stack([h[t] @ w[p + f"moe.experts.{e[t]}.weight"].T for t in range(T)])
+    return P.rms_norm(x, w["toy.norm.weight"], cfg["eps"]) @ w["toy.head.weight"].T
+
+
+def test_a_cache_need_of_the_mixers_own_and_positions_on_two_axes():
+    """Registered here, with zero edits to the framework: pages that hold one 32-bit vector per position (no values, not
+    the run's cache type) in a group of their own beside a group of keys and values, and a position encoding that
+    reads two axes (given per request, or the token's place on both)."""
+    from allpaca_amd.engine.batch import Entry
+    from allpaca_amd.engine.runner import ModelRunner
+    from allpaca_amd.models import load_model
+    from allpaca_amd.weights import write_model_folder
+    register_toy2()
+    folder = os.path.join(H.tmp_root(), "toy2_model")
+    write_model_folder(folder, TOY2, seed=6, dtype=torch.float32, std=0.25, norm_std=0.1)
+    cfg, model = load_model(folder, torch.float32, "cuda:0")
+    runner = ModelRunner(model, 4, 30, 3, use_graphs=True)
+    assert not runner.use_graphs and runner.position_axes == 2
+    kinds = [type(g.need).__name__ for g in runner.cache.paged_groups]
+    assert kinds == ["LatentPages", "PagedKV"]
+    assert tuple(runner.storage.paged[0].shape) == (1, 31, 4, 5) and runner.storage.paged[0].dtype == torch.float32
+    _, w = P.read_model_folder(folder)
+    toks = {"a": H.random_tokens(70, 37, seed=1), "b": H.random_tokens(70, 12, seed=2)}
+    axis1 = {"a": None, "b": [(7 * i) % 5 for i in range(12)]}
+    want = {k: toy2_plain(TOY2, w, t, axis1[k]) for k, t in toks.items()}
+    got = {k: [] for k in toks}
+    at = {k: 0 for k in toks}
+    for k in toks:
+        runner.admit(k)
+    for batch in ([("a", 9), ("b", 3)], [("a", 1), ("b", 1)], [("a", 20), ("b", 1)], [("b", 7), ("a", 1)], [("a", 6)]):
+        entries = []
+        for k, n in batch:
+            pos = None if axis1[k] is None else [[at[k] + i, axis1[k][at[k] + i]] for i in range(n)]
+            entries.append(Entry(k, toks[k][at[k]:at[k] + n], list(range(n)), pos))
+        lg = runner.step(entries).cpu().numpy()
+        r = 0
+        for k, n in batch:
+            got[k].append(lg[r:r + n])
+            r += n
+            at[k] += n
+    for k in toks:
+        assert np.abs(np.concatenate(got[k]) - want[k]).max() < 1e-4, k
+    for k in toks:
+        runner.release(k)
+    runner.cache.check()
+    assert [runner.cache.free_pages(g) for g in range(2)] == [30, 30]
+
+
+def test_a_feed_forward_that_plans_on_the_host_keeps_the_model_out_of_graphs():
+    """Attention (which may be replayed) beside a routed feed-forward that gathers rows per expert on the host: asked
+    for graphs, the runner replays none, and decode steps whose rows go to other experts from step to step are right."""
+    from allpaca_amd.engine.batch import Entry
+    from allpaca_amd.engine.runner import ModelRunner
+    from allpaca_amd.models import load_model
+    from allpaca_amd.weights import write_model_folder
+    register_toy2()
+    cfgj = dict(TOY2, layers=["rope_attn_routed", "rope_attn_routed"], axes=1)
+    folder = os.path.join(H.tmp_root(), "toy2_routed")
+    write_model_folder(folder, cfgj, seed=8, dtype=torch.float32, std=0.25, norm_std=0.1)
+    cfg, model = load_model(folder, torch.float32, "cuda:0")
+    assert all(b.mixer.graph_safe for b in model.blocks) and not any(b.parts["ffn"].graph_safe for b in model.blocks)
+    runner = ModelRunner(model, 4, 30, 3, use_graphs=True)
+    assert not runner.use_graphs
+    _, w = P.read_model_folder(folder)
+    toks = {"a": H.random_tokens(70, 30, seed=3), "b": H.random_tokens(70, 25, seed=4)}
+    want = {k: toy2_plain(cfgj, w, t) for k, t in toks.items()}
+    for k in toks:
+        runner.admit(k)
+    runner.step([Entry("a", toks["a"][:10], []), Entry("b", toks["b"][:5], [])])
+    for j in range(20):
+        lg = runner.step([Entry("a", [toks["a"][10 + j]], [0]), Entry("b", [toks["b"][5 + j]], [0])]).cpu().numpy()
+        assert np.abs(lg[0] - want["a"][10 + j]).max() < 1e-4 and np.abs(lg[1] - want["b"][5 + j]).max() < 1e-4, j
+    assert runner.graph_replays == 0

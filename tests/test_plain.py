@@ -122,6 +122,35 @@ def test_llama3_scaling_regions():
     assert np.isclose(at(lam1 * (1 + 1e-9)), at(lam1 * (1 - 1e-9)), rtol=1e-6)
 
 
+def test_llama3_scaling_inside_the_blended_band():
+    """The regions, monotony and continuity above hold for a blend that is linear in the wavelength as well; the
+    rule blends linearly in L / wavelength.  The band's values as numbers (factor by which a pair's frequency is
+    multiplied), worked out by hand for the two tiny tables and for the table of the 8B models: with
+    r = L * inv_freq / (2 pi), s = (r - low) / (high - low), the factor is (1 - s) / factor + s.  Tiny B, pair 2:
+    inv_freq = 500000^(-2/16) = 0.19391, r = 64 * 0.19391 / 6.28319 = 1.97512, s = 0.32504, factor
+    0.67496 / 8 + 0.32504 = 0.40941 (the full digits below).  A blend linear in the wavelength would give
+    0.70 there.  The reference has no text for this rule; both the plain implementation and the engine's table are
+    held to these numbers."""
+    from allpaca_amd.parts.rope import inverse_frequencies
+    cases = [
+        (32, 500000.0, dict(factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=64),
+         {2: 0.4094569168877563}, 2, 3),
+        (48, 250000.0, dict(factor=4.0, low_freq_factor=1.0, high_freq_factor=2.0, original_max_position_embeddings=32),
+         {2: 0.8558231322063858, 3: 0.30777214364746464}, 2, 4),
+        (128, 500000.0, dict(factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=8192),
+         {29: 0.8281684118371798, 30: 0.6437431331275951, 31: 0.49350712273197106, 32: 0.37112227951784466,
+          33: 0.2714254770727862, 34: 0.19021074364065016}, 29, 35),
+    ]
+    for d, theta, scaling, band, first, end in cases:
+        base = np.array([theta ** (-2.0 * i / d) for i in range(d // 2)])
+        for table in (P.rope_inv_freq(d, theta, scaling), inverse_frequencies(d, theta, dict(scaling, rope_type="llama3"))):
+            ratio = np.asarray(table, np.float64) / base
+            for i, want in band.items():
+                assert abs(ratio[i] - want) <= 1e-12 * want, (d, i, ratio[i], want)
+            assert np.allclose(ratio[:first], 1.0, rtol=1e-13) and np.allclose(ratio[end:], 1.0 / scaling["factor"], rtol=1e-13)
+            assert sorted(band) == list(range(first, end))     # the band is exactly these pairs
+
+
 # ---- attention ------------------------------------------------------------
 def test_attention_single_key_and_uniform_keys():
     d = 4

@@ -1,9 +1,13 @@
 """Kernel paths that only the sizes of real models select (a vocabulary of 128,256: the argmax in pieces, the
 streaming product with two bands a block, the sampler over a long row), each against the plain implementation or a
 float64 product.  The tiny configurations never reach them."""
+import os
+
 import numpy as np
 import pytest
 import torch
+
+import helpers as H
 
 import plain_llama as P
 from test_kernels_plain import DEV, f64, gen
@@ -119,3 +123,47 @@ def test_sampler_over_a_real_vocabulary():
             if got[r] not in near:
                 bad.append((r, got[r], want))
     assert not bad, bad
+
+
+def test_a_folder_at_the_widths_of_a_3b_model_through_the_front_door(tmp_path):
+    """config.json + model.safetensors of two layers at the widths of Llama-3.2-3B (hidden 3072, 24 heads over 8 of
+    128, feed-forward 8192, vocabulary 128,256, tied head: 1.2 GB in bfloat16) written tensor by tensor, loaded by
+    `Engine(folder)` with a pool sized from free device memory, and run: greedy tokens are the plain implementation's
+    choice or within bfloat16's noise of it."""
+    import resource
+    import time
+    from allpaca_amd.config import preset
+    from allpaca_amd.engine import Engine
+    from allpaca_amd.sampling import GenerationParams
+    from allpaca_amd.weights import write_model_folder
+    cfg_json = dict(preset("llama-3.2-3b"), num_hidden_layers=2)
+    folder = str(tmp_path / "m3b")
+    assert write_model_folder(folder, cfg_json, 11, torch.bfloat16, keep_tensors=False, device=DEV) is None
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    torch.cuda.reset_peak_memory_stats()
+    free_before, _ = torch.cuda.mem_get_info()
+    t0 = time.time()
+    eng = Engine(folder, dtype="bfloat16", max_active_requests=4, kv_reserve_bytes=8 << 30)
+    load_s = time.time() - t0
+    weights = sum(os.path.getsize(os.path.join(folder, f)) for f in os.listdir(folder))
+    pool = eng.runner.cache.paged_groups[0].pool.num_pages
+    # the pool: what 4 requests of the longest context need (131,072 positions each), since that fits this card; with
+    # a budget given in bytes, floor(budget / bytes of a page over both layers) less the spare page
+    assert pool == 4 * (131072 // 16)
+    page = 2 * 2 * 8 * 16 * 128 * 2
+    assert Engine.pages_that_fit(eng.model, type(eng.config)(kv_bytes=1000 * page + 5, max_active_requests=4)) == 999
+    prompts = [H.random_tokens(VOCAB, n, seed=n) for n in (5, 40)]
+    outs = eng.generate(prompts, GenerationParams(max_tokens=4, temperature=0.0))
+    cfg, w = P.read_model_folder(folder)
+    for p, o in zip(prompts, outs):
+        lg = P.llama_forward(cfg, w, p + o.token_ids[:-1])[len(p) - 1:]
+        for j, t in enumerate(o.token_ids):
+            assert lg[j].max() - lg[j][t] <= 0.02 * np.abs(lg[j]).max(), (j, t)
+    peak_dev = torch.cuda.max_memory_allocated()
+    peak_host = resource.getrusage(resource.RUSAGE_SELF).ru_maxrss * 1024
+    print(f"\n3B widths, 2 layers: file {weights / 2**30:.2f} GiB, load {load_s:.2f} s, device peak "
+          f"{peak_dev / 2**30:.2f} GiB (pool {eng.runner.storage.bytes() / 2**30:.2f} GiB), host peak rss "
+          f"{peak_host / 2**30:.2f} GiB, free before {free_before / 2**30:.1f} GiB")
+    # the weights once, the pool, and working memory: never the model twice over
+    assert peak_dev <= eng.runner.storage.bytes() + weights + (3 << 30)
