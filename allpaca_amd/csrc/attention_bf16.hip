@@ -527,21 +527,40 @@ struct KVRegs {
   Frag v[DP / 16];     // 32 positions of 16 value elements per tile
 };
 
-// WHOLE = false: a block is 4 parts of one (row, kv head); its waves leave their results in `parts` and
-// attn_merge_kernel finishes.  WHOLE = true: the block's 4 waves take all ranges of KW keys of the (row, kv head) in
-// turn (wave w the ranges w, w + 4, ..), meet in LDS and the block writes the finished heads itself: no second kernel
-// and no trip through memory, which pays once the (row, kv head) pairs alone fill the chip (8B shapes, 2,048 keys a
-// row: 32 rows 52.9 -> 49.1 us, 64 rows 98.2 -> 91.6 us, 128 rows 196 -> 181 us; with 16 rows 30.2 -> 34.7 us.  Blocks of 8
-// waves were 2 % faster at one block a compute unit and 8-15 % slower at two).
+// Three ways to the finished heads of a (row, kv head):
+//  DEC_PARTS  a block is 4 parts (ranges of KW keys) of the pair; its waves leave their results in `parts` and
+//             attn_merge_kernel, a second launch, finishes.  Kept for the sizes the other two do not take.
+//  DEC_LAST   the same split over blocks, but a block first adds its 4 waves' results in LDS, leaves ONE partial
+//             result, and the block of a pair that finishes last adds the blocks' results in block order and writes
+//             the heads: no second launch (4.7-5.6 us a layer at 8B shapes, as much as the attention itself with one
+//             row).  Who is last is found with one counter per pair (a block adds 1 when its result is in memory;
+//             the one that reads blocks - 1 is last, and sets the counter back to 0 for the next launch).  The
+//             partial results go through memory with stores and loads that are coherent across the chip's eight L2
+//             caches one by one (sc1), not with a fence: a device-wide fence writes back and invalidates a whole L2
+//             and cost ten times what the second launch did.
+//  DEC_WHOLE  the block's 4 waves take all ranges of KW keys of the pair in turn (wave w the ranges w, w + 4, ..),
+//             meet in LDS and the block writes the finished heads itself: no partial result goes through memory,
+//             which pays once the pairs alone fill the chip (8B shapes, 2,048 keys a row: 32 rows 52.9 -> 49.1 us, 64
+//             rows 98.2 -> 91.6 us, 128 rows 196 -> 181 us; with 16 rows 30.2 -> 34.7 us.  Blocks of 8 waves were 2 %
+//             faster at one block a compute unit and 8-15 % slower at two).
+// The order of additions for a row depends on its position, KW and the number of parts only.
 constexpr int NW = 4;  // waves of a block of the decode kernel
-template <int DP, bool WHOLE>
+enum { DEC_PARTS = 0, DEC_WHOLE = 1, DEC_LAST = 2 };
+__device__ __forceinline__ void st_coh(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ld_coh(const float* p) {
+  return __hip_atomic_load(const_cast<float*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <int DP, int MODE>
 __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int ldq, int q_off, int H, int Hk, int d, const bf16_t* __restrict__ cache, int P,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ positions,
     const int* __restrict__ row_seg, const int* __restrict__ rows, int window, float scale, int KW, int n_parts,
-    float* __restrict__ parts, bf16_t* __restrict__ out, int ldo) {
+    float* __restrict__ parts, bf16_t* __restrict__ out, int ldo, int* __restrict__ counters) {
+  constexpr bool WHOLE = MODE == DEC_WHOLE, LAST = MODE == DEC_LAST;
   __shared__ __attribute__((aligned(16))) bf16_t Ps[NW * 16 * (32 + KPAD)];
-  extern __shared__ __attribute__((aligned(16))) float meet[];  // WHOLE: [NW][heads of the tile][d + 2]
+  extern __shared__ __attribute__((aligned(16))) float meet[];  // WHOLE, LAST: [NW][heads of the tile][d + 2]
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const int li = lane % 16, lc = lane / 16;
   const int G = H / Hk, gtiles = (G + 15) / 16;
@@ -551,8 +570,10 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(
   const int part = blockIdx.z * NW + wave;
   const int pos = positions[row];
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  if (!WHOLE && (part >= n_parts || max(part * KW, (first / 32) * 32) >= min((part + 1) * KW, pos + 1)))
-    return;  // nothing to see for this part (whole wave leaves together)
+  // nothing to see for this part: the wave leaves (DEC_PARTS), or stays with an empty result (DEC_LAST: the block's
+  // waves meet)
+  const bool empty = !WHOLE && (part >= n_parts || max(part * KW, (first / 32) * 32) >= min((part + 1) * KW, pos + 1));
+  if (MODE == DEC_PARTS && empty) return;
   const int* bt = block_table + (size_t)row_seg[row] * max_blocks;
   const size_t page_stride = (size_t)2 * Hk * P * d;
   const size_t head_off = (size_t)kvh * P * d, v_off = (size_t)Hk * P * d;
@@ -686,7 +707,7 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(
       const int k_lo = max(r * KW, (first / 32) * 32), k_hi = min((r + 1) * KW, pos + 1);
       if (k_lo < k_hi) run_range(k_lo, k_hi);
     }
-  } else {
+  } else if (!empty) {
     run_range(max(part * KW, (first / 32) * 32), min((part + 1) * KW, pos + 1));
   }
 
@@ -694,8 +715,8 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(
   const int g = gt * 16 + li;
   const int tile_heads = min(G - gt * 16, 16);
   if (g < G) {
-    float* dst = WHOLE ? meet + ((size_t)wave * tile_heads + li) * (d + 2)
-                       : parts + (((size_t)ri * H + (kvh * G + g)) * n_parts + part) * (d + 2);
+    float* dst = (WHOLE || LAST) ? meet + ((size_t)wave * tile_heads + li) * (d + 2)
+                                 : parts + (((size_t)ri * H + (kvh * G + g)) * n_parts + part) * (d + 2);
 #pragma unroll
     for (int dt = 0; dt < DP / 16; ++dt) {
       const int e = dt * 16 + lc * 4;
@@ -724,6 +745,71 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(
         const float wgt = pm == -INFINITY ? 0.f : exp2_neg(pm - m);
         l += ws[d + 1] * wgt;
         acc = fmaf(ws[e], wgt, acc);
+      }
+      out[(size_t)row * ldo + (size_t)(kvh * G + gt * 16 + hg) * d + e] = float_to_bf16(acc / l);
+    }
+  }
+  if constexpr (LAST) {
+    // The block's partial result for every head of the tile: the waves' results added in wave order, not divided by
+    // the sum; to parts[row][head][block][d + 2] = o, maximum, sum.
+    __syncthreads();
+    const int stride = d + 2, nz = gridDim.z, z = blockIdx.z;
+    for (int idx = threadIdx.x; idx < tile_heads * d; idx += NW * 64) {
+      const int hg = idx / d, e = idx % d;
+      const float* src = meet + (size_t)hg * stride;
+      float m = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) m = fmaxf(m, src[(size_t)w * tile_heads * stride + d]);
+      float l = 0.f, acc = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        const float* ws = src + (size_t)w * tile_heads * stride;
+        const float pm = ws[d];
+        const float wgt = pm == -INFINITY ? 0.f : exp2_neg(pm - m);
+        l += ws[d + 1] * wgt;
+        acc = fmaf(ws[e], wgt, acc);
+      }
+      float* dst = parts + (((size_t)ri * H + (kvh * G + gt * 16 + hg)) * nz + z) * stride;
+      st_coh(dst + e, acc);
+      if (e == 0) {
+        st_coh(dst + d, m);
+        st_coh(dst + d + 1, l);
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's stores have reached memory
+    __syncthreads();
+    __shared__ int is_last;
+    int* counter = counters + (size_t)ri * gridDim.y + blockIdx.y;
+    if (threadIdx.x == 0) {
+      const int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      is_last = before == nz - 1;
+      if (is_last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+    }
+    __syncthreads();
+    if (!is_last) return;
+    // the last block of the pair: the blocks' results of every head, in block order (only blocks with a visible key)
+    const int p_lo = ((first / 32) * 32) / KW, p_hi = min(pos / KW, n_parts - 1);
+    const int z_lo = p_lo / NW, nzv = p_hi / NW - z_lo + 1;
+    float* ml = meet;  // [heads of the tile][nzv][2]: maximum, sum (the waves' results are not needed any more)
+    for (int idx = threadIdx.x; idx < tile_heads * nzv; idx += NW * 64) {
+      const int hg = idx / nzv, zz = idx % nzv;
+      const float* src = parts + (((size_t)ri * H + (kvh * G + gt * 16 + hg)) * nz + z_lo + zz) * stride;
+      ml[idx * 2] = ld_coh(src + d);
+      ml[idx * 2 + 1] = ld_coh(src + d + 1);
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < tile_heads * d; idx += NW * 64) {
+      const int hg = idx / d, e = idx % d;
+      const float* src = parts + (((size_t)ri * H + (kvh * G + gt * 16 + hg)) * nz + z_lo) * stride + e;
+      const float* mlh = ml + (size_t)hg * nzv * 2;
+      float m = -INFINITY;
+      for (int zz = 0; zz < nzv; ++zz) m = fmaxf(m, mlh[zz * 2]);
+      float l = 0.f, acc = 0.f;
+      for (int zz = 0; zz < nzv; ++zz) {
+        const float pm = mlh[zz * 2];
+        const float wgt = pm == -INFINITY ? 0.f : exp2_neg(pm - m);
+        l += mlh[zz * 2 + 1] * wgt;
+        acc = fmaf(ld_coh(src + (size_t)zz * stride), wgt, acc);
       }
       out[(size_t)row * ldo + (size_t)(kvh * G + gt * 16 + hg) * d + e] = float_to_bf16(acc / l);
     }
@@ -836,13 +922,25 @@ static bool whole_fits(int G, int d) {
   return (long)NW * (G < 16 ? G : 16) * (d + 2) * sizeof(float) <= 65536;
 }
 
-// workspace: n_rows * H * n_parts * (d + 2) floats, or null: then every (row, kv head) is one block that finishes its
-// heads itself (`apc_attention_decode_whole_fits` says whether it can; n_parts is not used).
+// Whether the blocks of a (row, kv head) can leave one partial result each and the last one finish (DEC_LAST): the
+// meeting place must fit, and the maxima and sums of the blocks' results must fit into it afterwards.
+static bool last_fits(int G, int d, int n_parts) {
+  return whole_fits(G, d) && (n_parts + NW - 1) / NW <= 2 * (d + 2);
+}
+
+// Three ways (see attn_decode_kernel), chosen by the operands:
+//   workspace null                every (row, kv head) is one block that finishes its heads itself
+//                                 (`apc_attention_decode_whole_fits` says whether it can; n_parts is not used);
+//   workspace and counters        workspace: n_rows * H * ceil(n_parts / 4) * (d + 2) floats; counters: one int per
+//                                 (row, kv head tile) = n_rows * Hk * ceil(H / Hk / 16), zero before the first call
+//                                 (every call leaves them zero); `apc_attention_decode_last_fits` says whether it can;
+//   workspace, counters null      workspace: n_rows * H * n_parts * (d + 2) floats; a second kernel merges.
+// Calls that share counters or a workspace must not overlap (one stream).
 APC_EXPORT int apc_attention_decode_bf16(const void* q, int ldq, int q_off, void* out, int ldo, int n_rows, int H,
                                          int Hk, int d, const void* cache, int page_tokens, const int* block_table,
                                          int max_blocks, const int* positions, const int* row_seg, const int* rows,
                                          int window, float scale, int keys_per_part, int n_parts, float* workspace,
-                                         hipStream_t stream) {
+                                         int* counters, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   int e = check_common(q, ldq, q_off, cache, H, Hk, d, page_tokens);
   if (e) return e;
@@ -850,42 +948,47 @@ APC_EXPORT int apc_attention_decode_bf16(const void* q, int ldq, int q_off, void
   if (keys_per_part / page_tokens + 2 > 64) return APC_ERR_BAD_ARG;  // a wave keeps one page id per lane
   const int G = H / Hk, gtiles = (G + 15) / 16;
   if (Hk * gtiles > 65535 || H > 65535) return APC_ERR_BAD_ARG;
+  const size_t lds = (size_t)NW * (G < 16 ? G : 16) * (d + 2) * sizeof(float);
+#define DEC_LAUNCH(DP_, MODE_, GRID_, LDS_, PARTS_, WS_, CTR_)                                                         \
+  hipLaunchKernelGGL((attn_decode_kernel<DP_, MODE_>), GRID_, dim3(NW * 64), LDS_, stream, (const bf16_t*)q, ldq, q_off, \
+                     H, Hk, d, (const bf16_t*)cache, page_tokens, block_table, max_blocks, positions, row_seg, rows,   \
+                     window, scale, keys_per_part, PARTS_, WS_, (bf16_t*)out, ldo, CTR_)
+#define DEC_BY_HEAD(MODE_, GRID_, LDS_, PARTS_, WS_, CTR_)            \
+  if (d <= 32) DEC_LAUNCH(32, MODE_, GRID_, LDS_, PARTS_, WS_, CTR_);  \
+  else if (d <= 64) DEC_LAUNCH(64, MODE_, GRID_, LDS_, PARTS_, WS_, CTR_);  \
+  else if (d <= 96) DEC_LAUNCH(96, MODE_, GRID_, LDS_, PARTS_, WS_, CTR_);  \
+  else if (d <= 128) DEC_LAUNCH(128, MODE_, GRID_, LDS_, PARTS_, WS_, CTR_); \
+  else if (d <= 192) DEC_LAUNCH(192, MODE_, GRID_, LDS_, PARTS_, WS_, CTR_); \
+  else DEC_LAUNCH(256, MODE_, GRID_, LDS_, PARTS_, WS_, CTR_)
   if (!workspace) {
     if (!whole_fits(G, d)) return APC_ERR_UNSUPPORTED;
-    const size_t lds = (size_t)NW * (G < 16 ? G : 16) * (d + 2) * sizeof(float);
     dim3 grid(n_rows, Hk * gtiles, 1);
-#define DW_LAUNCH(DP_)                                                                                           \
-  hipLaunchKernelGGL((attn_decode_kernel<DP_, true>), grid, dim3(NW * 64), lds, stream, (const bf16_t*)q, ldq, q_off, \
-                     H, Hk, d, (const bf16_t*)cache, page_tokens, block_table, max_blocks, positions, row_seg, rows,   \
-                     window, scale, keys_per_part, 0, (float*)nullptr, (bf16_t*)out, ldo)
-    if (d <= 32) DW_LAUNCH(32);
-    else if (d <= 64) DW_LAUNCH(64);
-    else if (d <= 96) DW_LAUNCH(96);
-    else if (d <= 128) DW_LAUNCH(128);
-    else if (d <= 192) DW_LAUNCH(192);
-    else DW_LAUNCH(256);
-#undef DW_LAUNCH
+    DEC_BY_HEAD(DEC_WHOLE, grid, lds, 0, (float*)nullptr, (int*)nullptr);
     APC_LAUNCH_CHECK();
     return 0;
   }
   if (n_parts <= 0 || (n_parts + 3) / 4 > 65535) return APC_ERR_BAD_ARG;
-  dim3 grid(n_rows, Hk * gtiles, (n_parts + NW - 1) / NW), block(NW * 64);
-#define DC_LAUNCH(DP_)                                                                                            \
-  hipLaunchKernelGGL((attn_decode_kernel<DP_, false>), grid, block, 0, stream, (const bf16_t*)q, ldq, q_off, H, \
-                     Hk, d, (const bf16_t*)cache, page_tokens, block_table, max_blocks, positions, row_seg, rows,   \
-                     window, scale, keys_per_part, n_parts, workspace, (bf16_t*)nullptr, 0)
-  if (d <= 32) DC_LAUNCH(32);
-  else if (d <= 64) DC_LAUNCH(64);
-  else if (d <= 96) DC_LAUNCH(96);
-  else if (d <= 128) DC_LAUNCH(128);
-  else if (d <= 192) DC_LAUNCH(192);
-  else DC_LAUNCH(256);
-#undef DC_LAUNCH
+  dim3 grid(n_rows, Hk * gtiles, (n_parts + NW - 1) / NW);
+  if (counters) {
+    if (!last_fits(G, d, n_parts)) return APC_ERR_UNSUPPORTED;
+    DEC_BY_HEAD(DEC_LAST, grid, lds, n_parts, workspace, counters);
+    APC_LAUNCH_CHECK();
+    return 0;
+  }
+  DEC_BY_HEAD(DEC_PARTS, grid, 0, n_parts, workspace, (int*)nullptr);
+#undef DEC_BY_HEAD
+#undef DEC_LAUNCH
   APC_LAUNCH_CHECK();
   hipLaunchKernelGGL(attn_merge_kernel, dim3(n_rows, H), dim3(MERGE_NT), 0, stream,
                      workspace, n_parts, keys_per_part, H, d, positions, rows, window, (bf16_t*)out, ldo);
   APC_LAUNCH_CHECK();
   return 0;
+}
+
+// 1 if the blocks of a (row, kv head) can leave one partial result each and the last one finish, at these sizes.
+APC_EXPORT int apc_attention_decode_last_fits(int H, int Hk, int d, int n_parts) {
+  if (H <= 0 || Hk <= 0 || H % Hk || d <= 0 || n_parts <= 0) return 0;
+  return last_fits(H / Hk, d, n_parts) ? 1 : 0;
 }
 
 // Rows of a tile of the prefill kernels: the caller cuts every segment of several rows into tiles of at most this many

@@ -299,6 +299,22 @@ WHOLE_MIN_PAIRS = 256
 WHOLE_WAVES = 4   # waves of such a block (NW in attention_bf16.hip)
 
 
+# With fewer pairs: the blocks of a pair leave one partial result each and the one that finishes last adds them (no
+# second kernel), where the sizes allow; False: partial results per wave and a kernel that merges them.
+LAST_BLOCK_MERGES = True
+_counters: dict = {}
+
+
+def _pair_counters(device: torch.device, pairs: int) -> torch.Tensor:
+    """Zeroed int32 counters, one per (row, kv head tile), that live as long as the process: a call leaves them zero
+    again, and a replayed graph keeps pointing at them.  Grown by allocating anew; the old ones stay (graphs)."""
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    have = _counters.setdefault(key, [])
+    if not have or have[-1].numel() < pairs:
+        have.append(torch.zeros(max(1024, pairs), dtype=torch.int32, device=device))
+    return have[-1]
+
+
 def _keys_per_wave_whole(max_context: int, page_tokens: int) -> int:
     """Keys of a range in the kernel that takes a (row, kv head) whole: the context spread over the block's waves,
     64 to 512 keys, and no more pages than a wave keeps ids for (one per lane)."""
@@ -344,20 +360,30 @@ def attention_bf16(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int,
         n = step.n_decode_rows
         span = min(step.max_decode_context, window) if window else step.max_decode_context
         rows = step.decode_rows.data_ptr() if step.decode_rows is not None else 0
-        if (n * n_kv_heads * -(-(n_heads // n_kv_heads) // 16) >= WHOLE_MIN_PAIRS
-                and L.apc_attention_decode_whole_fits(n_heads, n_kv_heads, head_dim)):
+        pairs = n * n_kv_heads * -(-(n_heads // n_kv_heads) // 16)
+        if pairs >= WHOLE_MIN_PAIRS and L.apc_attention_decode_whole_fits(n_heads, n_kv_heads, head_dim):
             kw = _keys_per_wave_whole(span, page_tokens)
             _lib.check(L.apc_attention_decode_bf16(
                 q.data_ptr(), ldq, q_off, out.data_ptr(), ldo, n, n_heads, n_kv_heads, head_dim, cache.data_ptr(),
                 page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
-                step.row_seg.data_ptr(), rows, int(window), sc, kw, 0, 0, stream), "attention_decode_bf16 (whole)")
+                step.row_seg.data_ptr(), rows, int(window), sc, kw, 0, 0, 0, stream), "attention_decode_bf16 (whole)")
             return True
         kw = _keys_per_part(n, n_kv_heads, span, page_tokens)
         n_parts = -(-step.max_decode_context // kw)
+        if LAST_BLOCK_MERGES and L.apc_attention_decode_last_fits(n_heads, n_kv_heads, head_dim, n_parts):
+            # one partial result a block; the block of a (row, kv head) that finishes last adds them: one launch
+            nz = -(-n_parts // WHOLE_WAVES)
+            ws = torch.empty(n * n_heads * nz * (head_dim + 2), dtype=torch.float32, device=q.device)
+            _lib.check(L.apc_attention_decode_bf16(
+                q.data_ptr(), ldq, q_off, out.data_ptr(), ldo, n, n_heads, n_kv_heads, head_dim, cache.data_ptr(),
+                page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
+                step.row_seg.data_ptr(), rows, int(window), sc, kw, n_parts, ws.data_ptr(),
+                _pair_counters(q.device, pairs).data_ptr(), stream), "attention_decode_bf16 (last block merges)")
+            return True
         ws = torch.empty(n * n_heads * n_parts * (head_dim + 2), dtype=torch.float32, device=q.device)
         _lib.check(L.apc_attention_decode_bf16(
             q.data_ptr(), ldq, q_off, out.data_ptr(), ldo, n, n_heads, n_kv_heads, head_dim, cache.data_ptr(),
             page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
-            step.row_seg.data_ptr(), rows, int(window), sc, kw, n_parts, ws.data_ptr(), stream),
+            step.row_seg.data_ptr(), rows, int(window), sc, kw, n_parts, ws.data_ptr(), 0, stream),
             "attention_decode_bf16")
     return True

@@ -458,29 +458,37 @@ def run_attention(H, Hk, d, P_, lens, rows_per_seg, window=0, seed=0, stale=0.0)
         at += r
 
 
+@pytest.fixture(params=["last block merges", "merge kernel"])
+def decode_path(request, monkeypatch):
+    """Single rows whose keys are split over blocks: the block that finishes last adds the blocks' results (the
+    default), or a second kernel does."""
+    monkeypatch.setattr(tuned(), "LAST_BLOCK_MERGES", request.param == "last block merges")
+    return request.param
+
+
 @pytest.mark.parametrize("d", [16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 256])
-def test_attention_every_head_size(d):
+def test_attention_every_head_size(d, decode_path):
     run_attention(H=4, Hk=2, d=d, P_=16, lens=[150, 70, 33], rows_per_seg=[150, 1, 5], seed=d)
 
 
 @pytest.mark.parametrize("H,Hk", [(1, 1), (3, 3), (5, 1), (6, 2), (32, 8), (20, 1), (34, 2)])
-def test_attention_heads_and_groups(H, Hk):
+def test_attention_heads_and_groups(H, Hk, decode_path):
     # 20:1 and 17:1 groups are wider than one 16-row MFMA tile
     run_attention(H=H, Hk=Hk, d=32, P_=16, lens=[100, 260, 64], rows_per_seg=[1, 1, 64], seed=H)
 
 
 @pytest.mark.parametrize("P_", [8, 16, 24, 32, 64, 128])
-def test_attention_page_sizes(P_):
+def test_attention_page_sizes(P_, decode_path):
     run_attention(H=4, Hk=1, d=64, P_=P_, lens=[300, 129, 64, 1], rows_per_seg=[1, 129, 2, 1], seed=P_)
 
 
 @pytest.mark.parametrize("window", [1, 5, 64, 100, 1000])
-def test_attention_windows(window):
+def test_attention_windows(window, decode_path):
     run_attention(H=4, Hk=2, d=32, P_=16, lens=[300, 200, 90], rows_per_seg=[1, 200, 17], window=window, seed=window)
 
 
 @pytest.mark.parametrize("d,window", [(192, 100), (256, 37), (128, 70), (160, 130)])
-def test_attention_windows_with_large_heads(d, window):
+def test_attention_windows_with_large_heads(d, window, decode_path):
     # the 16-rows-a-wave kernel (head sizes above 128) and the 32-row one, portions longer than a tile of rows, a
     # window that is no multiple of the key tile, pages in front of the window given back
     run_attention(H=4, Hk=2, d=d, P_=16, lens=[400, 230, 90], rows_per_seg=[1, 150, 70], window=window, seed=d)
@@ -489,7 +497,7 @@ def test_attention_windows_with_large_heads(d, window):
 
 @pytest.mark.parametrize("d", [16, 64, 128, 192, 256])
 @pytest.mark.parametrize("whole", [False, True])
-def test_attention_ignores_what_it_does_not_see(monkeypatch, d, whole):
+def test_attention_ignores_what_it_does_not_see(monkeypatch, d, whole, decode_path):
     """NaN in every slot beyond a sequence's last key (what a page's last owner may have left there) and in the
     spare page that stands for pages in front of a window: those positions get a weight of 0, and 0 x NaN must
     not reach the output."""
@@ -500,7 +508,7 @@ def test_attention_ignores_what_it_does_not_see(monkeypatch, d, whole):
     run_attention(H=4, Hk=1, d=d, P_=24, lens=[300, 203, 9], rows_per_seg=[1, 66, 9], window=100, seed=d, stale=nan)
 
 
-def test_attention_long_context_decode_and_portion_over_history():
+def test_attention_long_context_decode_and_portion_over_history(decode_path):
     # the reference's long rows (crates/allpaca-hip/src/lib.rs:23162-23175: 3000 and 1300 keys) and a portion
     # of 70 rows over 2,000 keys of history
     run_attention(H=4, Hk=2, d=128, P_=16, lens=[3000, 1300, 2070], rows_per_seg=[1, 2, 70], seed=1)
@@ -552,3 +560,16 @@ def test_attention_finds_a_far_key_in_every_path(monkeypatch):
         for h in range(H):
             want = vs[0][key, h // 2].float()
             assert torch.allclose(out[-1, h * d:(h + 1) * d].float().cpu(), want, atol=2.0 ** -7 * 4)
+
+
+def test_attention_decode_many_launches_leave_the_counters_at_zero():
+    """The counters that tell the last block of a (row, kv head) are set back by that block: launch after launch on
+    the same counters, with other batch sizes, contexts and head counts in between, gives the right rows."""
+    t = tuned()
+    for rep in range(3):
+        run_attention(H=8, Hk=2, d=128, P_=16, lens=[2049, 700, 33, 1], rows_per_seg=[1, 1, 1, 1], seed=rep)
+        run_attention(H=4, Hk=4, d=64, P_=8, lens=[5000], rows_per_seg=[1], seed=10 + rep)
+        run_attention(H=32, Hk=8, d=128, P_=16, lens=[2048 + 7 * i for i in range(8)], rows_per_seg=[1] * 8, seed=20 + rep)
+    for dev_counters in t._counters.values():
+        for c in dev_counters:
+            assert int(c.abs().max()) == 0
