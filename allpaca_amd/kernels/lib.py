@@ -63,13 +63,77 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
     },
 }
 
-_loaded: Dict[str, ctypes.CDLL] = {}
+_loaded: Dict[str, "Library"] = {}
 
 ERRORS = {-1: "bad argument (shape or stride the kernel does not accept)", -2: "size not supported by this kernel",
           -3: "more rows than the entry point that allocates nothing has room for"}
 
 
-def load(name: str) -> ctypes.CDLL:
+class KernelTimer:
+    """Event timers around every call of an entry point while it is active (`with lib.timing() as t:`): for a pass
+    of its own beside the measured one, as the reference keeps its per-kernel timers out of the measured run
+    (one forward in 16 is timed with events and bucketed per kernel, crates/allpaca-hip/src/lib.rs:7776-7790).
+    `records`: (entry point, its arguments of C type int in order, start event, end event)."""
+
+    def __init__(self):
+        self.records = []
+
+    def totals(self) -> Dict[str, dict]:
+        """entry point -> {"calls", "us", "args": integer arguments of its calls in order}; waits for the GPU."""
+        import torch
+        torch.cuda.synchronize()
+        out: Dict[str, dict] = {}
+        for name, ints, e0, e1 in self.records:
+            t = out.setdefault(name, {"calls": 0, "us": 0.0, "args": []})
+            t["calls"] += 1
+            t["us"] += e0.elapsed_time(e1) * 1e3
+            t["args"].append(ints)
+        return out
+
+
+_timer = None
+# entry points that launch nothing (questions about sizes): never timed
+NOT_KERNELS = {"apc_attention_decode_whole_fits", "apc_attention_decode_last_fits", "apc_attention_prefill_tile_rows"}
+
+
+class timing:
+    def __enter__(self) -> KernelTimer:
+        global _timer
+        _timer = KernelTimer()
+        return _timer
+
+    def __exit__(self, *exc) -> None:
+        global _timer
+        _timer = None
+
+
+class _EntryPoint:
+    __slots__ = ("name", "fn", "int_at")
+
+    def __init__(self, name: str, fn, argtypes):
+        self.name, self.fn = name, fn
+        self.int_at = tuple(i for i, t in enumerate(argtypes) if t is I)
+
+    def __call__(self, *args):
+        if _timer is None or self.name in NOT_KERNELS:
+            return self.fn(*args)
+        import torch
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        code = self.fn(*args)
+        e1.record()
+        _timer.records.append((self.name, tuple(int(args[i]) for i in self.int_at), e0, e1))
+        return code
+
+
+class Library:
+    """The entry points of one kernel library as attributes (each may be timed, see `timing`)."""
+
+    def __init__(self, cdll: ctypes.CDLL, path: str):
+        self._cdll, self.path = cdll, path
+
+
+def load(name: str) -> Library:
     """The library `name`, built first if it is missing or stale."""
     lib = _loaded.get(name)
     if lib is not None:
@@ -79,16 +143,18 @@ def load(name: str) -> ctypes.CDLL:
     except _build.KernelBuildError as e:
         raise KernelLibraryError(f"kernel library '{name}' is not available: {e}") from None
     try:
-        lib = ctypes.CDLL(path)
+        cdll = ctypes.CDLL(path)
     except OSError as e:
         raise KernelLibraryError(f"cannot load {path}: {e}") from None
+    lib = Library(cdll, path)
     for fn, args in SIGNATURES[name].items():
         try:
-            f = getattr(lib, fn)
+            f = getattr(cdll, fn)
         except AttributeError:
             raise KernelLibraryError(f"{path} lacks entry point {fn}") from None
         f.argtypes = args
         f.restype = I
+        setattr(lib, fn, _EntryPoint(fn, f, args))
     _loaded[name] = lib
     return lib
 

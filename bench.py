@@ -8,7 +8,8 @@ The engine is set up for sequences of up to 8,192 tokens (--max-context), page s
 run with every sequence at 2,048 tokens (--context).
 Prints one JSON line: `value` = decoded tokens per second at the given batch; `prefill` = a 2,048-token
 prompt in one step; `roofline` = bytes a decode step has to read (every weight once, and the cache of the
-live requests) over its time, against 8 TB/s; `points` = decode at batch 1 and 64.  The way of reporting
+live requests) over its time, against 8 TB/s, and beside it what a plain streaming read reaches on this card
+(`measured_peak`); `points` = decode at batch 1 and 64.  The way of reporting
 follows the reference's bench tool (bytes per token, effective GB/s, share of the peak:
 tools/bench/src/roofline.rs:35-70).  Peaks: MI355X HBM3E 8 TB/s; dense bf16 MFMA 2.5 PFLOP/s."""
 import argparse
@@ -201,6 +202,124 @@ def prefill_flops(cfg, layers, T):
     return layers * (linear + attn) + 2 * D * V
 
 
+# ---- per-kernel times (a pass of its own, never inside the measured steps) -----------------------------------
+# entry point -> (indices of M, N, K among its int arguments, matrices read); N of the q/k/v product comes from its heads
+_PRODUCTS = {
+    "apc_skinny_gemm_bf16": ((2, 3, 4), 1), "apc_skinny_gemm_emit_bf16": ((2, 3, 4), 1),
+    "apc_skinny_gemm_pre_bf16": ((3, 4, 5), 1), "apc_skinny_swiglu_bf16": ((2, 3, 4), 2),
+    "apc_skinny_swiglu_pre_bf16": ((3, 4, 5), 2), "apc_gemm_bf16": ((2, 3, 4), 1), "apc_gemm_swiglu_bf16": ((2, 3, 4), 2),
+    "apc_gemm_splitk_emit_bf16": ((2, 3, 4), 1),
+}
+
+
+def _product_work(name, ints):
+    """(rows, weight bytes read, flops) of one call of a matrix product's entry point, or None."""
+    if name in _PRODUCTS:
+        (m, n, k), mats = _PRODUCTS[name]
+        M, N, K = ints[m], ints[n], ints[k]
+    elif name in ("apc_skinny_qkv_rope_bf16", "apc_gemm_splitk_qkv_rope_bf16"):
+        M, K, H, Hk, d = ints[3:8]
+        N, mats = (H + 2 * Hk) * d, 1
+    elif name in ("apc_gemm_pre_bf16", "apc_gemm_splitk_pre_bf16"):
+        M, N, K, mode = ints[3:7]
+        mats = 2 if mode == 3 else 1
+    elif name == "apc_gemm_splitk_bf16":
+        M, N, K, mode = ints[2:6]
+        mats = 2 if mode == 3 else 1
+    else:
+        return None
+    return M, mats * N * K * 2, 2 * mats * M * N * K
+
+
+def kernel_table(totals, steps, attention_bytes=0, attention_flops=0):
+    """Per entry point: calls and microseconds a step, and for the products and the attention what they read or
+    compute and at what rate, against the published peaks."""
+    rows = []
+    for name, t in sorted(totals.items(), key=lambda kv: -kv[1]["us"]):
+        r = {"kernel": name, "calls": round(t["calls"] / steps, 1), "us": round(t["us"] / steps, 1)}
+        works = [_product_work(name, a) for a in t["args"]]
+        nbytes = flops = 0
+        if works and works[0] is not None:
+            nbytes, flops = sum(w[1] for w in works) / steps, sum(w[2] for w in works) / steps
+            r["rows"] = works[0][0]
+        elif name == "apc_attention_decode_bf16":
+            nbytes = attention_bytes
+        elif name == "apc_attention_prefill_bf16":
+            flops = attention_flops
+        sec = t["us"] / steps * 1e-6
+        if nbytes and (not flops or flops / nbytes < 300):     # below the ridge: bound by reading
+            r.update({"GB": round(nbytes / 1e9, 3), "GB/s": round(nbytes / sec / 1e9, 1),
+                      "frac_hbm": round(nbytes / sec / 1e9 / HBM_PEAK_GBS, 3)})
+        elif flops:
+            r.update({"TFLOP": round(flops / 1e12, 3), "TFLOP/s": round(flops / sec / 1e12, 1),
+                      "frac_mfma": round(flops / sec / PEAK_FLOPS["bf16"], 3)})
+        rows.append(r)
+    return rows
+
+
+def kernel_times(cfg_json, args, layers):
+    """Event timers around every kernel launch of a decode step, a 2,048-token prefill and a mixed step (a portion of
+    512 tokens beside the decoding rows), run eagerly in passes of their own; and the host's time to launch a mixed step."""
+    import numpy as np
+    import torch
+
+    from allpaca_amd.engine.batch import Entry
+    from allpaca_amd.kernels import lib as klib
+    from allpaca_amd.sampling import GenerationParams
+    B, ctx = args.batch, args.context
+    cfg, eng = build_engine(cfg_json, args.dtype, B + 1, ctx, 600, layers, use_graphs=False, max_context=args.max_context)
+    rng = np.random.default_rng(0)
+    gp = GenerationParams(max_tokens=64, temperature=0.0)
+    for _ in range(B):
+        eng.add_request(rng.integers(0, cfg.vocab_size, size=ctx - 1).tolist(), gp)
+    while any(not r.decoding for r in eng.scheduler.running) or eng.scheduler.waiting:
+        eng.step()
+    for _ in range(3):
+        eng.step()
+    out = {}
+    steps = 4
+    with klib.timing() as t:
+        for _ in range(steps):
+            eng.step()
+    kv = kv_bytes_per_token(cfg, layers, 2 if args.dtype == "bf16" else 4)
+    out[f"decode_b{B}_ctx{ctx}"] = kernel_table(t.totals(), steps, attention_bytes=B * (ctx + 5) * kv)
+    # a mixed step: 512 tokens of a new prompt beside the B decoding rows; host time = until the launches are queued
+    ids = [r.id for r in eng.scheduler.running]
+    eng.runner.admit("mixed")
+    mixed = lambda at: [Entry("mixed", rng.integers(0, cfg.vocab_size, size=512).tolist(), [511])] + \
+        [Entry(i, [1], [0]) for i in ids]
+    eng.runner.step(mixed(0))
+    torch.cuda.synchronize()
+    host, gpu = [], []
+    for rep in range(3):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        batch = mixed(rep)
+        t0 = time.perf_counter()
+        e0.record()
+        eng.runner.step(batch)
+        e1.record()
+        host.append((time.perf_counter() - t0) * 1e6)
+        e1.synchronize()
+        gpu.append(e0.elapsed_time(e1) * 1e3)
+    with klib.timing() as t:
+        eng.runner.step(mixed(9))
+    hd = cfg.num_attention_heads * cfg.head_dim
+    out[f"mixed_512_plus_b{B}"] = kernel_table(t.totals(), 1, attention_bytes=B * ctx * kv,
+                                               attention_flops=layers * 4 * hd * 512 * (512 * 4 + 256))
+    out["host_us_mixed_step"] = {"host_launch_us": round(min(host), 1), "gpu_us": round(min(gpu), 1)}
+    eng.runner.release("mixed")
+    # prefill of 2,048 tokens in one step
+    T = 2048
+    eng.runner.admit("pf")
+    eng.runner.step([Entry("pf", rng.integers(0, cfg.vocab_size, size=T).tolist(), [T - 1])])
+    eng.runner.release("pf")
+    eng.runner.admit("pf2")
+    with klib.timing() as t:
+        eng.runner.step([Entry("pf2", rng.integers(0, cfg.vocab_size, size=T).tolist(), [T - 1])])
+    out[f"prefill_{T}"] = kernel_table(t.totals(), 1, attention_flops=layers * 4 * hd * (T * (T + 1) // 2))
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -222,6 +341,9 @@ def main() -> int:
     ap.add_argument("--max-prompt", type=int, default=4096)
     ap.add_argument("--new-tokens", type=int, default=256)
     ap.add_argument("--chunk", type=int, default=512, help="largest portion of a prompt in a step (with --requests)")
+    ap.add_argument("--kernel-times", action="store_true",
+                    help="instead of the measured steps: event timers around every kernel of a decode step, a mixed step "
+                         "and a 2,048-token prefill (eager passes of their own), and the host's time to launch a mixed step")
     ap.add_argument("--only", choices=["decode", "prefill"], default=None,
                     help="for profiling: only the decode steps at --batch (as --no-points), or only the 2,048-token "
                          "prefill (prints its figures as the line's value)")
@@ -240,6 +362,13 @@ def main() -> int:
     klib.load("plain")
     klib.load("tuned")
 
+    if args.kernel_times:
+        print(json.dumps({"metric": "microseconds per kernel and step (event timers, eager passes)", "unit": "us",
+                          "n_gpus": 1, "dtype": args.dtype,
+                          "config": {"model": args.preset, "layers": layers, "layers_of_configuration": full_layers,
+                                     "global_batch": args.batch, "seq_len": args.context},
+                          "kernel_times": kernel_times(cfg_json, args, layers)}), flush=True)
+        return 0
     if args.requests:
         n = args.requests
         top = args.max_prompt + args.new_tokens
@@ -279,6 +408,10 @@ def main() -> int:
                           "config": {"model": args.preset, "layers": layers}}), flush=True)
         return 0
 
+    # what this card delivers: a streaming read of 8 GiB and a loop of MFMAs from registers (allpaca_amd/csrc/probe.hip)
+    from allpaca_amd.kernels import probe
+    measured_gbs = probe.read_bandwidth(8.0)
+    measured_tflops = probe.mfma_rate() if args.dtype == "bf16" else None
     points = {}
     batches = [args.batch] + ([] if args.no_points else [b for b in (1, 64) if b != args.batch])
     ms = {}
@@ -297,13 +430,16 @@ def main() -> int:
             total = wbytes + b * ctx_mid * kv_bytes_per_token(cfg, layers, 2 if args.dtype == "bf16" else 4)
             gbs = total / sec / 1e9
             roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": round(gbs / HBM_PEAK_GBS, 4)}
+                    "frac": round(gbs / HBM_PEAK_GBS, 4), "measured_peak": round(measured_gbs, 1),
+                    "frac_of_measured": round(gbs / measured_gbs, 4)}
             if not args.no_points:
                 T = 2048
                 psec = prefill_run(eng, cfg, T)
                 fl = prefill_flops(cfg, layers, T)
                 prefill = {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3),
                            "frac": round(fl / psec / PEAK_FLOPS[args.dtype], 4)}
+                if measured_tflops:
+                    prefill["measured_peak_tflops"] = round(measured_tflops, 1)
         else:
             points[f"decode_b{b}"] = round(b / sec, 1)
         del eng
