@@ -18,6 +18,7 @@
 // Reference counterpart: gemm_nt_bf16_tiled_kernel, hip/src/kernels.cpp:634 (no matrix cores there).
 #include <type_traits>
 
+#include "gemm_direct.h"
 #include "gemm_wide.h"
 #include "mfma.h"
 
@@ -292,6 +293,10 @@ template <int MODE, bool PRE = false>
 static int launch_gemm(const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M, int N,
                        int K, hipStream_t stream, TiledPre pre = TiledPre{}) {
   constexpr int NB = MODE == G_SWIGLU ? BN / 2 : BN;
+  if constexpr (!PRE) {
+    // many rows, K a multiple of 128: the kernel that keeps the weights out of LDS (same sums, bit for bit)
+    if (gemm_direct_takes(MODE, A, lda, C, ldc, M, N, K)) return launch_gemm_direct(MODE, A, lda, W, W2, C, ldc, M, N, K, stream);
+  }
   if constexpr (MODE == G_SWIGLU) {
     // From 1,024 rows on the tile of 256 rows x 128 outputs takes as many columns as make whole rounds of one tile a
     // compute unit (at least two rounds), and the 128-row tile, two blocks a unit and so finer grained, the rest:

@@ -1,0 +1,14 @@
+// The product for many rows that loads its weights straight into registers (gemm_direct_bf16.hip), called from the
+// tiled product's launch code.
+#pragma once
+#include "common.h"
+
+// Fewer rows than this stay with the 128 x 128 tile and its K slices (too few blocks of 128 rows for the chip).
+constexpr int GEMM_DIRECT_MIN_ROWS = 1024;
+
+// mode: 0 store bfloat16, 1 store float32, 2 add into float32, 3 SwiGLU (W = gate, W2 = up, N = the width of each).
+// True if launch_gemm_direct runs this shape (K a multiple of 128, N and ldc of 4, 16-byte aligned A and C, ...).
+bool gemm_direct_takes(int mode, const void* A, int lda, const void* C, int ldc, int M, int N, int K);
+// W, W2 in the tiled layout.  APC_ERR_UNSUPPORTED for a shape that gemm_direct_takes refuses.
+int launch_gemm_direct(int mode, const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M,
+                       int N, int K, hipStream_t stream);

@@ -1,0 +1,293 @@
+// Matrix product for many rows whose weight operand never touches LDS:  C[M,N] = A[M,K] . W[N,K]^T.
+//
+// The tiled layout of W (16 outputs x 32 columns = 1 KiB in the lane order of a v_mfma_f32_16x16x32_bf16 operand)
+// is what a wave's load of 16 bytes a lane returns, so a wave takes its weight fragments straight from global memory
+// into a ring of registers, three steps of 32 columns ahead of their use.  The four waves of a block stand side by
+// side along N: each owns NF bands of 16 outputs and all 128 rows of the block, so no weight byte is loaded twice and
+// none crosses LDS.  The activations are shared by the four waves: they go from global memory into LDS with direct
+// loads (no registers in between), already in fragment order (a 16 x 32 fragment = one load instruction = 1 KiB
+// that a later ds_read_b128 returns lane by lane, free of bank conflicts), in four stages of 64 columns.
+// Per 64 columns a block moves 16 KiB of A and 8 NF KiB of W through the load path and reads 64 KiB from LDS, where
+// the 128 x 128 tile of gemm_bf16.hip moves 32 KiB and 96 KiB for half as many MFMAs (NF = 8).  What bounds it at
+// the shapes of a 2,048-row step is the L2: every block streams (128 + 64 NF) K 2 bytes through it, the counters
+// show the L2 busy three quarters of the time, and the vendor library's products sit at the same bound.
+//
+// The accumulators (8 row groups x NF bands x 4 registers) live in the accumulation registers; the MFMA is written as
+// an instruction with that register class, because left to itself the compiler moved accumulators between the two
+// files inside the loop for some epilogues.  Waits on the direct loads are counted by hand (they return in order:
+// at the barrier in front of a stage, all but the NVM youngest loads are complete); the loop issues the same loads
+// in every stage, beyond the end of K they fetch the last stage again, so that the count holds to the end.
+// MFMA operands are swapped against gemm_bf16.hip (weights as the first operand): a lane then holds four
+// consecutive outputs of one row and stores them as one 8 or 16 byte piece.
+// Sums are added in the same order as in gemm_bf16.hip (K ascending, 32 at a time): results are equal bit for bit.
+// K must be a multiple of 128, N of 4.
+// Reference counterpart: gemm_nt_bf16_tiled_kernel, hip/src/kernels.cpp:634 (no matrix cores there).
+#include "gemm_direct.h"
+#include "mfma.h"
+
+namespace {
+
+enum { D_STORE_BF16 = 0, D_STORE_F32 = 1, D_ACC_F32 = 2, D_SWIGLU = 3 };
+
+constexpr int R = 4;           // ring slots of W fragments: loads run R - 1 steps of 32 columns ahead
+constexpr int S = 4;           // LDS stages of A, 64 columns each
+constexpr int LEAD = R - 1;
+constexpr int PA = 3;          // fragments of A read from LDS ahead of the MFMAs that use them
+
+__device__ __forceinline__ void load_to_lds(BufferRsrc rsrc, void* lds, int lane_bytes, int scalar_bytes) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)lds, 16, lane_bytes,
+                                           scalar_bytes, 0, 0);
+}
+
+// c += a . b with c in accumulation registers
+__device__ __forceinline__ void mfma16_acc(floatx4& c, const Frag& a, const Frag& b) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  const u32x4 av = __builtin_bit_cast(u32x4, a), bv = __builtin_bit_cast(u32x4, b);
+  asm("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(av), "v"(bv));
+}
+
+template <int N>
+__device__ __forceinline__ void wait_loads_but() {  // until at most N vector memory loads of this wave are in flight
+  // vmcnt: bits [3:0] and [15:14]; expcnt [6:4] = 7 and lgkmcnt [11:8] = 15 wait for nothing
+  __builtin_amdgcn_s_waitcnt(((N & 15) | ((N >> 4) << 14)) | 0x0f70);
+}
+
+// Row group a (0..BMG-1) of a step issues the load of band f of the step LEAD ahead when a == f * BMG / NF
+// (BMG row groups of 16 rows a block: one load in some of the groups, or several a group when NF > BMG).
+template <int BMG, int NF>
+__host__ __device__ constexpr bool band_loaded_at(int f, int a) { return f * BMG / NF == a; }
+// W loads that a stage issues behind its last direct load of A (which goes out in group BMG / 2 - 1)
+template <int BMG, int NF>
+__host__ __device__ constexpr int loads_behind_a() {
+  int n = 0;
+  for (int g = BMG / 2; g < 2 * BMG; ++g)
+    for (int f = 0; f < NF; ++f)
+      if (band_loaded_at<BMG, NF>(f, g % BMG)) ++n;
+  return n;
+}
+
+// The tile of block `bid` of a product with BMG * 16 rows a block.
+template <int BMG, int NF, int MODE>
+__device__ __forceinline__ void direct_tile(int bid, const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
+                                            const bf16_t* __restrict__ W2, int chunks, void* __restrict__ C, int ldc,
+                                            int M, int N, int K) {
+  static_assert(R % 2 == 0, "ring slots are static over two stages");
+  constexpr int NP = BMG / 2;  // direct loads of A a wave and stage (BMG * 2 fragments over 4 waves)
+  constexpr int G = 2 * BMG;   // groups of NF MFMAs a stage: (chunk of 32 columns, row group)
+  static_assert(NP % 2 == 0 && G % (PA + 1) == 0, "a wave loads whole row groups; fragment registers are static");
+  constexpr int U = R / 2;     // stages per pass of the loop
+  // loads a wave issues between its last direct load of a stage and the barrier in front of that stage's use
+  constexpr int NVM = loads_behind_a<BMG, NF>() + (S - 2) * (NP + 2 * NF);
+  static_assert(NVM < 64, "the counter has 6 bits");
+  __shared__ __attribute__((aligned(1024))) unsigned char As[S][BMG * 2][1024];
+  const int tid = threadIdx.x, lane = tid % WAVE, wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+  constexpr int NOUT = MODE == D_SWIGLU ? NF / 2 : NF;  // bands of outputs a wave writes
+  constexpr int NB = 4 * NOUT * 16;                     // outputs of a block
+  int mt, nt;
+  {
+    // consecutive block ids go to the 8 XCDs in turn (an L2 each): XCD x takes the column tiles x, x + 8, ..; inside
+    // it groups of up to 16 row tiles sweep those columns, row tile fastest, so the blocks that run on an XCD at one
+    // time share a few panels of W
+    const int MT = ceil_div(M, BMG * 16), NT = ceil_div(N, NB), NL = ceil_div(NT, 8);
+    constexpr int GM = 16;
+    const int xcd = bid % 8, j = bid / 8;
+    const int first_m = j / (GM * NL) * GM, gsz = min(MT - first_m, GM), jj = j % (GM * NL);
+    mt = first_m + jj % gsz;
+    nt = jj / gsz * 8 + xcd;
+    if (nt >= NT || mt >= MT) return;
+  }
+  const int m0 = mt * BMG * 16;
+  const int bands = (N + 15) / 16;
+  const int band0 = nt * (4 * NOUT) + wave * NOUT;  // first band of this wave
+  const int base_band = min(band0, bands - 1);
+  const BufferRsrc abuf = make_rsrc(A + (size_t)m0 * lda);
+  const BufferRsrc wbuf = make_rsrc(W + (size_t)base_band * chunks * 512);
+  const BufferRsrc ubuf = make_rsrc((MODE == D_SWIGLU ? W2 : W) + (size_t)base_band * chunks * 512);
+  int woff[NF];  // SwiGLU: NOUT gate bands, then the same bands of up
+#pragma unroll
+  for (int f = 0; f < NF; ++f) woff[f] = (min(band0 + f % NOUT, bands - 1) - base_band) * chunks * 1024 + lane * 16;
+  int aoff[NP / 2];  // this wave's row groups wave * NP / 2 + j: lane -> (row lane % 16, 8 columns lane / 16)
+#pragma unroll
+  for (int j = 0; j < NP / 2; ++j)
+    aoff[j] = (min(m0 + (wave * (NP / 2) + j) * 16 + lane % 16, M - 1) - m0) * lda * 2 + (lane / 16) * 16;
+
+  floatx4 acc[BMG][NF];
+#pragma unroll
+  for (int a = 0; a < BMG; ++a)
+#pragma unroll
+    for (int f = 0; f < NF; ++f) acc[a][f] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int ktiles = K / 64;
+  auto a_piece = [&](int kt, int p) {  // piece p (0..NP-1) of this wave's share of stage kt
+    const int j = p / 2, c = p % 2;
+    load_to_lds(abuf, &As[kt % S][(wave * (NP / 2) + j) * 2 + c][0], aoff[j], min(kt, ktiles - 1) * 128 + c * 64);
+  };
+  Frag ring[R][NF];
+  auto w_piece = [&](int slot, int q, int f) {  // band f of step q (32 columns)
+    ring[slot][f] = load_frag_buffer((MODE == D_SWIGLU && f >= NOUT) ? ubuf : wbuf, woff[f],
+                                     min(q, 2 * ktiles - 1) * 1024);
+  };
+  // stages 0..S-2 of A and steps 0..LEAD-1 of W
+#pragma unroll
+  for (int s = 0; s < S - 1; ++s)
+#pragma unroll
+    for (int p = 0; p < NP; ++p) a_piece(s, p);
+#pragma unroll
+  for (int d = 0; d < LEAD; ++d)
+#pragma unroll
+    for (int f = 0; f < NF; ++f) w_piece(d, d, f);
+  wait_loads_but<0>();
+  // the compiler may have moved the W loads behind that wait; a use makes it wait for them here, so that the loop
+  // starts with nothing in flight and the counts below hold from the first stage on
+#pragma unroll
+  for (int d = 0; d < LEAD; ++d)
+#pragma unroll
+    for (int f = 0; f < NF; ++f)
+      asm volatile("" : "+v"(ring[d][f].w[0]), "+v"(ring[d][f].w[1]), "+v"(ring[d][f].w[2]), "+v"(ring[d][f].w[3]));
+
+  for (int t = 0; t < ktiles; t += U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int stage = t + u;
+      __builtin_amdgcn_sched_barrier(0);
+      wait_loads_but<NVM>();             // this wave's pieces of the stage are in LDS ...
+      __builtin_amdgcn_s_barrier();      // ... and so are the other waves'; all have left the stage before
+      __builtin_amdgcn_sched_barrier(0);
+      const unsigned char* abase = &As[stage % S][0][lane * 16];
+      Frag fa[PA + 1];  // group g reads fragment (row group g % BMG, chunk g / BMG)
+#pragma unroll
+      for (int g = 0; g < PA; ++g) fa[g] = *reinterpret_cast<const Frag*>(abase + g * 2048);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const int c = g / BMG, a = g % BMG;
+        const int slot = (2 * u + c) % R;          // ring slot of step 2 * stage + c
+        const int into = (2 * u + c + LEAD) % R;   // slot of the step LEAD ahead: the step before this one has left it
+        if (g + PA < G)
+          fa[(g + PA) % (PA + 1)] =
+              *reinterpret_cast<const Frag*>(abase + ((g + PA) % BMG) * 2048 + ((g + PA) / BMG) * 1024);
+        if (g < NP) a_piece(stage + S - 1, g);     // into the stage that every wave left at the barrier above
+#pragma unroll
+        for (int f = 0; f < NF; ++f)
+          if (band_loaded_at<BMG, NF>(f, a)) w_piece(into, 2 * stage + c + LEAD, f);
+#pragma unroll
+        for (int f = 0; f < NF; ++f) mfma16_acc(acc[a][f], ring[slot][f], fa[g % (PA + 1)]);
+        __builtin_amdgcn_sched_barrier(0);         // keeps a group's memory instructions with its MFMAs
+      }
+    }
+    // The last MFMAs must have left the matrix cores before their results are read.  The compiler does not know these
+    // instructions, so it neither waits by itself nor keeps its reads of the accumulators behind a wait that stands
+    // after the loop (it has read them right behind the last MFMA); inside the loop it reads none.
+    if (t + U >= ktiles) asm volatile("s_nop 15\n\ts_nop 15");
+  }
+  wait_loads_but<0>();
+
+  // D[i][j]: i = output (lane / 16) * 4 + r within the band, j = row lane % 16 within the row group
+  const int mi = lane % 16, nq = lane / 16;
+#pragma unroll
+  for (int a = 0; a < BMG; ++a) {
+    const int m = m0 + a * 16 + mi;
+    if constexpr (MODE == D_ACC_F32) {
+      floatx4 cv[NOUT];  // all loads of the residual first: a store between two loads would make the second wait
+#pragma unroll
+      for (int f = 0; f < NOUT; ++f) {
+        const int n = (band0 + f) * 16 + nq * 4;
+        cv[f] = (m < M && n < N) ? *reinterpret_cast<const floatx4*>((const float*)C + (size_t)m * ldc + n)
+                                 : floatx4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int f = 0; f < NOUT; ++f) {
+        const int n = (band0 + f) * 16 + nq * 4;
+        if (m < M && n < N) *reinterpret_cast<floatx4*>((float*)C + (size_t)m * ldc + n) = cv[f] + acc[a][f];
+      }
+    } else {
+      if (m >= M) continue;
+#pragma unroll
+      for (int f = 0; f < NOUT; ++f) {
+        const int n = (band0 + f) * 16 + nq * 4;
+        if (n >= N) continue;  // N is a multiple of 4: a piece is inside or outside as a whole
+        if constexpr (MODE == D_STORE_F32) {
+          *reinterpret_cast<floatx4*>((float*)C + (size_t)m * ldc + n) = acc[a][f];
+        } else {
+          float v[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            v[r] = MODE == D_STORE_BF16 ? acc[a][f][r] : silu_f(acc[a][f][r]) * acc[a][NOUT + f][r];
+          uint2 o;
+          o.x = pack_bf16x2(v[0], v[1]);
+          o.y = pack_bf16x2(v[2], v[3]);
+          *reinterpret_cast<uint2*>((bf16_t*)C + (size_t)m * ldc + n) = o;
+        }
+      }
+    }
+  }
+}
+
+template <int NF, int MODE>
+__global__ __launch_bounds__(256, 1) void gemm_direct_kernel(const bf16_t* __restrict__ A, int lda,
+                                                             const bf16_t* __restrict__ W,
+                                                             const bf16_t* __restrict__ W2, int chunks,
+                                                             void* __restrict__ C, int ldc, int M, int N, int K) {
+  direct_tile<8, NF, MODE>(blockIdx.x, A, lda, W, W2, chunks, C, ldc, M, N, K);
+}
+
+// Which NF takes a shape: a launch runs ceil(blocks / 256) rounds of one block a compute unit, and a round of blocks
+// with NF bands a wave takes about 44 + 7.25 NF time units (measured at 2,048 rows: 73, 84 and 102 us a round of 4,096
+// columns of K for NF = 4, 6, 8).
+// (Tried and taken out: one launch in which the columns of a nearly empty last round go to tiles of 64 rows.  With
+// 2,048 rows x 14,336 SwiGLU outputs, 3.5 rounds of 128-row tiles, it took 589 us against 453 us: a 64-row tile moves
+// 72 KiB through the load path per 64 columns of K for half the MFMAs.)
+int pick_bands(int M, int N, bool swiglu) {
+  const int mt = ceil_div(M, 128);
+  int best = 0;
+  double best_cost = 0.0;
+  for (int nf : {4, 6, 8}) {
+    const int nb = 4 * (swiglu ? nf / 2 : nf) * 16;
+    const long blocks = (long)mt * ceil_div(N, nb);
+    const double cost = (double)((blocks + 255) / 256) * (44.0 + 7.25 * nf);
+    if (!best || cost <= best_cost) best = nf, best_cost = cost;
+  }
+  return best;
+}
+
+template <int NF, int MODE>
+int launch(const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M, int N, int K,
+           hipStream_t stream) {
+  constexpr int NB = 4 * (MODE == D_SWIGLU ? NF / 2 : NF) * 16;
+  const long blocks = 8L * ceil_div(ceil_div(N, NB), 8) * ceil_div(M, 128);
+  if (blocks > 0x7fffffffL) return APC_ERR_BAD_ARG;
+  hipLaunchKernelGGL((gemm_direct_kernel<NF, MODE>), dim3((unsigned)blocks), dim3(256), 0, stream, A, lda, W, W2,
+                     ceil_div(K, 32), C, ldc, M, N, K);
+  APC_LAUNCH_CHECK();
+  return 0;
+}
+
+template <int MODE>
+int launch_mode(int nf, const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M, int N,
+                int K, hipStream_t stream) {
+  if (nf == 4) return launch<4, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream);
+  if (nf == 6) return launch<6, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream);
+  return launch<8, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream);
+}
+
+}  // namespace
+
+bool gemm_direct_takes(int mode, const void* A, int lda, const void* C, int ldc, int M, int N, int K) {
+  if (mode < 0 || mode > D_SWIGLU || M < GEMM_DIRECT_MIN_ROWS || K < 128 || K % 128 || N % 4 || ldc % 4) return false;
+  if (((uintptr_t)A & 15u) || ((uintptr_t)C & 15u) || lda % 8) return false;
+  // the lanes' byte offsets into the block's rows of A and the wave's bands of W are 32-bit
+  if ((long)128 * lda * 2 >= 0x7fffffffL || (long)8 * ceil_div(K, 32) * 1024 >= 0x7fffffffL) return false;
+  return true;
+}
+
+int launch_gemm_direct(int mode, const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M,
+                       int N, int K, hipStream_t stream) {
+  if (!gemm_direct_takes(mode, A, lda, C, ldc, M, N, K) || (mode == D_SWIGLU) != (W2 != nullptr)) return APC_ERR_UNSUPPORTED;
+  const int nf = pick_bands(M, N, mode == D_SWIGLU);
+  switch (mode) {
+    case D_STORE_BF16: return launch_mode<D_STORE_BF16>(nf, A, lda, W, W2, C, ldc, M, N, K, stream);
+    case D_STORE_F32: return launch_mode<D_STORE_F32>(nf, A, lda, W, W2, C, ldc, M, N, K, stream);
+    case D_ACC_F32: return launch_mode<D_ACC_F32>(nf, A, lda, W, W2, C, ldc, M, N, K, stream);
+    default: return launch_mode<D_SWIGLU>(nf, A, lda, W, W2, C, ldc, M, N, K, stream);
+  }
+}

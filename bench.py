@@ -13,6 +13,7 @@ live requests) over its time, against 8 TB/s, and beside it what a plain streami
 follows the reference's bench tool (bytes per token, effective GB/s, share of the peak:
 tools/bench/src/roofline.rs:35-70).  Peaks: MI355X HBM3E 8 TB/s; dense bf16 MFMA 2.5 PFLOP/s."""
 import argparse
+import gc
 import json
 import os
 import sys
@@ -443,6 +444,7 @@ def main() -> int:
         else:
             points[f"decode_b{b}"] = round(b / sec, 1)
         del eng
+        gc.collect()                 # an engine holds cycles (graphs, parts): without this the next one is built beside it
         torch.cuda.empty_cache()
 
     sec = ms[args.batch] / 1e3

@@ -54,7 +54,13 @@ GEMM_SHAPES = [(1, 5, 16), (3, 100, 136), (8, 4096, 512), (16, 33, 1208), (17, 2
                # enough blocks for the 256-row tiles: a last tile of 232 rows, K a multiple of 64 and not
                (1000, 8192, 200), (1024, 8190, 192),
                # 129..1024 rows and few output columns: K in slices (5, 2 and 3 of them), a last row tile of 44 rows
-               (512, 384, 2048), (200, 4096, 520), (300, 1100, 1024)]
+               (512, 384, 2048), (200, 4096, 520), (300, 1100, 1024),
+               # 1,024 rows or more, K a multiple of 128, N of 4: the kernel whose weights go straight into registers.
+               # One and several passes of its loop over K; a last row tile of 76 and of 6 rows; a last band of 4
+               # columns; 4, 6 and 8 bands a wave (6,144 and 8,192 columns at 2,048 rows)
+               (1024, 256, 128), (1100, 1028, 384), (1030, 2500, 640), (2048, 6144, 128), (2048, 8192, 256),
+               (2048, 4096, 1024),
+               (2048, 10240, 128), (1100, 16384, 256)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
@@ -287,7 +293,11 @@ def test_embedding_from_the_tiled_table():
                                    (100, 72, 2048), (300, 200, 320), (1000, 4096, 200), (1024, 4090, 128),
                                    # the 256-row tile (1,024 rows or more, K a multiple of 64, 512 tiles or more): last
                                    # row tile of 76 rows, last column tile of 16 columns; one and three K steps
-                                   (2048, 8192, 128), (1100, 13200, 192), (1024, 16640, 64)])
+                                   (2048, 8192, 128), (1100, 13200, 192), (1024, 16640, 64),
+                                   # weights straight into registers (K a multiple of 128): 2, 3 and 4 gate bands a
+                                   # wave, a last band of 8 columns, a last row tile of 76 rows
+                                   (1024, 136, 128), (1100, 13208, 256), (2048, 3072, 384), (2048, 14336 // 2, 128),
+                                   (2048, 14336, 128)])
 def test_swiglu_bf16(M, F, K):
     t = tuned()
     h = gen(M, K, seed=1, dtype=BF).to(DEV)
