@@ -233,7 +233,7 @@ __global__ __launch_bounds__(256, 1) void gemm_direct_kernel(const bf16_t* __res
 
 // Which NF takes a shape: a launch runs ceil(blocks / 256) rounds of one block a compute unit, and a round of blocks
 // with NF bands a wave takes about 44 + 7.25 NF time units (measured at 2,048 rows: 73, 84 and 102 us a round of 4,096
-// columns of K for NF = 4, 6, 8).
+// columns of K for NF = 4, 6, 8); 3 and 5 bands give the 3,072 and 5,120 columns of a 3B model one full round.
 // (Tried and taken out: one launch in which the columns of a nearly empty last round go to tiles of 64 rows.  With
 // 2,048 rows x 14,336 SwiGLU outputs, 3.5 rounds of 128-row tiles, it took 589 us against 453 us: a 64-row tile moves
 // 72 KiB through the load path per 64 columns of K for half the MFMAs.)
@@ -241,7 +241,8 @@ int pick_bands(int M, int N, bool swiglu) {
   const int mt = ceil_div(M, 128);
   int best = 0;
   double best_cost = 0.0;
-  for (int nf : {4, 6, 8}) {
+  for (int nf : {3, 4, 5, 6, 8}) {
+    if (swiglu && nf % 2) continue;  // half of a wave's bands are gate, half up
     const int nb = 4 * (swiglu ? nf / 2 : nf) * 16;
     const long blocks = (long)mt * ceil_div(N, nb);
     const double cost = (double)((blocks + 255) / 256) * (44.0 + 7.25 * nf);
@@ -265,6 +266,10 @@ int launch(const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C,
 template <int MODE>
 int launch_mode(int nf, const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M, int N,
                 int K, hipStream_t stream) {
+  if constexpr (MODE != D_SWIGLU) {
+    if (nf == 3) return launch<3, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream);
+    if (nf == 5) return launch<5, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream);
+  }
   if (nf == 4) return launch<4, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream);
   if (nf == 6) return launch<6, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream);
   return launch<8, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream);

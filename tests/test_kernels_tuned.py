@@ -60,7 +60,9 @@ GEMM_SHAPES = [(1, 5, 16), (3, 100, 136), (8, 4096, 512), (16, 33, 1208), (17, 2
                # columns; 4, 6 and 8 bands a wave (6,144 and 8,192 columns at 2,048 rows)
                (1024, 256, 128), (1100, 1028, 384), (1030, 2500, 640), (2048, 6144, 128), (2048, 8192, 256),
                (2048, 4096, 1024),
-               (2048, 10240, 128), (1100, 16384, 256)]
+               (2048, 10240, 128), (1100, 16384, 256),
+               # 3 and 5 bands a wave: the widths of a 3B model (3,072 and 5,120 columns)
+               (2048, 3072, 128), (2048, 5120, 256)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
