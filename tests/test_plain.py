@@ -381,3 +381,15 @@ def test_sampler_frequencies_match_softmax():
     p /= p.sum()
     chi2 = ((counts - n * p) ** 2 / (n * p)).sum()
     assert chi2 < 16.27  # 3 degrees of freedom, p = 0.001
+
+
+def test_uniform_numbers_of_many_rows_equal_the_ones_of_each_row():
+    """The sampler draws a step's uniform numbers for all rows at once (64-bit arithmetic that wraps in numpy); they
+    are the numbers `uniform_for` gives row by row with Python integers."""
+    from allpaca_amd.sampling.sampler import uniform_for, uniforms_for
+    rng = np.random.default_rng(0)
+    seeds = [int(x) for x in rng.integers(0, 2 ** 63, size=500)] + [0, 1, 2 ** 64 - 1, 2 ** 63, 12345]
+    idx = [int(x) for x in rng.integers(0, 1 << 20, size=len(seeds))]
+    one = np.asarray([uniform_for(s, i) for s, i in zip(seeds, idx)], dtype=np.float32)
+    many = uniforms_for(seeds, idx)
+    assert many.dtype == np.float32 and np.array_equal(one, many) and (many >= 0).all() and (many < 1).all()
