@@ -394,6 +394,10 @@ static int launch_partials(const void* A, int lda, const void* W, const void* Wu
   if (K % 8 || lda % 8 || !aligned16(A) || !aligned16(W) || (Wu && !aligned16(Wu))) return APC_ERR_UNSUPPORTED;
   const int n_mats = Wu ? 2 : 1;
   if (k_split * n_mats > 65535) return APC_ERR_BAD_ARG;
+  if (!Wu) {  // many rows: the slices on the kernel that keeps the weights out of LDS, where it takes them
+    const int e = launch_gemm_direct_slices((const bf16_t*)A, lda, (const bf16_t*)W, workspace, M, N, K, k_split, stream);
+    if (e != APC_ERR_UNSUPPORTED) return e;
+  }
   // up to 64 rows: tiles of 64 rows (half the loads of activations and half the MFMAs of a 128-row tile)
 #define PARTIAL_LAUNCH(EVEN_, BM_)                                                                                  \
   hipLaunchKernelGGL((gemm_bf16_kernel<G_PARTIAL, EVEN_, BM_>), dim3(ceil_div(N, BN), ceil_div(M, BM_), k_split * n_mats), \
@@ -411,6 +415,33 @@ static int launch_partials(const void* A, int lda, const void* W, const void* Wu
   return 0;
 }
 
+// The plain finishing steps (no folded norm, no SwiGLU) four outputs a thread: the slices added in order, then stored
+// or added into the residual.  N and ldc multiples of 4, 16-byte aligned rows.  (One output a thread takes 34 us for
+// 2,048 x 4,096 outputs in two slices, this 13.)
+__global__ __launch_bounds__(256) void gemm_finish4_kernel(const float* __restrict__ partials, int k_split, int M, int N,
+                                                           int mode, void* __restrict__ C, int ldc) {
+  const int n4 = N / 4;
+  const size_t total = (size_t)M * n4, plane = (size_t)M * N;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+    const int m = (int)(i / n4), n = (int)(i % n4) * 4;
+    const float* src = partials + (size_t)m * N + n;
+    floatx4 g = *reinterpret_cast<const floatx4*>(src);
+    for (int s = 1; s < k_split; ++s) g += *reinterpret_cast<const floatx4*>(src + s * plane);
+    const size_t o = (size_t)m * ldc + n;
+    if (mode == G_STORE_BF16) {
+      uint2 pk;
+      pk.x = pack_bf16x2(g[0], g[1]);
+      pk.y = pack_bf16x2(g[2], g[3]);
+      *reinterpret_cast<uint2*>((bf16_t*)C + o) = pk;
+    } else if (mode == G_STORE_F32) {
+      *reinterpret_cast<floatx4*>((float*)C + o) = g;
+    } else {
+      floatx4* dst = reinterpret_cast<floatx4*>((float*)C + o);
+      *dst = *dst + g;
+    }
+  }
+}
+
 static int launch_splitk(const void* A, int lda, const void* W, const void* Wu, void* C, int ldc, int M, int N, int K,
                          int mode, int k_split, float* workspace, int pre, int emit, FinishNorm norm,
                          hipStream_t stream) {
@@ -419,6 +450,13 @@ static int launch_splitk(const void* A, int lda, const void* W, const void* Wu, 
   if (mode < 0 || mode > G_SWIGLU || (mode == G_SWIGLU) != (Wu != nullptr)) return APC_ERR_BAD_ARG;
   const int e = launch_partials(A, lda, W, Wu, M, N, K, k_split, workspace, stream);
   if (e) return e;
+  if (!pre && !emit && mode != G_SWIGLU && N % 4 == 0 && ldc % 4 == 0 && aligned16(C) && (long)M * N >= (1L << 20)) {
+    const long want = ((long)M * (N / 4) + 255) / 256;
+    hipLaunchKernelGGL(gemm_finish4_kernel, dim3((unsigned)(want < 8192 ? want : 8192)), dim3(256), 0, stream, workspace,
+                       k_split, M, N, mode, C, ldc);
+    APC_LAUNCH_CHECK();
+    return 0;
+  }
   const dim3 grid(ceil_div(N, 256), M);
 #define FINISH(PRE_, EMIT_)                                                                                     \
   hipLaunchKernelGGL((gemm_finish_kernel<PRE_, EMIT_>), grid, dim3(256), 0, stream, workspace, k_split, M, N, K, mode, \
@@ -492,6 +530,10 @@ __global__ __launch_bounds__(256) void gemm_finish_qkv_rope_kernel(const float* 
 // Product for 17..128 rows: K is cut into `k_split` slices that different blocks multiply, so that matrices with
 // few output columns still give the chip enough blocks; `workspace` holds (Wu ? 2 : 1) * k_split * M * N floats.
 // mode as below, or 3 for SwiGLU (W = gate, Wu = up).
+// How many slices of K the product of many rows (gemm_direct_bf16.hip) wants for this shape: 1, or 2 when narrow
+// tiles would be needed to fill the chip otherwise.  The caller brings the workspace for apc_gemm_splitk_bf16.
+APC_EXPORT int apc_gemm_direct_k_split(int M, int N, int K) { return gemm_direct_k_split(M, N, K); }
+
 APC_EXPORT int apc_gemm_splitk_bf16(const void* A, int lda, const void* W, const void* Wu, void* C, int ldc, int M,
                                     int N, int K, int mode, int k_split, float* workspace, hipStream_t stream) {
   return launch_splitk(A, lda, W, Wu, C, ldc, M, N, K, mode, k_split, workspace, 0, 0, FinishNorm{}, stream);

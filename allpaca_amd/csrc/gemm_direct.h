@@ -12,3 +12,8 @@ bool gemm_direct_takes(int mode, const void* A, int lda, const void* C, int ldc,
 // W, W2 in the tiled layout.  APC_ERR_UNSUPPORTED for a shape that gemm_direct_takes refuses.
 int launch_gemm_direct(int mode, const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M,
                        int N, int K, hipStream_t stream);
+// Slices of K that a product of M rows into N columns should be cut into (1: none).  With more than one:
+// launch_gemm_direct_slices leaves float32 sums in partials[slice][M][N], K a multiple of k_split * 128.
+int gemm_direct_k_split(int M, int N, int K);
+int launch_gemm_direct_slices(const bf16_t* A, int lda, const bf16_t* W, float* partials, int M, int N, int K,
+                              int k_split, hipStream_t stream);

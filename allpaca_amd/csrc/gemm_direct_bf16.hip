@@ -231,23 +231,36 @@ __global__ __launch_bounds__(256, 1) void gemm_direct_kernel(const bf16_t* __res
   direct_tile<8, NF, MODE>(blockIdx.x, A, lda, W, W2, chunks, C, ldc, M, N, K);
 }
 
+// K in `gridDim.y` slices of k_slice columns: slice s leaves its float32 sums in partials[s][M][N] (the tiled product's
+// finishing kernel adds the slices in order and runs the epilogue).
+template <int NF>
+__global__ __launch_bounds__(256, 1) void gemm_direct_slices_kernel(const bf16_t* __restrict__ A, int lda,
+                                                                    const bf16_t* __restrict__ W, int chunks,
+                                                                    float* __restrict__ partials, int M, int N,
+                                                                    int k_slice) {
+  const int s = blockIdx.y;
+  direct_tile<8, NF, D_STORE_F32>(blockIdx.x, A + (size_t)s * k_slice, lda, W + (size_t)s * (k_slice / 32) * 512, nullptr,
+                                  chunks, partials + (size_t)s * M * N, N, M, N, k_slice);
+}
+
 // Which NF takes a shape: a launch runs ceil(blocks / 256) rounds of one block a compute unit, and a round of blocks
 // with NF bands a wave takes about 44 + 7.25 NF time units (measured at 2,048 rows: 73, 84 and 102 us a round of 4,096
 // columns of K for NF = 4, 6, 8); 3 and 5 bands give the 3,072 and 5,120 columns of a 3B model one full round.
 // (Tried and taken out: one launch in which the columns of a nearly empty last round go to tiles of 64 rows.  With
 // 2,048 rows x 14,336 SwiGLU outputs, 3.5 rounds of 128-row tiles, it took 589 us against 453 us: a 64-row tile moves
 // 72 KiB through the load path per 64 columns of K for half the MFMAs.)
-int pick_bands(int M, int N, bool swiglu) {
+int pick_bands(int M, int N, bool swiglu, int k_split = 1, double* cost_out = nullptr) {
   const int mt = ceil_div(M, 128);
   int best = 0;
   double best_cost = 0.0;
   for (int nf : {3, 4, 5, 6, 8}) {
     if (swiglu && nf % 2) continue;  // half of a wave's bands are gate, half up
     const int nb = 4 * (swiglu ? nf / 2 : nf) * 16;
-    const long blocks = (long)mt * ceil_div(N, nb);
+    const long blocks = (long)mt * ceil_div(N, nb) * k_split;
     const double cost = (double)((blocks + 255) / 256) * (44.0 + 7.25 * nf);
     if (!best || cost <= best_cost) best = nf, best_cost = cost;
   }
+  if (cost_out) *cost_out = best_cost;
   return best;
 }
 
@@ -277,6 +290,44 @@ int launch_mode(int nf, const bf16_t* A, int lda, const bf16_t* W, const bf16_t*
 
 }  // namespace
 
+// A product with few output columns fills one round of blocks only with narrow tiles (4 bands a wave for the 4,096
+// columns of an 8B model at 2,048 rows), which move the most bytes through L2 per MFMA.  K in two slices gives the
+// wide tiles (8 bands) a full round: down of an 8B model (K = 14,336) 276 -> 207 us plus the kernel that adds the
+// slices.  Time units as in pick_bands, per 4,096 columns of K; the adding kernel about 12 units per 2,048 x 4,096
+// outputs and slice pair, and a launch 5.
+int gemm_direct_k_split(int M, int N, int K) {
+  if (M < GEMM_DIRECT_MIN_ROWS || K % 256 || N % 4 || K < 4096) return 1;
+  double whole = 0.0, halves = 0.0;
+  pick_bands(M, N, false, 1, &whole);
+  pick_bands(M, N, false, 2, &halves);
+  const double k_units = K / 4096.0;
+  const double add = 12.0 * ((double)M * N / (2048.0 * 4096.0)) + 5.0;
+  return halves * k_units / 2 + add < 0.92 * whole * k_units ? 2 : 1;
+}
+
+int launch_gemm_direct_slices(const bf16_t* A, int lda, const bf16_t* W, float* partials, int M, int N, int K,
+                              int k_split, hipStream_t stream) {
+  if (k_split < 1 || k_split > 65535 || K % k_split) return APC_ERR_UNSUPPORTED;
+  const int k_slice = K / k_split;
+  if (!gemm_direct_takes(D_STORE_F32, A, lda, partials, N, M, N, k_slice)) return APC_ERR_UNSUPPORTED;
+  const int nf = pick_bands(M, N, false, k_split);
+  const int nb = 4 * nf * 16;
+  const long blocks = 8L * ceil_div(ceil_div(N, nb), 8) * ceil_div(M, 128);
+  if (blocks > 0x7fffffffL) return APC_ERR_BAD_ARG;
+  const dim3 grid((unsigned)blocks, (unsigned)k_split);
+#define SLICES(NF_)                                                                                              \
+  hipLaunchKernelGGL((gemm_direct_slices_kernel<NF_>), grid, dim3(256), 0, stream, A, lda, W, ceil_div(K, 32), partials, \
+                     M, N, k_slice)
+  if (nf == 3) SLICES(3);
+  else if (nf == 4) SLICES(4);
+  else if (nf == 5) SLICES(5);
+  else if (nf == 6) SLICES(6);
+  else SLICES(8);
+#undef SLICES
+  APC_LAUNCH_CHECK();
+  return 0;
+}
+
 bool gemm_direct_takes(int mode, const void* A, int lda, const void* C, int ldc, int M, int N, int K) {
   if (mode < 0 || mode > D_SWIGLU || M < GEMM_DIRECT_MIN_ROWS || K < 128 || K % 128 || N % 4 || ldc % 4) return false;
   if (((uintptr_t)A & 15u) || ((uintptr_t)C & 15u) || lda % 8) return false;
@@ -285,14 +336,47 @@ bool gemm_direct_takes(int mode, const void* A, int lda, const void* C, int ldc,
   return true;
 }
 
-int launch_gemm_direct(int mode, const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M,
-                       int N, int K, hipStream_t stream) {
-  if (!gemm_direct_takes(mode, A, lda, C, ldc, M, N, K) || (mode == D_SWIGLU) != (W2 != nullptr)) return APC_ERR_UNSUPPORTED;
-  const int nf = pick_bands(M, N, mode == D_SWIGLU);
+namespace {
+int launch_columns(int nf, int mode, const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M,
+                   int N, int K, hipStream_t stream) {
   switch (mode) {
     case D_STORE_BF16: return launch_mode<D_STORE_BF16>(nf, A, lda, W, W2, C, ldc, M, N, K, stream);
     case D_STORE_F32: return launch_mode<D_STORE_F32>(nf, A, lda, W, W2, C, ldc, M, N, K, stream);
     case D_ACC_F32: return launch_mode<D_ACC_F32>(nf, A, lda, W, W2, C, ldc, M, N, K, stream);
     default: return launch_mode<D_SWIGLU>(nf, A, lda, W, W2, C, ldc, M, N, K, stream);
   }
+}
+}  // namespace
+
+int launch_gemm_direct(int mode, const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M,
+                       int N, int K, hipStream_t stream) {
+  if (!gemm_direct_takes(mode, A, lda, C, ldc, M, N, K) || (mode == D_SWIGLU) != (W2 != nullptr)) return APC_ERR_UNSUPPORTED;
+  const bool swiglu = mode == D_SWIGLU;
+  double whole = 0.0;
+  const int nf = pick_bands(M, N, swiglu, 1, &whole);
+  // A launch whose last round is far from full (2,048 rows x 14,336 SwiGLU outputs: 3.5 rounds of tiles with 8 bands a
+  // wave) in two: the columns that make whole rounds, then the rest on whatever tile fills a round best (there: 4
+  // bands, a round of 0.72 of the time).  3 time units for the second launch.
+  const int mt = ceil_div(M, 128);
+  int best_nf = 0, best_cols = 0, rest_nf = 0;
+  double best = whole;
+  if (mt <= 256) {
+    for (int f : {3, 4, 5, 6, 8}) {
+      if (swiglu && f % 2) continue;
+      const int nb = 4 * (swiglu ? f / 2 : f) * 16, nt = ceil_div(N, nb);
+      const int big_cols = (int)((long)mt * nt / 256 * 256 / mt);
+      if (big_cols <= 0 || big_cols >= nt) continue;
+      double rest = 0.0;
+      const int rf = pick_bands(M, N - big_cols * nb, swiglu, 1, &rest);
+      const double cost = (double)ceil_div((long)big_cols * mt, 256L) * (44.0 + 7.25 * f) + rest + 3.0;
+      if (cost < 0.97 * best) best = cost, best_nf = f, best_cols = big_cols * nb, rest_nf = rf;
+    }
+  }
+  if (!best_nf) return launch_columns(nf, mode, A, lda, W, W2, C, ldc, M, N, K, stream);
+  const int e = launch_columns(best_nf, mode, A, lda, W, W2, C, ldc, M, best_cols, K, stream);
+  if (e) return e;
+  const size_t w_skip = (size_t)(best_cols / 16) * ceil_div(K, 32) * 512;  // whole bands of the tiled layout
+  const size_t elem = (mode == D_STORE_BF16 || swiglu) ? 2 : 4;
+  return launch_columns(rest_nf, mode, A, lda, W + w_skip, swiglu ? W2 + w_skip : W2, (char*)C + (size_t)best_cols * elem,
+                        ldc, M, N - best_cols, K, stream);
 }

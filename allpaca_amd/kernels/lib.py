@@ -51,6 +51,7 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_gemm_splitk_qkv_rope_bf16": [P, I, P, I, F, P, P, I, I, I, I, I, I, P, P, P, P, I, P, I, I, P, P],
         "apc_gemm_splitk_pre_bf16": [P, I, P, I, F, P, P, P, I, I, I, I, I, I, P, P],
         "apc_gemm_splitk_bf16": [P, I, P, P, P, I, I, I, I, I, I, P, P],
+        "apc_gemm_direct_k_split": [I, I, I],
         "apc_skinny_gemm_bf16": [P, I, P, P, I, I, I, I, I, P],
         "apc_skinny_swiglu_bf16": [P, I, P, P, P, I, I, I, I, P],
         "apc_attention_prefill_bf16": [P, I, I, P, I, I, I, I, P, I, P, I, P, P, P, P, I, I, F, P],
@@ -93,7 +94,8 @@ class KernelTimer:
 
 _timer = None
 # entry points that launch nothing (questions about sizes): never timed
-NOT_KERNELS = {"apc_attention_decode_whole_fits", "apc_attention_decode_last_fits", "apc_attention_prefill_tile_rows"}
+NOT_KERNELS = {"apc_attention_decode_whole_fits", "apc_attention_decode_last_fits", "apc_attention_prefill_tile_rows",
+               "apc_gemm_direct_k_split"}
 
 
 class timing:

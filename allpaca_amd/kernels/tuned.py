@@ -81,8 +81,9 @@ def gemm_bf16(a: torch.Tensor, w: PackedWeight, out: torch.Tensor, accumulate: b
     lda, ldc = _ops._rows(a, "a"), _ops._rows(out, "out")
     mode = 2 if accumulate else (0 if out.dtype == torch.bfloat16 else 1)
     L = _lib.load("tuned")
-    if SKINNY_MAX_ROWS < M <= MANY_ROWS_SPLIT_MAX:
-        ks = _tiled_k_split(M, N, K)
+    if M > SKINNY_MAX_ROWS:
+        # more than 1,024 rows: the product of many rows says itself whether it wants K in two slices
+        ks = _tiled_k_split(M, N, K) if M <= MANY_ROWS_SPLIT_MAX else L.apc_gemm_direct_k_split(M, N, K)
         if ks > 1:
             ws = torch.empty(ks * M * N, dtype=torch.float32, device=a.device)
             _lib.check(L.apc_gemm_splitk_bf16(a.data_ptr(), lda, w.data.data_ptr(), 0, out.data_ptr(), ldc, M, N, K,

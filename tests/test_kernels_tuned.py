@@ -62,7 +62,9 @@ GEMM_SHAPES = [(1, 5, 16), (3, 100, 136), (8, 4096, 512), (16, 33, 1208), (17, 2
                (2048, 4096, 1024),
                (2048, 10240, 128), (1100, 16384, 256),
                # 3 and 5 bands a wave: the widths of a 3B model (3,072 and 5,120 columns)
-               (2048, 3072, 128), (2048, 5120, 256)]
+               (2048, 3072, 128), (2048, 5120, 256),
+               # few output columns and a long K: K in two slices on that kernel, then the kernel that adds them
+               (2048, 1024, 8192), (1100, 512, 4096)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
