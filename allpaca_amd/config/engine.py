@@ -22,6 +22,9 @@ class EngineConfig:
     max_active_requests: int = 64
     max_batch_tokens: int = 2048       # token budget of one step
     chunk_tokens: int = 512            # largest portion of one prompt in a step
+    # rows of a tile of the bfloat16 matrix products: a step that overshoots a multiple of it by a few rows has its
+    # last prompt portion cut back to the multiple (0: never)
+    step_row_tile: int = 128
     seed: int = 0xA110ACA              # crates/allpaca-core/src/sampling.rs:5-8
     use_graphs: bool = True            # replay decode-only steps as HIP graphs
     device: str = "cuda:0"

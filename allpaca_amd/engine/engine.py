@@ -52,7 +52,8 @@ class Engine:
         self.config, self.model_config, self.model = cfg, model_config, model
         num_pages = cfg.num_pages or -(-cfg.max_tokens // cfg.page_tokens) or self.pages_that_fit(model, cfg)
         self.runner = ModelRunner(model, cfg.page_tokens, num_pages, cfg.max_active_requests, use_graphs=cfg.use_graphs)
-        self.scheduler = Scheduler(self.runner.cache, cfg.max_active_requests, cfg.max_batch_tokens, cfg.chunk_tokens)
+        self.scheduler = Scheduler(self.runner.cache, cfg.max_active_requests, cfg.max_batch_tokens, cfg.chunk_tokens,
+                                   row_tile=cfg.step_row_tile if cfg.dtype == "bfloat16" else 0)
         self.sampler = Sampler(self.runner.rt.device, cfg.seed)
         self.requests: Dict[int, Request] = {}
         self._ahead: Optional[_AheadStep] = None

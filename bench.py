@@ -284,10 +284,15 @@ def kernel_times(cfg_json, args, layers):
             eng.step()
     kv = kv_bytes_per_token(cfg, layers, 2 if args.dtype == "bf16" else 4)
     out[f"decode_b{B}_ctx{ctx}"] = kernel_table(t.totals(), steps, attention_bytes=B * (ctx + 5) * kv)
-    # a mixed step: 512 tokens of a new prompt beside the B decoding rows; host time = until the launches are queued
+    # a mixed step: a portion of a new prompt beside the B decoding rows, as long as the scheduler makes it (a chunk of
+    # 512 tokens, cut back so that the step's rows are whole tiles); host time = until the launches are queued
     ids = [r.id for r in eng.scheduler.running]
     eng.runner.admit("mixed")
-    mixed = lambda at: [Entry("mixed", rng.integers(0, cfg.vocab_size, size=512).tolist(), [511])] + \
+    tile = eng.scheduler.row_tile
+    portion = 512
+    if tile and 0 < (portion + B) % tile <= tile // 4:
+        portion -= (portion + B) % tile
+    mixed = lambda at: [Entry("mixed", rng.integers(0, cfg.vocab_size, size=portion).tolist(), [portion - 1])] + \
         [Entry(i, [1], [0]) for i in ids]
     eng.runner.step(mixed(0))
     torch.cuda.synchronize()
@@ -305,8 +310,8 @@ def kernel_times(cfg_json, args, layers):
     with klib.timing() as t:
         eng.runner.step(mixed(9))
     hd = cfg.num_attention_heads * cfg.head_dim
-    out[f"mixed_512_plus_b{B}"] = kernel_table(t.totals(), 1, attention_bytes=B * ctx * kv,
-                                               attention_flops=layers * 4 * hd * 512 * (512 * 4 + 256))
+    out[f"mixed_{portion}_plus_b{B}"] = kernel_table(t.totals(), 1, attention_bytes=B * ctx * kv,
+                                                     attention_flops=layers * 4 * hd * portion * (portion * 4 + portion // 2))
     out["host_us_mixed_step"] = {"host_launch_us": round(min(host), 1), "gpu_us": round(min(gpu), 1)}
     eng.runner.release("mixed")
     # prefill of 2,048 tokens in one step

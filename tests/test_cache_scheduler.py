@@ -405,3 +405,36 @@ def test_a_cache_need_must_describe_itself():
         kind = "pages"
     with pytest.raises(TypeError, match="page_shape"):
         CacheManager([Nothing()], 8, 4, 2)
+
+
+def test_a_step_that_overshoots_a_multiple_of_the_row_tile_is_trimmed():
+    """Two decoded tokens beside a prompt portion of 32 would be 34 rows, two more than two tiles of 16: the portion
+    is cut back to 30 and the two tokens go into the next one.  Nothing is trimmed when the overshoot is more than a
+    quarter tile, when the step has fewer than two tiles, or when the portion would lose more than half."""
+    cm = CacheManager([FULL], 4, 64, max_requests=4)
+    s = Scheduler(cm, 4, 64, 32, row_tile=16)
+    d1, d2, a = req(0, 3, max_tokens=50), req(1, 2, max_tokens=50), req(2, 70)
+    s.add(d1)
+    s.add(d2)
+    run_step(cm, s)                      # both short prompts whole: 5 rows, nothing to trim
+    s.add(a)
+    p = run_step(cm, s)
+    assert [(e.request.id, e.count, e.samples) for e in p.scheduled] == [(0, 1, True), (1, 1, True), (2, 30, False)]
+    p = run_step(cm, s)                  # 2 + 32 again: 30 more
+    assert [(e.request.id, e.start, e.count) for e in p.scheduled] == [(0, 4, 1), (1, 3, 1), (2, 30, 30)]
+    p = run_step(cm, s)                  # 10 left: 12 rows, under two tiles, untouched, and it samples
+    assert [(e.request.id, e.start, e.count, e.samples) for e in p.scheduled][-1] == (2, 60, 10, True)
+    # an overshoot of 6 of 16 stays (more than a quarter tile)
+    cm2 = CacheManager([FULL], 4, 64, max_requests=4)
+    s2 = Scheduler(cm2, 4, 64, 38, row_tile=16)
+    s2.add(req(0, 38))
+    assert [e.count for e in run_step(cm2, s2).scheduled] == [38]
+    # a portion that would lose more than half of itself stays: 31 decoded rows beside a portion of 3 are 34 rows
+    cm3 = CacheManager([FULL], 4, 256, max_requests=40)
+    s3 = Scheduler(cm3, 40, 64, 32, row_tile=16)
+    for i in range(31):
+        s3.add(req(i, 1, max_tokens=50))
+    run_step(cm3, s3)
+    s3.add(req(99, 3))
+    p = run_step(cm3, s3)                # cutting 2 of 3 is not allowed: it stays whole
+    assert p.scheduled[-1].count == 3 and p.scheduled[-1].samples
