@@ -85,16 +85,20 @@ __device__ __forceinline__ void direct_tile(int bid, const bf16_t* __restrict__ 
   constexpr int NB = 4 * NOUT * 16;                     // outputs of a block
   int mt, nt;
   {
-    // consecutive block ids go to the 8 XCDs in turn (an L2 each): XCD x takes the column tiles x, x + 8, ..; inside
-    // it groups of up to 16 row tiles sweep those columns, row tile fastest, so the blocks that run on an XCD at one
-    // time share a few panels of W
-    const int MT = ceil_div(M, BMG * 16), NT = ceil_div(N, NB), NL = ceil_div(NT, 8);
+    // Consecutive block ids go to the 8 XCDs in turn (an L2 each).  The tiles are put in one order: groups of up to 16
+    // row tiles, inside a group column tile by column tile, row tile fastest; XCD x takes the x-th eighth of that
+    // order, so the blocks that run on an XCD at one time share a few panels of W, and every XCD gets the same number
+    // of tiles whatever the number of column tiles (20 column tiles of 12 rows each dealt out by whole columns gave
+    // four XCDs 36 tiles for their 32 compute units and the others 24: two rounds for 240 tiles).
+    const int MT = ceil_div(M, BMG * 16), NT = ceil_div(N, NB);
     constexpr int GM = 16;
-    const int xcd = bid % 8, j = bid / 8;
-    const int first_m = j / (GM * NL) * GM, gsz = min(MT - first_m, GM), jj = j % (GM * NL);
-    mt = first_m + jj % gsz;
-    nt = jj / gsz * 8 + xcd;
-    if (nt >= NT || mt >= MT) return;
+    const int per_xcd = ceil_div(MT * NT, 8);
+    const int slot = bid / 8;
+    const int t = (bid % 8) * per_xcd + slot;
+    if (slot >= per_xcd || t >= MT * NT) return;
+    const int group = t / (GM * NT), first_m = group * GM, gsz = min(MT - first_m, GM), r = t - group * GM * NT;
+    nt = r / gsz;
+    mt = first_m + r % gsz;
   }
   const int m0 = mt * BMG * 16;
   const int bands = (N + 15) / 16;
@@ -244,11 +248,13 @@ __global__ __launch_bounds__(256, 1) void gemm_direct_slices_kernel(const bf16_t
 }
 
 // Which NF takes a shape: a launch runs ceil(blocks / 256) rounds of one block a compute unit, and a round of blocks
-// with NF bands a wave takes about 44 + 7.25 NF time units (measured at 2,048 rows: 73, 84 and 102 us a round of 4,096
-// columns of K for NF = 4, 6, 8); 3 and 5 bands give the 3,072 and 5,120 columns of a 3B model one full round.
+// with NF bands a wave takes about 27 + 10.8 NF time units (measured at 2,048 rows with weights from HBM: 58, 74, 86, 92
+// and 112 us a round of 4,096 columns of K for NF = 3, 4, 5, 6, 8); 3 and 5 bands give the 3,072 and 5,120 columns of
+// a 3B model one full round.
 // (Tried and taken out: one launch in which the columns of a nearly empty last round go to tiles of 64 rows.  With
 // 2,048 rows x 14,336 SwiGLU outputs, 3.5 rounds of 128-row tiles, it took 589 us against 453 us: a 64-row tile moves
 // 72 KiB through the load path per 64 columns of K for half the MFMAs.)
+constexpr double round_cost(int nf) { return 27.0 + 10.8 * nf; }
 int pick_bands(int M, int N, bool swiglu, int k_split = 1, double* cost_out = nullptr) {
   const int mt = ceil_div(M, 128);
   int best = 0;
@@ -257,7 +263,7 @@ int pick_bands(int M, int N, bool swiglu, int k_split = 1, double* cost_out = nu
     if (swiglu && nf % 2) continue;  // half of a wave's bands are gate, half up
     const int nb = 4 * (swiglu ? nf / 2 : nf) * 16;
     const long blocks = (long)mt * ceil_div(N, nb) * k_split;
-    const double cost = (double)((blocks + 255) / 256) * (44.0 + 7.25 * nf);
+    const double cost = (double)((blocks + 255) / 256) * round_cost(nf);
     if (!best || cost <= best_cost) best = nf, best_cost = cost;
   }
   if (cost_out) *cost_out = best_cost;
@@ -268,7 +274,7 @@ template <int NF, int MODE>
 int launch(const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M, int N, int K,
            hipStream_t stream) {
   constexpr int NB = 4 * (MODE == D_SWIGLU ? NF / 2 : NF) * 16;
-  const long blocks = 8L * ceil_div(ceil_div(N, NB), 8) * ceil_div(M, 128);
+  const long blocks = 8L * ceil_div((long)ceil_div(N, NB) * ceil_div(M, 128), 8L);
   if (blocks > 0x7fffffffL) return APC_ERR_BAD_ARG;
   hipLaunchKernelGGL((gemm_direct_kernel<NF, MODE>), dim3((unsigned)blocks), dim3(256), 0, stream, A, lda, W, W2,
                      ceil_div(K, 32), C, ldc, M, N, K);
@@ -293,15 +299,15 @@ int launch_mode(int nf, const bf16_t* A, int lda, const bf16_t* W, const bf16_t*
 // A product with few output columns fills one round of blocks only with narrow tiles (4 bands a wave for the 4,096
 // columns of an 8B model at 2,048 rows), which move the most bytes through L2 per MFMA.  K in two slices gives the
 // wide tiles (8 bands) a full round: down of an 8B model (K = 14,336) 276 -> 207 us plus the kernel that adds the
-// slices.  Time units as in pick_bands, per 4,096 columns of K; the adding kernel about 12 units per 2,048 x 4,096
-// outputs and slice pair, and a launch 5.
+// slices.  Time units as in pick_bands, per 4,096 columns of K; the adding kernel about 22 units per 2,048 x 4,096
+// outputs and slice pair, and a launch 3.
 int gemm_direct_k_split(int M, int N, int K) {
   if (M < GEMM_DIRECT_MIN_ROWS || K % 256 || N % 4 || K < 4096) return 1;
   double whole = 0.0, halves = 0.0;
   pick_bands(M, N, false, 1, &whole);
   pick_bands(M, N, false, 2, &halves);
   const double k_units = K / 4096.0;
-  const double add = 12.0 * ((double)M * N / (2048.0 * 4096.0)) + 5.0;
+  const double add = 22.0 * ((double)M * N / (2048.0 * 4096.0)) + 3.0;
   return halves * k_units / 2 + add < 0.92 * whole * k_units ? 2 : 1;
 }
 
@@ -312,7 +318,7 @@ int launch_gemm_direct_slices(const bf16_t* A, int lda, const bf16_t* W, float* 
   if (!gemm_direct_takes(D_STORE_F32, A, lda, partials, N, M, N, k_slice)) return APC_ERR_UNSUPPORTED;
   const int nf = pick_bands(M, N, false, k_split);
   const int nb = 4 * nf * 16;
-  const long blocks = 8L * ceil_div(ceil_div(N, nb), 8) * ceil_div(M, 128);
+  const long blocks = 8L * ceil_div((long)ceil_div(N, nb) * ceil_div(M, 128), 8L);
   if (blocks > 0x7fffffffL) return APC_ERR_BAD_ARG;
   const dim3 grid((unsigned)blocks, (unsigned)k_split);
 #define SLICES(NF_)                                                                                              \
@@ -368,7 +374,7 @@ int launch_gemm_direct(int mode, const bf16_t* A, int lda, const bf16_t* W, cons
       if (big_cols <= 0 || big_cols >= nt) continue;
       double rest = 0.0;
       const int rf = pick_bands(M, N - big_cols * nb, swiglu, 1, &rest);
-      const double cost = (double)ceil_div((long)big_cols * mt, 256L) * (44.0 + 7.25 * f) + rest + 3.0;
+      const double cost = (double)ceil_div((long)big_cols * mt, 256L) * round_cost(f) + rest + 3.0;
       if (cost < 0.97 * best) best = cost, best_nf = f, best_cols = big_cols * nb, rest_nf = rf;
     }
   }
