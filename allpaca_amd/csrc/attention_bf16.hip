@@ -20,11 +20,14 @@
 // value product (as every activation between two matrix products is in this path).
 // Formula: crates/allpaca-cpu/src/kernels.rs:293-356.  Reference kernels (contiguous K/V, no matrix
 // cores): attention_qtile_kernel hip/src/kernels.cpp:2203, attention_split_gqa_kernel 2276, merges 2479-2516.
+#include "attention_wide.h"
 #include "mfma.h"
 #include <math.h>
 
 constexpr int KT = 64;            // keys per tile in the prefill kernel
-constexpr int QT = 64;            // rows per tile in the prefill kernel (4 waves x 16)
+constexpr int QT = 64;            // rows per block in the prefill kernels of this file
+constexpr int TILE_ROWS = ATTN_WIDE_ROWS;  // rows of a tile as the step packs them: two blocks here, one of the wide kernel
+static_assert(TILE_ROWS == 2 * QT, "a tile is two halves");
 constexpr int KPAD = 8;
 
 // Both kernels compute the transposed products  S^T = K Q^T  and  O^T = V^T P^T : the MFMA result then holds, per
@@ -89,7 +92,10 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
       h = id / n_tiles;
     }
   }
-  const int row0 = tile_row0[tile], nrows = tile_rows[tile];
+  // the step's tiles have up to TILE_ROWS rows; this kernel takes them in halves of QT rows (n_tiles counts halves)
+  const int nrows = min(tile_rows[tile / 2] - (tile % 2) * QT, QT);
+  if (nrows <= 0) return;
+  const int row0 = tile_row0[tile / 2] + (tile % 2) * QT;
   const int kvh = h / (H / Hk);
   const int pos0 = positions[row0];
   const int* bt = block_table + (size_t)row_seg[row0] * max_blocks;
@@ -318,7 +324,10 @@ __global__ __launch_bounds__(256) void attn_prefill32_kernel(
       h = id / n_tiles;
     }
   }
-  const int row0 = tile_row0[tile], nrows = tile_rows[tile];
+  // the step's tiles have up to TILE_ROWS rows; this kernel takes them in halves of QT rows (n_tiles counts halves)
+  const int nrows = min(tile_rows[tile / 2] - (tile % 2) * QT, QT);
+  if (nrows <= 0) return;
+  const int row0 = tile_row0[tile / 2] + (tile % 2) * QT;
   const int kvh = h / (H / Hk);
   const int pos0 = positions[row0];
   const int* bt = block_table + (size_t)row_seg[row0] * max_blocks;
@@ -887,7 +896,7 @@ static int check_common(const void* q, int ldq, int q_off, const void* cache, in
 APC_EXPORT int apc_attention_prefill_bf16(const void* q, int ldq, int q_off, void* out, int ldo, int H, int Hk, int d,
                                           const void* cache, int page_tokens, const int* block_table, int max_blocks,
                                           const int* positions, const int* row_seg, const int* tile_row0,
-                                          const int* tile_rows, int n_tiles, int window, float scale,
+                                          const int* tile_rows, int n_tiles, int n_rows, int window, float scale,
                                           hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   int e = check_common(q, ldq, q_off, cache, H, Hk, d, page_tokens);
@@ -895,6 +904,14 @@ APC_EXPORT int apc_attention_prefill_bf16(const void* q, int ldq, int q_off, voi
   if (ldo % 4 || ((uintptr_t)out & 7u)) return APC_ERR_UNSUPPORTED;  // outputs are stored 8 bytes at a time
   if (max_blocks <= 0 || window < 0 || (long)n_tiles * H > 0x7fffffffL) return APC_ERR_BAD_ARG;
   if (!(scale > 0.f)) return APC_ERR_UNSUPPORTED;  // the kernel takes the maximum before it scales
+  // n_rows: the rows of all tiles together.  Tiles that are mostly whole go to the kernel that takes 128 rows a block;
+  // short ones (ends of prompts, many small requests) would leave half of its waves without rows.
+  if (attn_wide_takes(d, page_tokens) && (long)n_rows * 4 >= (long)n_tiles * TILE_ROWS * 3)
+    return launch_attn_prefill_wide((const bf16_t*)q, ldq, q_off, (bf16_t*)out, ldo, H, Hk, (const bf16_t*)cache,
+                                    page_tokens, block_table, max_blocks, positions, row_seg, tile_row0, tile_rows,
+                                    n_tiles, window, scale, stream);
+  n_tiles *= 2;  // halves
+  if ((long)n_tiles * H > 0x7fffffffL) return APC_ERR_BAD_ARG;
   dim3 grid(n_tiles * H), block(256);
 #define PF_LAUNCH(DP_)                                                                                             \
   hipLaunchKernelGGL((attn_prefill_kernel<DP_>), grid, block, 0, stream, (const bf16_t*)q, ldq, q_off, (bf16_t*)out, \
@@ -993,7 +1010,7 @@ APC_EXPORT int apc_attention_decode_last_fits(int H, int Hk, int d, int n_parts)
 
 // Rows of a tile of the prefill kernels: the caller cuts every segment of several rows into tiles of at most this many
 // consecutive rows (tile_row0, tile_rows).
-APC_EXPORT int apc_attention_prefill_tile_rows() { return QT; }
+APC_EXPORT int apc_attention_prefill_tile_rows() { return TILE_ROWS; }
 
 // 1 if a block can take a (row, kv head) whole at these sizes (workspace = null above), else 0.
 APC_EXPORT int apc_attention_decode_whole_fits(int H, int Hk, int d) {

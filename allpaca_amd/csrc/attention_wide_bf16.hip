@@ -1,0 +1,601 @@
+// Attention of prompt portions over the paged cache for a head size of 128: tiles of 128 rows, keys and values
+// straight from global memory into LDS, softmax and matrix products of one wave woven together by hand.
+//
+// A block of 4 waves takes up to 128 consecutive rows of one request and one head: wave (rh, kh) owns the rows
+// rh * 64 .. + 63 (two MFMA tiles of 32 rows, "row tiles") and the keys kh * 32 .. + 31 of every tile of 64 keys, with a
+// reference and a sum per row of its own; the two waves of a row half meet once at the end through LDS.  As in
+// attention_bf16.hip the products are S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16_bf16, so a lane holds
+// scores of one row and P goes from the first product's result registers into the second product's operand.
+// What differs from the 64-row kernel there, and why (that kernel ran at 28 % of the matrix cores' rate on long
+// prompts, with LDS, vector instructions and matrix cores each busy half of the time and waiting for one another):
+// * An operand read from LDS feeds two MFMAs (the two row tiles of the wave) instead of one: one read per MFMA is
+//   all that LDS can deliver when the matrix cores run at their full rate.
+// * Keys and values go from global memory into LDS by direct loads (no registers, no LDS store instructions, no
+//   address arithmetic: a wave's 16 keys lie in one page, whose descriptors sit in scalar registers), four tiles
+//   ahead of their use in four stages.  K rows are not padded; a piece of 16 bytes lies at (piece index XOR row
+//   index) instead, which the direct load does by fetching the piece that belongs at its lane's place, and reads of
+//   16 lanes still fall into different banks.  The rows of a K tile are stored in the order in which the first
+//   product's result registers want them (bits 2 and 3 of the key index swapped), so that a lane's 8 results of a
+//   16-key step are 8 consecutive keys and the matching values are one 16-byte piece of V^T as a page holds it.
+//   V^T lies in LDS as the page holds it for 16 positions ([element of d][16 positions]): a wave's read of 32
+//   elements x 16 keys is 1 KiB in lane order.
+// * One wave a SIMD (O of 64 rows x 128 alone takes 128 accumulation registers), so nothing overlaps by itself: a
+//   pass of the loop is two slots of 16 MFMAs each, and the vector work of one row tile's softmax stands in the
+//   issue slots between the MFMAs of the other's products:
+//     slot A: S0(i + 1) = K(i + 1) Q0 and O0 += V(i) P0(i), beside the softmax of S1(i)
+//     slot B: S1(i + 1) = K(i + 1) Q1 and O1 += V(i) P1(i), beside the softmax of S0(i + 1)
+//   (0, 1: the row tiles; i: the tile of keys).  The fragments of K(i + 1) and V(i) are read from LDS in slot A and
+//   stay in registers for slot B.  Exponentials (a quarter of the rate of other vector instructions) and MFMAs take
+//   about the same time per tile; this order is what lets both run.  Each result is written in one slot and read
+//   in the next, so nothing needs a second set of registers and the loop body has no branch.
+// * A row's reference for the exponents is the largest score among its first keys (the first tile of its wave that
+//   it sees a key of) and stays: O lives in accumulation registers that only MFMAs touch in the loop, so it cannot
+//   shrink there.  P = 2^(score - reference) may then exceed 1: up to 2^64 is let through (sums stay far inside
+//   float32).  If a row ever meets a score beyond that, the block throws its work away and computes its rows again
+//   in a plain loop (one thing after the other, references that move, as attn_prefill32_kernel does).
+// The MFMAs are written as instructions: the compiler does not know them, so it neither waits for their results
+// nor keeps reads behind them; the order of the slots keeps every read of a result at least one MFMA behind the
+// one that wrote it, and the accumulators of O are read only after the loop, behind a wait.
+// Positions outside a block's view that lie in stale slots are cleared in LDS before the value product sees them
+// (only tiles at the edge of a request's keys have any).
+// Formula: crates/allpaca-cpu/src/kernels.rs:293-356.  Reference kernel (contiguous K/V, no matrix cores):
+// attention_qtile_kernel hip/src/kernels.cpp:2203.
+#include "attention_wide.h"
+#include "mfma.h"
+#include <math.h>
+#include <type_traits>
+
+namespace {
+
+constexpr int KT = 64;                     // keys a tile
+constexpr int HD = ATTN_WIDE_HEAD;         // head size
+constexpr int STG = 4;                     // stages of K and of V in LDS
+constexpr int K_STAGE = KT * HD * 2;       // bytes: [64 rows][256]
+constexpr int V_STAGE = HD * KT * 2;       // bytes: [4 groups of 16 keys][128 elements][32]
+constexpr int V_BASE = STG * K_STAGE;
+constexpr int LDS_BYTES = STG * (K_STAGE + V_STAGE);  // of the stages; the block asks for 16 more
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float RISE = 64.f;               // by how much (in powers of 2) a score may exceed its row's reference
+constexpr int LOADS_PER_TILE = 8;          // a wave's direct loads per pass of the loop: 4 of K, 4 of V
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void* lds_ptr;
+
+// The fragments of K and V come out of LDS through ds_read_b128 written as an instruction, and the MFMA that takes one
+// waits for it by count (LDS returns in order; LGKM = how many younger LDS reads may still be out).  Left to the
+// compiler, every LDS read behind a direct load waits until all direct loads have landed: it cannot tell that the
+// loads in flight fill other stages than the one being read.
+template <int OFFSET>
+__device__ __forceinline__ Frag lds_frag(int addr) {
+  u32x4 v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
+  return __builtin_bit_cast(Frag, v);
+}
+#define WAIT_LDS "s_waitcnt lgkmcnt(%3)\n\t"
+// c = a . q and c += a . q with the result in vector registers and q, the wave's query rows, which only MFMAs read, in
+// accumulation registers (an MFMA takes its operands from either file); c += a . b with c in accumulation registers.
+template <int LGKM>
+__device__ __forceinline__ void mfma_set(floatx16& c, const Frag& a, const Frag& q) {
+  asm volatile(WAIT_LDS "v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0"
+               : "=&v"(c) : "v"(__builtin_bit_cast(u32x4, a)), "a"(__builtin_bit_cast(u32x4, q)), "n"(LGKM));
+}
+template <int LGKM>
+__device__ __forceinline__ void mfma_add(floatx16& c, const Frag& a, const Frag& q) {
+  asm volatile(WAIT_LDS "v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0"
+               : "+v"(c) : "v"(__builtin_bit_cast(u32x4, a)), "a"(__builtin_bit_cast(u32x4, q)), "n"(LGKM));
+}
+template <int LGKM>
+__device__ __forceinline__ void mfma_acc(floatx16& c, const Frag& a, const Frag& b) {
+  asm volatile(WAIT_LDS "v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0"
+               : "+a"(c) : "v"(__builtin_bit_cast(u32x4, a)), "v"(__builtin_bit_cast(u32x4, b)), "n"(LGKM));
+}
+#undef WAIT_LDS
+constexpr int NO_WAIT = 15;  // the counter's largest value: an operand that has been in registers for long
+
+template <int N>
+__device__ __forceinline__ void wait_loads_but() {  // until at most N vector memory loads of this wave are in flight
+  __builtin_amdgcn_s_waitcnt(((N & 15) | ((N >> 4) << 14)) | 0x0f70);
+}
+
+// The two halves of a wave exchange a value: every lane gets f(lower half's value, upper half's value).
+__device__ __forceinline__ float halves_max(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float halves_sum(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float exp2_neg(float x) { return __builtin_amdgcn_exp2f(x); }
+// the instruction itself: fmaxf on values the compiler has not seen computed first makes each of them canonical
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
+// all but the positions lo <= p < hi of the 8 that a value piece holds are cleared
+__device__ __forceinline__ void keep_positions(Frag& v, int lo, int hi) {
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const uint32_t a = (2 * w >= lo && 2 * w < hi) ? 0x0000ffffu : 0u;
+    const uint32_t b = (2 * w + 1 >= lo && 2 * w + 1 < hi) ? 0xffff0000u : 0u;
+    v.w[w] &= a | b;
+  }
+}
+
+// Softmax state of one row tile of a wave (a lane: one row, half of the wave's 32 keys of a tile)
+struct Soft {
+  float m, l;      // the row's reference (-inf before its first key) and sum
+  float mx, sum;   // of the tile in work
+  int beyond;      // a score went beyond the reference by more than RISE: the woven loop's result is not to be used
+  int pos, lo;     // the row sees keys lo .. pos
+};
+
+// Step h (0..15) of the softmax of 16 scores: the work is cut up so that it can stand between MFMAs.  s: raw
+// scores, then P; pf: P as the second product's operand; tk: the first of the wave's 32 keys of this tile.
+// Register r of a lane holds key tk + 16 (r / 8) + 8 lh + r % 8.
+__device__ __forceinline__ constexpr int score_step(int r) { return 3 + r * 12 / 16; }
+template <bool MASKED>
+__device__ __forceinline__ void soft_step(int h, floatx16& s, Frag (&pf)[2], Soft& st, int tk, int lh, float sc2) {
+  if (h == 0 || h == 1) {
+    const int r0 = h * 8;
+    if (MASKED) {
+#pragma unroll
+      for (int r = r0; r < r0 + 8; ++r) {
+        const int t = tk + 16 * (r / 8) + 8 * lh + r % 8;
+        s[r] = (t >= st.lo && t <= st.pos) ? s[r] : -INFINITY;
+      }
+    }
+    float mx = h == 0 ? max3(s[0], s[1], s[2]) : max3(st.mx, s[8], s[9]);
+    mx = max3(mx, s[r0 + 3], s[r0 + 4]);
+    mx = max3(mx, s[r0 + 5], s[r0 + 6]);
+    mx = h == 0 ? max3(mx, s[7], s[7]) : max3(mx, s[10], s[15]);
+    st.mx = h == 0 ? mx : halves_max(mx) * sc2;
+  }
+  if (h == 2) {
+    const bool fresh = st.m == -INFINITY;
+    st.beyond |= (!fresh && st.mx > st.m + RISE) ? 1 : 0;
+    st.m = fresh ? st.mx : st.m;
+    st.sum = 0.f;
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    if (score_step(r) == h) {
+      // a row that has seen no key yet: m = -inf and every score is -inf; -inf - -inf would be NaN
+      s[r] = exp2_neg(fmaf(s[r], sc2, st.m == -INFINITY ? 0.f : -st.m));
+      st.sum += s[r];
+    }
+    if ((r & 1) && score_step(r) + 1 == h) pf[r / 8].w[(r % 8) / 2] = pack_bf16x2(s[r - 1], s[r]);
+  }
+  if (h == 15) st.l += halves_sum(st.sum);
+}
+
+__global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
+    const bf16_t* __restrict__ q, int ldq, int q_off, bf16_t* __restrict__ out, int ldo, int H, int Hk,
+    const bf16_t* __restrict__ cache, int lgP, const int* __restrict__ block_table, int max_blocks,
+    const int* __restrict__ positions, const int* __restrict__ row_seg, const int* __restrict__ tile_row0,
+    const int* __restrict__ tile_rows, int n_tiles, int window, float scale) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  constexpr int d = HD;
+  constexpr int DT = d / 32;
+  const int P = 1 << lgP;
+  const int tid = threadIdx.x, lane = tid % WAVE, wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+  const int li = lane % 32, lh = lane / 32;
+  const int rh = wave / 2, kh = wave % 2;  // half of the rows, half of each tile's keys
+  int tile, h;
+  {
+    // heads of one kv head go to one XCD (their keys and values then lie in one L2), long tiles first
+    const int id = blockIdx.x, G = H / Hk;
+    if (Hk % 8 == 0) {
+      const int xcd = id % 8, slot = id / 8;
+      const int lhd = slot / n_tiles;
+      tile = n_tiles - 1 - slot % n_tiles;
+      h = (xcd + 8 * (lhd / G)) * G + lhd % G;
+    } else {
+      tile = n_tiles - 1 - id % n_tiles;
+      h = id / n_tiles;
+    }
+  }
+  const int row0 = tile_row0[tile], nrows = tile_rows[tile];
+  const int kvh = h / (H / Hk);
+  const int pos0 = positions[row0];
+  const int* bt = block_table + (size_t)row_seg[row0] * max_blocks;
+  const int last = pos0 + nrows - 1;
+  const int first = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const size_t page_stride = (size_t)2 * Hk * P * d;
+  const int t_begin = (first / KT) * KT;
+  const int n_kt = (last - t_begin) / KT + 1;
+  const int last16 = (last / 16) * 16;
+  const bf16_t* k_head = cache + (size_t)kvh * P * d;
+  const bf16_t* v_head = cache + (size_t)(Hk + kvh) * P * d;
+  const float sc2 = scale * LOG2E;
+
+  // the wave's 2 x 32 query rows as second operands: row = lane % 32, 8 elements of d per lane and step of 16
+  Frag qf[2][d / 16];
+  Soft st[2];
+  {
+    u32x4 qv[2][d / 16];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+      const int my_row = rh * 64 + rt * 32 + li;
+      const bf16_t* qrow = q + (size_t)(row0 + min(my_row, nrows - 1)) * ldq + q_off + (size_t)h * d;
+#pragma unroll
+      for (int ks = 0; ks < d / 16; ++ks) qv[rt][ks] = __builtin_bit_cast(u32x4, load_frag(qrow + ks * 16 + lh * 8));
+      st[rt].m = -INFINITY;
+      st[rt].l = 0.f;
+      st[rt].mx = st[rt].sum = 0.f;
+      st[rt].beyond = 0;
+      st[rt].pos = pos0 + my_row;
+      st[rt].lo = (window > 0 && st[rt].pos - window + 1 > 0) ? st[rt].pos - window + 1 : 0;
+    }
+    // from here on the values live in accumulation registers (left to the compiler, they are copied there in every pass)
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int ks = 0; ks < d / 16; ++ks) {
+        asm volatile("" : "+a"(qv[rt][ks]));
+        qf[rt][ks] = __builtin_bit_cast(Frag, qv[rt][ks]);
+      }
+  }
+  // whether every row of row tile rt sees all of the wave's 32 keys of the tile that starts at t0
+  auto sees_all = [&](int rt, int t0) {
+    const int tk = t0 + kh * 32, low = pos0 + rh * 64 + rt * 32, top = low + 31;
+    const int win_lo = (window > 0 && top - window + 1 > 0) ? top - window + 1 : 0;
+    return tk + 31 <= low && tk >= win_lo;
+  };
+
+  // ---- direct loads.  Wave w brings the keys 16 w .. + 15 of a tile and their values: they lie in one page (pages
+  // hold a multiple of 16 positions), whose descriptors sit in scalar registers, so a load costs no address arithmetic.
+  // K: load i brings LDS rows 16 w + 4 i .. + 3 = keys 16 w + 4 sw(i) .. + 3, lane -> (row lane / 16, place lane % 16,
+  // which holds piece place ^ row).  V^T: load i brings elements 32 i .. + 31 of the wave's 16 keys, lane -> (element
+  // lane / 2, half lane % 2), into [group w][element][16 keys].
+  int koff[4], voff[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int sw = 2 * (i & 1) + (i >> 1);
+    koff[i] = (4 * sw + lane / 16) * (d * 2) + (((lane % 16) ^ (lane / 16) ^ (4 * i)) * 16);
+    voff[i] = (32 * i + lane / 2) * (P * 2) + (lane % 2) * 16;
+  }
+  auto group_of = [&](int j) { return min(t_begin + j * KT + 16 * wave, last16); };  // first key of the wave's 16
+  auto page_of = [&](int j) { return __builtin_amdgcn_readfirstlane(bt[group_of(j) >> lgP]); };
+  auto k_load = [&](int j, int page) {
+    const BufferRsrc kr = make_rsrc(k_head + (size_t)__builtin_amdgcn_readfirstlane(page) * page_stride);
+    const int soff = (group_of(j) & (P - 1)) * (d * 2);
+    unsigned char* dst = smem + (j % STG) * K_STAGE + (16 * wave) * 256;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, (lds_ptr)(dst + i * 1024), 16, koff[i], soff, 0, 0);
+  };
+  auto v_load = [&](int j, int page) {
+    const BufferRsrc vr = make_rsrc(v_head + (size_t)__builtin_amdgcn_readfirstlane(page) * page_stride);
+    const int soff = (group_of(j) & (P - 1)) * 2;
+    unsigned char* dst = smem + V_BASE + (j % STG) * V_STAGE + wave * 4096;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, (lds_ptr)(dst + i * 1024), 16, voff[i], soff, 0, 0);
+  };
+  // Stale positions of the V^T stage of tile j are cleared: what lies beyond the last key or in front of the first
+  // one that a row of the block sees may be anything, and 0 x NaN is NaN.  (A group of 16 keys beyond the last one
+  // holds a copy of the last group.)
+  auto clear_unseen = [&](int j) {
+    const int t0 = t_begin + j * KT;
+    unsigned char* stage = smem + V_BASE + (j % STG) * V_STAGE;
+    for (int idx = tid; idx < HD * 8; idx += 256) {  // piece idx: group idx / 256, element (idx % 256) / 2, half idx % 2
+      const int t16 = t0 + 16 * (idx / 256), tg = t16 + 8 * (idx % 2);
+      Frag* piece = reinterpret_cast<Frag*>(stage + idx * 16);
+      if (t16 > last16) {
+        *piece = zero_frag();
+      } else if (first - tg > 0 || last - tg + 1 < 8) {
+        Frag f = *piece;
+        keep_positions(f, first - tg, last - tg + 1);
+        *piece = f;
+      }
+    }
+  };
+  auto at_edge = [&](int j) {
+    const int t0 = t_begin + j * KT;
+    return t0 < first || t0 + KT - 1 > last;
+  };
+
+  // ---- operand reads.  K: lane (li, lh) reads piece 2 ks + lh of LDS row kh * 32 + li; V^T: the 16 keys' group
+  // 2 kh + j, element dt * 32 + li, half lh.
+  // (byte offsets in `smem`; the read instruction wants addresses in LDS, which begin at lds0)
+  const int lds0 = (int)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
+  int kaddr[d / 16];
+#pragma unroll
+  for (int ks = 0; ks < d / 16; ++ks) kaddr[ks] = (kh * 32 + li) * 256 + ((((2 * ks) | lh) ^ (li % 16)) * 16);
+  const int vaddr = V_BASE + 2 * kh * 4096 + li * 32 + lh * 16;
+  auto k_frag = [&](int stage_bytes, int ks) { return lds_frag<0>(lds0 + kaddr[ks] + stage_bytes); };
+  // the same through the compiler's own loads (the plain loop)
+  auto k_frag_plain = [&](int stage_bytes, int ks) { return *reinterpret_cast<const Frag*>(smem + kaddr[ks] + stage_bytes); };
+  auto v_frag_plain = [&](int stage_bytes, int g) {
+    return *reinterpret_cast<const Frag*>(smem + vaddr + stage_bytes + (g / 4) * 4096 + (g % 4) * 1024);
+  };
+
+  // The two key halves of a row half meet: wave kh = 1 leaves its reference, sum and O^T of row tile rt in LDS, wave
+  // kh = 0 adds its own and writes the rows.  LDS must be free of other use.
+  float* meet_o = reinterpret_cast<float*>(smem);            // [rh][rt][dt][r][lane]
+  float* meet_ml = meet_o + 2 * 2 * DT * 16 * 64;            // [rh][rt][m, l][32 rows]
+  auto leave = [&](int rt, const floatx16 (&o)[DT], float m, float l) {
+    if (kh != 1) return;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) meet_o[(((rh * 2 + rt) * DT + dt) * 16 + r) * 64 + lane] = o[dt][r];
+    if (lh == 0) {
+      meet_ml[((rh * 2 + rt) * 2 + 0) * 32 + li] = m;
+      meet_ml[((rh * 2 + rt) * 2 + 1) * 32 + li] = l;
+    }
+  };
+  auto add_and_write = [&](int rt, const floatx16 (&o)[DT], float m1, float l1) {
+    const int my_row = rh * 64 + rt * 32 + li;
+    if (kh != 0 || my_row >= nrows) return;
+    const float m2 = meet_ml[((rh * 2 + rt) * 2 + 0) * 32 + li], l2 = meet_ml[((rh * 2 + rt) * 2 + 1) * 32 + li];
+    const float m = fmaxf(m1, m2);
+    const float m_safe = m == -INFINITY ? 0.f : m;
+    const float a1 = exp2_neg(m1 - m_safe), a2 = exp2_neg(m2 - m_safe);
+    const float inv = 1.0f / (l1 * a1 + l2 * a2);
+    bf16_t* orow = out + (size_t)(row0 + my_row) * ldo + (size_t)h * d;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int e = dt * 32 + g * 8 + lh * 4;
+        float y[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          y[r] = (o[dt][g * 4 + r] * a1 + meet_o[(((rh * 2 + rt) * DT + dt) * 16 + g * 4 + r) * 64 + lane] * a2) * inv;
+        uint2 pk;
+        pk.x = pack_bf16x2(y[0], y[1]);
+        pk.y = pack_bf16x2(y[2], y[3]);
+        *reinterpret_cast<uint2*>(orow + e) = pk;
+      }
+    }
+  };
+
+  int& block_beyond = *reinterpret_cast<int*>(smem + LDS_BYTES);  // behind the stages
+  if (tid == 0) block_beyond = 0;
+  {
+    floatx16 o[2][DT];  // O^T of the two row tiles: element dt*32 + (r/4)*8 + lh*4 + r%4 of row li
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[rt][dt][r] = 0.f;
+    floatx16 s0, s1;     // raw scores of the two row tiles, then P
+    Frag p0[2], p1[2];   // P as the second product's operands
+
+    // ---- prologue: K(0); then what the passes -3, -2, -1 of the loop would have issued
+    int kpg, vpg;  // pages of the wave's keys of the tiles whose K and V the next pass loads
+    {
+      const int pg0 = page_of(0), pg1 = page_of(1), pg2 = page_of(2), pg3 = page_of(3);
+      k_load(0, pg0);
+      k_load(1, pg1);
+      v_load(0, pg0);
+      k_load(2, pg2);
+      v_load(1, pg1);
+      k_load(3, pg3);
+      v_load(2, pg2);
+      vpg = pg3;
+      kpg = page_of(4);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    wait_loads_but<3 * LOADS_PER_TILE>();
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    {  // S(0) of both row tiles and the softmax of row tile 0, one thing after the other
+      Frag kf[d / 16];
+#pragma unroll
+      for (int ks = 0; ks < d / 16; ++ks) kf[ks] = k_frag(0, ks);
+#pragma unroll
+      for (int ks = 0; ks < d / 16; ++ks) {
+        if (ks == 0) {
+          mfma_set<0>(s0, kf[ks], qf[0][ks]);
+          mfma_set<NO_WAIT>(s1, kf[ks], qf[1][ks]);
+        } else {
+          mfma_add<NO_WAIT>(s0, kf[ks], qf[0][ks]);
+          mfma_add<NO_WAIT>(s1, kf[ks], qf[1][ks]);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_nop 15\n\ts_nop 15");  // the MFMAs have left the matrix cores: their results may be read
+      __builtin_amdgcn_sched_barrier(0);
+      const int tk = t_begin + kh * 32;
+#pragma unroll
+      for (int hh = 0; hh < 16; ++hh) soft_step<true>(hh, s0, p0, st[0], tk, lh, sc2);
+    }
+
+    // ---- a pass of the loop.  Before pass i: S1(i) raw in s1, P0(i) in p0.  MASKED: some row may not see some key of
+    // tile i (row tile 1) or tile i + 1 (row tile 0), or tile i has stale positions.
+    auto pass = [&](auto MASKED_, int i) {
+      constexpr bool MASKED = decltype(MASKED_)::value;
+      const int t0 = t_begin + i * KT;
+      const int stage_k = ((i + 1) % STG) * K_STAGE, stage_v = (i % STG) * V_STAGE;
+      __builtin_amdgcn_sched_barrier(0);
+      wait_loads_but<2 * LOADS_PER_TILE>();      // K(i + 1) and V(i) are there ...
+      __builtin_amdgcn_s_barrier();              // ... for every wave, and every wave has left K(i) and V(i - 1)
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (MASKED) {
+        if (at_edge(i)) {
+          clear_unseen(i);
+          __syncthreads();
+        }
+      }
+      k_load(i + 4, kpg);
+      v_load(i + 3, vpg);
+      vpg = kpg;
+      kpg = page_of(i + 5);
+      __builtin_amdgcn_sched_barrier(0);
+      Frag kfr[8], vfr[8];
+      {  // slot A.  LDS reads go out two steps ahead, K(i + 1) and V(i) in turn: when a step's MFMA wants its
+         // fragment, the four reads behind it may still be out (fewer in the last steps).
+        const int tk = t0 + kh * 32;
+        const int va = lds0 + vaddr + stage_v;
+        kfr[0] = k_frag(stage_k, 0);
+        vfr[0] = lds_frag<0>(va);
+        kfr[1] = k_frag(stage_k, 1);
+        vfr[1] = lds_frag<1024>(va);
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+          constexpr int out_k[8] = {4, 4, 4, 4, 4, 4, 3, 1}, out_v[8] = {4, 4, 4, 4, 4, 4, 2, 0};
+          if (g + 2 < 8) kfr[g + 2] = k_frag(stage_k, g + 2);
+#define SLOT_A_STEP(G)                                                                      \
+  if (g == G) {                                                                             \
+    if (G == 0) mfma_set<out_k[G]>(s0, kfr[G], qf[0][G]);                                   \
+    else mfma_add<out_k[G]>(s0, kfr[G], qf[0][G]);                                          \
+    soft_step<MASKED>(2 * G, s1, p1, st[1], tk, lh, sc2);                                   \
+    __builtin_amdgcn_sched_barrier(0);                                                      \
+    if (G + 2 < 8) vfr[(G + 2) % 8] = lds_frag<((G + 2) % 8 / 4) * 4096 + ((G + 2) % 4) * 1024>(va); \
+    mfma_acc<out_v[G]>(o[0][G % 4], vfr[G], p0[G / 4]);                                     \
+    soft_step<MASKED>(2 * G + 1, s1, p1, st[1], tk, lh, sc2);                               \
+    __builtin_amdgcn_sched_barrier(0);                                                      \
+  }
+          SLOT_A_STEP(0) SLOT_A_STEP(1) SLOT_A_STEP(2) SLOT_A_STEP(3)
+          SLOT_A_STEP(4) SLOT_A_STEP(5) SLOT_A_STEP(6) SLOT_A_STEP(7)
+#undef SLOT_A_STEP
+        }
+      }
+      {  // slot B: every fragment is in registers
+        const int tk = t0 + KT + kh * 32;
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+          if (g == 0) mfma_set<NO_WAIT>(s1, kfr[g], qf[1][g]);
+          else mfma_add<NO_WAIT>(s1, kfr[g], qf[1][g]);
+          soft_step<MASKED>(2 * g, s0, p0, st[0], tk, lh, sc2);
+          __builtin_amdgcn_sched_barrier(0);
+          mfma_acc<NO_WAIT>(o[1][g % 4], vfr[g], p1[g / 4]);
+          soft_step<MASKED>(2 * g + 1, s0, p0, st[0], tk, lh, sc2);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      // The last MFMAs must have left the matrix cores before O is read.  The compiler does not know these
+      // instructions: it reads the accumulators right behind the loop, in front of any wait that stands there.
+      if (i + 1 >= n_kt) asm volatile("s_nop 15\n\ts_nop 15");
+    };
+    // Passes in which every row sees every key run without the masks: with a window the first passes need them, under
+    // the causal mask the last ones.
+    auto needs_mask = [&](int i) {
+      return !sees_all(1, t_begin + i * KT) || !sees_all(0, t_begin + (i + 1) * KT) || at_edge(i);
+    };
+    int i_open = 0;
+    while (i_open < n_kt && needs_mask(i_open)) ++i_open;
+    int i_close = i_open;
+    while (i_close < n_kt && !needs_mask(i_close)) ++i_close;
+    int i = 0;
+    for (; i < i_open; ++i) pass(std::true_type{}, i);
+    for (; i < i_close; ++i) pass(std::false_type{}, i);
+    for (; i < n_kt; ++i) pass(std::true_type{}, i);
+
+    __builtin_amdgcn_sched_barrier(0);
+    wait_loads_but<0>();                    // no direct load is on its way into LDS
+    __builtin_amdgcn_sched_barrier(0);
+    if (__builtin_amdgcn_ballot_w64((st[0].beyond | st[1].beyond) != 0) != 0 && lane == 0) block_beyond = 1;
+    __syncthreads();
+    if (!block_beyond) {
+      leave(0, o[0], st[0].m, st[0].l);
+      leave(1, o[1], st[1].m, st[1].l);
+      __syncthreads();
+      add_and_write(0, o[0], st[0].m, st[0].l);
+      add_and_write(1, o[1], st[1].m, st[1].l);
+      return;
+    }
+  }
+
+  // ---- the plain loop: a score outran its row's reference somewhere in the block.  One row tile after the other,
+  // one thing after the other, references that move and O shrunk by vector instructions when they do.
+  for (int rt = 0; rt < 2; ++rt) {
+    floatx16 o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+    const int my_pos = st[rt].pos, my_lo = st[rt].lo;
+    for (int j = 0; j < n_kt; ++j) {
+      __syncthreads();  // every wave has left the stage
+      const int pg = page_of(j);
+      k_load(j, pg);
+      v_load(j, pg);
+      wait_loads_but<0>();
+      __syncthreads();
+      if (at_edge(j)) {
+        clear_unseen(j);
+        __syncthreads();
+      }
+      const int stage_k = (j % STG) * K_STAGE, stage_v = (j % STG) * V_STAGE;
+      floatx16 s;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < d / 16; ++ks) s = mfma32(k_frag_plain(stage_k, ks), qf[rt][ks], s);
+      const int tk = t_begin + j * KT + kh * 32;
+      float mx = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int t = tk + 16 * (r / 8) + 8 * lh + r % 8;
+        s[r] = (t >= my_lo && t <= my_pos) ? s[r] : -INFINITY;
+        mx = fmaxf(mx, s[r]);
+      }
+      mx = halves_max(mx) * sc2;
+      const float m_new = fmaxf(m_run, mx);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = exp2_neg(m_run - m_safe);
+      float sum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        s[r] = exp2_neg(fmaf(s[r], sc2, -m_safe));
+        sum += s[r];
+      }
+      l_run = l_run * alpha + halves_sum(sum);
+      m_run = m_new;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj) {
+        Frag pf;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) pf.w[w] = pack_bf16x2(s[8 * jj + 2 * w], s[8 * jj + 2 * w + 1]);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[dt] = mfma32(v_frag_plain(stage_v, jj * 4 + dt), pf, o[dt]);
+      }
+    }
+    __syncthreads();
+    leave(rt, o, m_run, l_run);
+    __syncthreads();
+    add_and_write(rt, o, m_run, l_run);
+  }
+}
+
+}  // namespace
+
+bool attn_wide_takes(int d, int page_tokens) {
+  return d == ATTN_WIDE_HEAD && page_tokens >= 16 && (page_tokens & (page_tokens - 1)) == 0;
+}
+
+int launch_attn_prefill_wide(const bf16_t* q, int ldq, int q_off, bf16_t* out, int ldo, int H, int Hk,
+                             const bf16_t* cache, int page_tokens, const int* block_table, int max_blocks,
+                             const int* positions, const int* row_seg, const int* tile_row0, const int* tile_rows,
+                             int n_tiles, int window, float scale, hipStream_t stream) {
+  if (!attn_wide_takes(ATTN_WIDE_HEAD, page_tokens)) return APC_ERR_UNSUPPORTED;
+  int lgP = 0;
+  while ((1 << lgP) < page_tokens) ++lgP;
+  static bool configured[64] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= 64) return APC_ERR_UNSUPPORTED;
+  if (!configured[dev]) {  // more LDS than a kernel gets without asking
+    e = hipFuncSetAttribute((const void*)attn_prefill_wide_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES + 16);
+    if (e != hipSuccess) return (int)e;
+    configured[dev] = true;
+  }
+  hipLaunchKernelGGL(attn_prefill_wide_kernel, dim3(n_tiles * H), dim3(256), LDS_BYTES + 16, stream, q, ldq, q_off, out, ldo,
+                     H, Hk, cache, lgP, block_table, max_blocks, positions, row_seg, tile_row0, tile_rows, n_tiles,
+                     window, scale);
+  APC_LAUNCH_CHECK();
+  return 0;
+}

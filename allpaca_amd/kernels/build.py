@@ -23,10 +23,10 @@ CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
 
 LIBS: Dict[str, List[str]] = {
     "plain": ["plain_ops.hip", "plain_gemm.hip", "plain_attention.hip", "sampling.hip"],
-    "tuned": ["gemm_bf16.hip", "gemm_wide_bf16.hip", "gemm_direct_bf16.hip", "skinny_gemm_bf16.hip", "attention_bf16.hip", "rope_bf16.hip",
+    "tuned": ["gemm_bf16.hip", "gemm_wide_bf16.hip", "gemm_direct_bf16.hip", "skinny_gemm_bf16.hip", "attention_bf16.hip", "attention_wide_bf16.hip", "rope_bf16.hip",
               "probe.hip"],
 }
-HEADERS = ["common.h", "mfma.h", "gemm_wide.h", "gemm_direct.h", "no_alloc.h"]
+HEADERS = ["common.h", "mfma.h", "gemm_wide.h", "gemm_direct.h", "attention_wide.h", "no_alloc.h"]
 
 ARCH = "gfx950"
 # -packed-fp32-ops is switched off for device code: some packed forms have given wrong results on this hardware.
@@ -38,7 +38,7 @@ FLAGS = ["-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", f"--offload-arch={
          "-Wno-unused-result"]
 # Sources whose MFMA accumulators go into the accumulation registers (the compiler's default): a kernel there keeps 256
 # of them a wave, beside 256 vector registers for everything else.
-ACC_REGISTER_SOURCES = {"gemm_wide_bf16.hip", "gemm_direct_bf16.hip"}
+ACC_REGISTER_SOURCES = {"gemm_wide_bf16.hip", "gemm_direct_bf16.hip", "attention_wide_bf16.hip"}
 VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 
 

@@ -303,6 +303,9 @@ WHOLE_WAVES = 4   # waves of such a block (NW in attention_bf16.hip)
 # With fewer pairs: the blocks of a pair leave one partial result each and the one that finishes last adds them (no
 # second kernel), where the sizes allow; False: partial results per wave and a kernel that merges them.
 LAST_BLOCK_MERGES = True
+# Portions whose tiles of 128 rows are mostly whole (heads of 128, pages of a power of two from 16 on) run on the kernel
+# that takes such a tile a block (attention_wide_bf16.hip); False sends every portion to the kernels of 64-row blocks.
+WIDE_TILES = True
 _counters: dict = {}
 
 
@@ -356,7 +359,7 @@ def attention_bf16(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int,
             q.data_ptr(), ldq, q_off, out.data_ptr(), ldo, n_heads, n_kv_heads, head_dim, cache.data_ptr(),
             page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
             step.row_seg.data_ptr(), step.tile_row0.data_ptr(), step.tile_rows.data_ptr(), step.n_tiles,
-            int(window), sc, stream), "attention_prefill_bf16")
+            (T - step.n_decode_rows) if WIDE_TILES else 0, int(window), sc, stream), "attention_prefill_bf16")
     if step.n_decode_rows:
         n = step.n_decode_rows
         span = min(step.max_decode_context, window) if window else step.max_decode_context

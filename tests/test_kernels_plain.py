@@ -144,9 +144,10 @@ def test_silu_mul_and_add():
     close(f64(acc), want, atol=1e-6, rtol=1e-6)
 
 
-def make_cache(n_seq_tokens, Hk, d, P_, dtype, seed=0, shuffle=True, stale=0.0):
+def make_cache(n_seq_tokens, Hk, d, P_, dtype, seed=0, shuffle=True, stale=0.0, loud=None):
     """Random keys/values for sequences of the given lengths laid into pages in a shuffled order.  `stale`: what
-    the slots beyond a sequence's last position and the three pages that belong to no sequence hold."""
+    the slots beyond a sequence's last position and the three pages that belong to no sequence hold.  `loud`:
+    (sequence, position, factor): that key is multiplied by the factor, so that its scores dwarf all others."""
     rng = np.random.default_rng(seed)
     n_blocks = [-(-n // P_) for n in n_seq_tokens]
     total = sum(n_blocks)
@@ -158,6 +159,8 @@ def make_cache(n_seq_tokens, Hk, d, P_, dtype, seed=0, shuffle=True, stale=0.0):
     for s, n in enumerate(n_seq_tokens):
         k = gen(n, Hk, d, seed=seed * 100 + 2 * s, dtype=dtype)
         v = gen(n, Hk, d, seed=seed * 100 + 2 * s + 1, dtype=dtype)
+        if loud is not None and loud[0] == s:
+            k[loud[1]] = (k[loud[1]].float() * loud[2]).to(dtype)
         ks.append(k)
         vs.append(v)
         for b in range(n_blocks[s]):

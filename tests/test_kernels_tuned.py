@@ -437,13 +437,15 @@ def test_product_for_q_k_v_that_rotates_declines_what_it_does_not_take():
                                   torch.zeros(17, dtype=torch.int32, device=DEV), bt, cache2, P_)
 
 
-def run_attention(H, Hk, d, P_, lens, rows_per_seg, window=0, seed=0, stale=0.0):
+def run_attention(H, Hk, d, P_, lens, rows_per_seg, window=0, seed=0, stale=0.0, loud=None):
     """Sequences of `lens` keys in the cache; the last `rows_per_seg[s]` positions of sequence s are the step's rows.
     `stale`: what lies in the slots beyond a sequence's last key and in the spare page; with a window, the pages that
-    every row of the step has passed are marked as given back in the block table (the spare page stands in)."""
+    every row of the step has passed are marked as given back in the block table (the spare page stands in).
+    `loud`: (sequence, position, factor) of a key whose scores dwarf all others."""
     from allpaca_amd.engine.batch import Entry, pack_step
+    from allpaca_amd.kernels import ops as kernel_ops
     t = tuned()
-    cache, bt, ks, vs = make_cache(lens, Hk, d, P_, BF, seed=seed, stale=stale)
+    cache, bt, ks, vs = make_cache(lens, Hk, d, P_, BF, seed=seed, stale=stale, loud=loud)
     pos0 = [n - r for n, r in zip(lens, rows_per_seg)]
     entries = [Entry(i, [0] * r, []) for i, r in enumerate(rows_per_seg)]
     tables = [[list(bt[i, : -(-n // P_)].cpu().numpy()) for i, n in enumerate(lens)]]
@@ -453,7 +455,8 @@ def run_attention(H, Hk, d, P_, lens, rows_per_seg, window=0, seed=0, stale=0.0)
         for tb, p0 in zip(tables[0], pos0):
             for b in range(max(0, p0 - window + 1) // P_):
                 tb[b] = -1
-    step = pack_step(entries, pos0, [0] * len(lens), tables, torch.device(DEV), [spare])
+    step = pack_step(entries, pos0, [0] * len(lens), tables, torch.device(DEV), [spare],
+                     tile_rows=kernel_ops.attention_tile_rows(BF))
     T = sum(rows_per_seg)
     # queries scaled up: scores of deviation ~2.5, so a few keys carry each row and a wrong or missing one shows
     q = gen(T, H * d + 16, seed=seed + 7, scale=2.5, dtype=BF).to(DEV)
@@ -507,6 +510,33 @@ def test_attention_windows_with_large_heads(d, window, decode_path):
     # window that is no multiple of the key tile, pages in front of the window given back
     run_attention(H=4, Hk=2, d=d, P_=16, lens=[400, 230, 90], rows_per_seg=[1, 150, 70], window=window, seed=d)
     run_attention(H=2, Hk=1, d=d, P_=8, lens=[333, 77], rows_per_seg=[100, 1], window=window, seed=d + 1)
+
+
+@pytest.mark.parametrize("P_", [16, 32, 64, 128])
+def test_attention_of_whole_tiles_of_128_rows(P_):
+    """Heads of 128 in portions that fill tiles of 128 rows: the kernel that takes such a tile a block (keys and values
+    by direct loads into LDS, one page per 16 keys).  Several requests, history in front of a portion, rows and keys
+    that are no multiple of a tile, one and several key tiles, every page size it takes."""
+    run_attention(H=4, Hk=2, d=128, P_=P_, lens=[640, 300, 128], rows_per_seg=[384, 300, 128], seed=P_)
+    run_attention(H=8, Hk=8, d=128, P_=P_, lens=[1000, 257, 1], rows_per_seg=[250, 257, 1], seed=P_ + 1)
+    run_attention(H=2, Hk=1, d=128, P_=P_, lens=[2500], rows_per_seg=[2500 - 1277], seed=P_ + 2)
+
+
+@pytest.mark.parametrize("window", [1, 37, 128, 200, 1000])
+def test_attention_of_whole_tiles_with_windows(window):
+    # windows that end inside the first key tile, that span several, that are wider than the keys; pages in front of
+    # the window given back (the spare page, full of NaN, stands in); NaN beyond the last key
+    run_attention(H=4, Hk=2, d=128, P_=16, lens=[900, 260], rows_per_seg=[500, 260], window=window, seed=window,
+                  stale=float("nan"))
+    run_attention(H=2, Hk=2, d=128, P_=32, lens=[700], rows_per_seg=[300], window=window, seed=window + 1,
+                  stale=float("nan"))
+
+
+@pytest.mark.parametrize("where", [3, 200, 519, 700])
+def test_attention_of_whole_tiles_when_a_late_key_dwarfs_the_first(where):
+    """The kernel for tiles of 128 rows keeps a row's first reference for its exponents; a key whose scores lie far
+    beyond it (here by hundreds of powers of two) sends the block to its plain loop, whose references move."""
+    run_attention(H=4, Hk=2, d=128, P_=16, lens=[768], rows_per_seg=[512], seed=where, loud=(0, where, 40.0))
 
 
 @pytest.mark.parametrize("d", [16, 64, 128, 192, 256])
