@@ -45,6 +45,13 @@
 #include <math.h>
 #include <type_traits>
 
+// #define APC_WIDE_CLOCKS 1
+#ifdef APC_WIDE_CLOCKS
+__device__ unsigned long long apc_wide_clocks[16];
+#define CLK(n) asm volatile("s_memtime %0" : "=s"(clk_t[n]))
+#else
+#define CLK(n)
+#endif
 namespace {
 
 constexpr int KT = 64;                     // keys a tile
@@ -71,26 +78,27 @@ __device__ __forceinline__ Frag lds_frag(int addr) {
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
   return __builtin_bit_cast(Frag, v);
 }
-#define WAIT_LDS "s_waitcnt lgkmcnt(%3)\n\t"
+constexpr int NO_WAIT = -1;  // an operand that has been in registers for long
 // c = a . q and c += a . q with the result in vector registers and q, the wave's query rows, which only MFMAs read, in
 // accumulation registers (an MFMA takes its operands from either file); c += a . b with c in accumulation registers.
 template <int LGKM>
 __device__ __forceinline__ void mfma_set(floatx16& c, const Frag& a, const Frag& q) {
-  asm volatile(WAIT_LDS "v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0"
-               : "=&v"(c) : "v"(__builtin_bit_cast(u32x4, a)), "a"(__builtin_bit_cast(u32x4, q)), "n"(LGKM));
+  const u32x4 av = __builtin_bit_cast(u32x4, a), qv = __builtin_bit_cast(u32x4, q);
+  if constexpr (LGKM < 0) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(av), "a"(qv));
+  else asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(av), "a"(qv), "n"(LGKM));
 }
 template <int LGKM>
 __device__ __forceinline__ void mfma_add(floatx16& c, const Frag& a, const Frag& q) {
-  asm volatile(WAIT_LDS "v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0"
-               : "+v"(c) : "v"(__builtin_bit_cast(u32x4, a)), "a"(__builtin_bit_cast(u32x4, q)), "n"(LGKM));
+  const u32x4 av = __builtin_bit_cast(u32x4, a), qv = __builtin_bit_cast(u32x4, q);
+  if constexpr (LGKM < 0) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "a"(qv));
+  else asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "a"(qv), "n"(LGKM));
 }
 template <int LGKM>
 __device__ __forceinline__ void mfma_acc(floatx16& c, const Frag& a, const Frag& b) {
-  asm volatile(WAIT_LDS "v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0"
-               : "+a"(c) : "v"(__builtin_bit_cast(u32x4, a)), "v"(__builtin_bit_cast(u32x4, b)), "n"(LGKM));
+  const u32x4 av = __builtin_bit_cast(u32x4, a), bv = __builtin_bit_cast(u32x4, b);
+  if constexpr (LGKM < 0) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(av), "v"(bv));
+  else asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(av), "v"(bv), "n"(LGKM));
 }
-#undef WAIT_LDS
-constexpr int NO_WAIT = 15;  // the counter's largest value: an operand that has been in registers for long
 
 template <int N>
 __device__ __forceinline__ void wait_loads_but() {  // until at most N vector memory loads of this wave are in flight
@@ -107,11 +115,25 @@ __device__ __forceinline__ float halves_sum(float v) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 __device__ __forceinline__ float exp2_neg(float x) { return __builtin_amdgcn_exp2f(x); }
-// the instruction itself: fmaxf on values the compiler has not seen computed first makes each of them canonical
-__device__ __forceinline__ float max3(float a, float b, float c) {
+// The largest of 8 scores and m, as instructions: fmaxf on values the compiler has not seen computed first makes each
+// of them canonical (one more instruction each), and one statement keeps the compiler's guard against what an unknown
+// instruction may need (a wait state in front of every reader) to one place.
+__device__ __forceinline__ float max_of_8(float m, const floatx16& s, int r0) {
   float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  if (r0 == 0)
+    asm("v_max3_f32 %0, %1, %2, %3\n\tv_max3_f32 %0, %0, %4, %5\n\tv_max3_f32 %0, %0, %6, %7\n\tv_max3_f32 %0, %0, %8, %9"
+        : "=&v"(r) : "v"(m), "v"(s[0]), "v"(s[1]), "v"(s[2]), "v"(s[3]), "v"(s[4]), "v"(s[5]), "v"(s[6]), "v"(s[7]));
+  else
+    asm("v_max3_f32 %0, %1, %2, %3\n\tv_max3_f32 %0, %0, %4, %5\n\tv_max3_f32 %0, %0, %6, %7\n\tv_max3_f32 %0, %0, %8, %9"
+        : "=&v"(r) : "v"(m), "v"(s[8]), "v"(s[9]), "v"(s[10]), "v"(s[11]), "v"(s[12]), "v"(s[13]), "v"(s[14]), "v"(s[15]));
   return r;
+}
+// sum + the two bfloat16 values of `pair` (v_dot2c_f32_bf16 with a pair of ones): the row's sum is taken over P as the
+// value product sees it, two values an instruction
+__device__ __forceinline__ float add_pair(float sum, uint32_t pair) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  const bf16x2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pair), ones, sum, false);
 }
 
 // all but the positions lo <= p < hi of the 8 that a value piece holds are cleared
@@ -141,16 +163,15 @@ __device__ __forceinline__ void soft_step(int h, floatx16& s, Frag (&pf)[2], Sof
   if (h == 0 || h == 1) {
     const int r0 = h * 8;
     if (MASKED) {
+      // key tk + 8 lh + c with c = 16 (r / 8) + r % 8: seen if lo <= key <= pos, that is first <= c <= last
+      const int base = tk + 8 * lh, first = st.lo - base, last = st.pos - base;
 #pragma unroll
       for (int r = r0; r < r0 + 8; ++r) {
-        const int t = tk + 16 * (r / 8) + 8 * lh + r % 8;
-        s[r] = (t >= st.lo && t <= st.pos) ? s[r] : -INFINITY;
+        const int c = 16 * (r / 8) + r % 8;
+        s[r] = (c >= first && c <= last) ? s[r] : -INFINITY;
       }
     }
-    float mx = h == 0 ? max3(s[0], s[1], s[2]) : max3(st.mx, s[8], s[9]);
-    mx = max3(mx, s[r0 + 3], s[r0 + 4]);
-    mx = max3(mx, s[r0 + 5], s[r0 + 6]);
-    mx = h == 0 ? max3(mx, s[7], s[7]) : max3(mx, s[10], s[15]);
+    const float mx = max_of_8(h == 0 ? -INFINITY : st.mx, s, r0);
     st.mx = h == 0 ? mx : halves_max(mx) * sc2;
   }
   if (h == 2) {
@@ -161,14 +182,37 @@ __device__ __forceinline__ void soft_step(int h, floatx16& s, Frag (&pf)[2], Sof
   }
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
-    if (score_step(r) == h) {
-      // a row that has seen no key yet: m = -inf and every score is -inf; -inf - -inf would be NaN
-      s[r] = exp2_neg(fmaf(s[r], sc2, st.m == -INFINITY ? 0.f : -st.m));
-      st.sum += s[r];
+    // a row that has seen no key yet: m = -inf and every score is -inf; -inf - -inf would be NaN
+    if (score_step(r) == h) s[r] = exp2_neg(fmaf(s[r], sc2, st.m == -INFINITY ? 0.f : -st.m));
+    if ((r & 1) && score_step(r) + 1 == h) {
+      const uint32_t pair = pack_bf16x2(s[r - 1], s[r]);
+      pf[r / 8].w[(r % 8) / 2] = pair;
+      st.sum = add_pair(st.sum, pair);
     }
-    if ((r & 1) && score_step(r) + 1 == h) pf[r / 8].w[(r % 8) / 2] = pack_bf16x2(s[r - 1], s[r]);
   }
   if (h == 15) st.l += halves_sum(st.sum);
+}
+
+// The same for a tile all of whose keys every row sees, when every row has its reference: no masks and no maximum
+// (a P beyond float32 shows in the sum, which is checked when all is done).  One score a step; the sum runs on
+// over the tiles per lane, and the two halves of the wave add theirs when the loop of such passes ends.
+__device__ __forceinline__ void soft_step_seen(int h, floatx16& s, Frag (&pf)[2], Soft& st, float sc2) {
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    if (r == h) s[r] = exp2_neg(fmaf(s[r], sc2, -st.m));
+    // a pair is packed two steps behind its second value: an exponential's result wants a wait state before its reader
+    if ((r & 1) && (r + 2 == h || (r == 15 && h == 15) || (r == 13 && h == 15))) {
+      const uint32_t pair = pack_bf16x2(s[r - 1], s[r]);
+      pf[r / 8].w[(r % 8) / 2] = pair;
+      st.sum = add_pair(st.sum, pair);
+    }
+  }
+}
+enum { SOFT_MASKED = 0, SOFT_SEEN = 1 };
+template <int MODE>
+__device__ __forceinline__ void soft_any(int h, floatx16& s, Frag (&pf)[2], Soft& st, int tk, int lh, float sc2) {
+  if constexpr (MODE == SOFT_SEEN) soft_step_seen(h, s, pf, st, sc2);
+  else soft_step<true>(h, s, pf, st, tk, lh, sc2);
 }
 
 __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
@@ -250,30 +294,56 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
   // K: load i brings LDS rows 16 w + 4 i .. + 3 = keys 16 w + 4 sw(i) .. + 3, lane -> (row lane / 16, place lane % 16,
   // which holds piece place ^ row).  V^T: load i brings elements 32 i .. + 31 of the wave's 16 keys, lane -> (element
   // lane / 2, half lane % 2), into [group w][element][16 keys].
+  // The 4 loads of a tile's K (and of its V) differ by 1 KiB in LDS, which the instruction's offset field gives; that
+  // field counts for the address in memory too, so the lanes' offsets take it back (and 3 KiB more, which the base
+  // gives back, so that none is negative).
   int koff[4], voff[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int sw = 2 * (i & 1) + (i >> 1);
-    koff[i] = (4 * sw + lane / 16) * (d * 2) + (((lane % 16) ^ (lane / 16) ^ (4 * i)) * 16);
-    voff[i] = (32 * i + lane / 2) * (P * 2) + (lane % 2) * 16;
+    koff[i] = (4 * sw + lane / 16) * (d * 2) + (((lane % 16) ^ (lane / 16) ^ (4 * i)) * 16) + 3072 - i * 1024;
+    voff[i] = (32 * i + lane % 32) * (P * 2) + (lane / 32) * 16 + 3072 - i * 1024;
   }
   auto group_of = [&](int j) { return min(t_begin + j * KT + 16 * wave, last16); };  // first key of the wave's 16
   auto page_of = [&](int j) { return __builtin_amdgcn_readfirstlane(bt[group_of(j) >> lgP]); };
-  auto k_load = [&](int j, int page) {
-    const BufferRsrc kr = make_rsrc(k_head + (size_t)__builtin_amdgcn_readfirstlane(page) * page_stride);
+  const bf16_t* k_head_low = k_head - 1536;  // 3 KiB lower
+  const bf16_t* v_head_low = v_head - 1536;
+  // one of the 4 loads of a tile's K or V (to stand between other work)
+  auto k_load_piece = [&](int j, int page, int i) {
+    const BufferRsrc kr = make_rsrc(k_head_low + (size_t)__builtin_amdgcn_readfirstlane(page) * page_stride);
     const int soff = (group_of(j) & (P - 1)) * (d * 2);
-    unsigned char* dst = smem + (j % STG) * K_STAGE + (16 * wave) * 256;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, (lds_ptr)(dst + i * 1024), 16, koff[i], soff, 0, 0);
+    const lds_ptr dst = (lds_ptr)(smem + (j % STG) * K_STAGE + (16 * wave) * 256);
+    if (i == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[0], soff, 0, 0);
+    if (i == 1) __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[1], soff, 1024, 0);
+    if (i == 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[2], soff, 2048, 0);
+    if (i == 3) __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[3], soff, 3072, 0);
+  };
+  auto v_load_piece = [&](int j, int page, int i) {
+    const BufferRsrc vr = make_rsrc(v_head_low + (size_t)__builtin_amdgcn_readfirstlane(page) * page_stride);
+    const int soff = (group_of(j) & (P - 1)) * 2;
+    const lds_ptr dst = (lds_ptr)(smem + V_BASE + (j % STG) * V_STAGE + wave * 4096);
+    if (i == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[0], soff, 0, 0);
+    if (i == 1) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[1], soff, 1024, 0);
+    if (i == 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[2], soff, 2048, 0);
+    if (i == 3) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[3], soff, 3072, 0);
+  };
+  auto k_load = [&](int j, int page) {
+    const BufferRsrc kr = make_rsrc(k_head_low + (size_t)__builtin_amdgcn_readfirstlane(page) * page_stride);
+    const int soff = (group_of(j) & (P - 1)) * (d * 2);
+    const lds_ptr dst = (lds_ptr)(smem + (j % STG) * K_STAGE + (16 * wave) * 256);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[0], soff, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[1], soff, 1024, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[2], soff, 2048, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[3], soff, 3072, 0);
   };
   auto v_load = [&](int j, int page) {
-    const BufferRsrc vr = make_rsrc(v_head + (size_t)__builtin_amdgcn_readfirstlane(page) * page_stride);
+    const BufferRsrc vr = make_rsrc(v_head_low + (size_t)__builtin_amdgcn_readfirstlane(page) * page_stride);
     const int soff = (group_of(j) & (P - 1)) * 2;
-    unsigned char* dst = smem + V_BASE + (j % STG) * V_STAGE + wave * 4096;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, (lds_ptr)(dst + i * 1024), 16, voff[i], soff, 0, 0);
+    const lds_ptr dst = (lds_ptr)(smem + V_BASE + (j % STG) * V_STAGE + wave * 4096);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[0], soff, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[1], soff, 1024, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[2], soff, 2048, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[3], soff, 3072, 0);
   };
   // Stale positions of the V^T stage of tile j are cleared: what lies beyond the last key or in front of the first
   // one that a row of the block sees may be anything, and 0 x NaN is NaN.  (A group of 16 keys beyond the last one
@@ -281,8 +351,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
   auto clear_unseen = [&](int j) {
     const int t0 = t_begin + j * KT;
     unsigned char* stage = smem + V_BASE + (j % STG) * V_STAGE;
-    for (int idx = tid; idx < HD * 8; idx += 256) {  // piece idx: group idx / 256, element (idx % 256) / 2, half idx % 2
-      const int t16 = t0 + 16 * (idx / 256), tg = t16 + 8 * (idx % 2);
+    for (int idx = tid; idx < HD * 8; idx += 256) {  // piece idx: group idx / 256, half (idx % 64) / 32 of an element
+      const int t16 = t0 + 16 * (idx / 256), tg = t16 + 8 * ((idx % 64) / 32);
       Frag* piece = reinterpret_cast<Frag*>(stage + idx * 16);
       if (t16 > last16) {
         *piece = zero_frag();
@@ -305,8 +375,18 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
   int kaddr[d / 16];
 #pragma unroll
   for (int ks = 0; ks < d / 16; ++ks) kaddr[ks] = (kh * 32 + li) * 256 + ((((2 * ks) | lh) ^ (li % 16)) * 16);
-  const int vaddr = V_BASE + 2 * kh * 4096 + li * 32 + lh * 16;
+  const int vaddr = V_BASE + 2 * kh * 4096 + lane * 16;
   auto k_frag = [&](int stage_bytes, int ks) { return lds_frag<0>(lds0 + kaddr[ks] + stage_bytes); };
+  auto read_v_frags = [&](Frag (&vf)[8], int va) {
+    vf[0] = lds_frag<0>(va);
+    vf[1] = lds_frag<1024>(va);
+    vf[2] = lds_frag<2048>(va);
+    vf[3] = lds_frag<3072>(va);
+    vf[4] = lds_frag<4096>(va);
+    vf[5] = lds_frag<5120>(va);
+    vf[6] = lds_frag<6144>(va);
+    vf[7] = lds_frag<7168>(va);
+  };
   // the same through the compiler's own loads (the plain loop)
   auto k_frag_plain = [&](int stage_bytes, int ks) { return *reinterpret_cast<const Frag*>(smem + kaddr[ks] + stage_bytes); };
   auto v_frag_plain = [&](int stage_bytes, int g) {
@@ -367,7 +447,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     floatx16 s0, s1;     // raw scores of the two row tiles, then P
     Frag p0[2], p1[2];   // P as the second product's operands
 
-    // ---- prologue: K(0); then what the passes -3, -2, -1 of the loop would have issued
+    // ---- prologue.  Tile j's K fragments are read from LDS in slot B of pass j - 2 and its V fragments in slot B of
+    // pass j - 1 (see below); the direct loads of K(j) and V(j - 1) go out in the middle of pass j - 5.
     int kpg, vpg;  // pages of the wave's keys of the tiles whose K and V the next pass loads
     {
       const int pg0 = page_of(0), pg1 = page_of(1), pg2 = page_of(2), pg3 = page_of(3);
@@ -382,9 +463,14 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
       kpg = page_of(4);
     }
     __builtin_amdgcn_sched_barrier(0);
-    wait_loads_but<3 * LOADS_PER_TILE>();
+    wait_loads_but<2 * LOADS_PER_TILE>();  // K(0), K(1), V(0)
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
+    if (at_edge(0)) {
+      clear_unseen(0);
+      __syncthreads();
+    }
+    Frag kfr[8], vfr[8];  // the fragments of K(i + 1) and V(i) of this wave, in registers through a pass
     {  // S(0) of both row tiles and the softmax of row tile 0, one thing after the other
       Frag kf[d / 16];
 #pragma unroll
@@ -400,94 +486,156 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
         }
       }
       __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int g = 0; g < 8; ++g) kfr[g] = k_frag(K_STAGE, g);
+      read_v_frags(vfr, lds0 + vaddr);
       asm volatile("s_nop 15\n\ts_nop 15");  // the MFMAs have left the matrix cores: their results may be read
       __builtin_amdgcn_sched_barrier(0);
       const int tk = t_begin + kh * 32;
 #pragma unroll
       for (int hh = 0; hh < 16; ++hh) soft_step<true>(hh, s0, p0, st[0], tk, lh, sc2);
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave has read K(0)
+      __builtin_amdgcn_s_barrier();        // every wave has: its stage may be filled again
+      __builtin_amdgcn_sched_barrier(0);
+      k_load(4, kpg);
+      v_load(3, vpg);
+      vpg = kpg;
+      kpg = page_of(5);
     }
 
-    // ---- a pass of the loop.  Before pass i: S1(i) raw in s1, P0(i) in p0.  MASKED: some row may not see some key of
-    // tile i (row tile 1) or tile i + 1 (row tile 0), or tile i has stale positions.
-    auto pass = [&](auto MASKED_, int i) {
-      constexpr bool MASKED = decltype(MASKED_)::value;
+    // ---- a pass of the loop.  Before pass i: S1(i) raw in s1, P0(i) in p0, the fragments of K(i + 1) and V(i) in kfr
+    // and vfr (on their way from LDS).  MASKED: some row may not see some key of tile i (row tile 1) or tile i + 1 (row
+    // tile 0), or tile i + 1 has stale positions.
+#ifdef APC_WIDE_CLOCKS
+    const bool clk_on = blockIdx.x == 0 && tid == 0;
+    unsigned long long clk_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, clk_t[8], clk_prev = 0;
+#endif
+    auto pass = [&](auto MODE_, int i, int i_last) {  // i_last: the last pass of this kind in a row
+      constexpr int MODE = decltype(MODE_)::value;
+      constexpr bool MASKED = MODE == SOFT_MASKED;
       const int t0 = t_begin + i * KT;
-      const int stage_k = ((i + 1) % STG) * K_STAGE, stage_v = (i % STG) * V_STAGE;
       __builtin_amdgcn_sched_barrier(0);
-      wait_loads_but<2 * LOADS_PER_TILE>();      // K(i + 1) and V(i) are there ...
-      __builtin_amdgcn_s_barrier();              // ... for every wave, and every wave has left K(i) and V(i - 1)
-      __builtin_amdgcn_sched_barrier(0);
-      if constexpr (MASKED) {
-        if (at_edge(i)) {
-          clear_unseen(i);
-          __syncthreads();
-        }
-      }
-      k_load(i + 4, kpg);
-      v_load(i + 3, vpg);
-      vpg = kpg;
-      kpg = page_of(i + 5);
-      __builtin_amdgcn_sched_barrier(0);
-      Frag kfr[8], vfr[8];
-      {  // slot A.  LDS reads go out two steps ahead, K(i + 1) and V(i) in turn: when a step's MFMA wants its
-         // fragment, the four reads behind it may still be out (fewer in the last steps).
+      CLK(0);
+      {  // slot A: the fragments have been asked for half a pass ago
         const int tk = t0 + kh * 32;
-        const int va = lds0 + vaddr + stage_v;
-        kfr[0] = k_frag(stage_k, 0);
-        vfr[0] = lds_frag<0>(va);
-        kfr[1] = k_frag(stage_k, 1);
-        vfr[1] = lds_frag<1024>(va);
+        const int va = lds0 + vaddr + (i % STG) * V_STAGE;
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
-          constexpr int out_k[8] = {4, 4, 4, 4, 4, 4, 3, 1}, out_v[8] = {4, 4, 4, 4, 4, 4, 2, 0};
-          if (g + 2 < 8) kfr[g + 2] = k_frag(stage_k, g + 2);
-#define SLOT_A_STEP(G)                                                                      \
-  if (g == G) {                                                                             \
-    if (G == 0) mfma_set<out_k[G]>(s0, kfr[G], qf[0][G]);                                   \
-    else mfma_add<out_k[G]>(s0, kfr[G], qf[0][G]);                                          \
-    soft_step<MASKED>(2 * G, s1, p1, st[1], tk, lh, sc2);                                   \
-    __builtin_amdgcn_sched_barrier(0);                                                      \
-    if (G + 2 < 8) vfr[(G + 2) % 8] = lds_frag<((G + 2) % 8 / 4) * 4096 + ((G + 2) % 4) * 1024>(va); \
-    mfma_acc<out_v[G]>(o[0][G % 4], vfr[G], p0[G / 4]);                                     \
-    soft_step<MASKED>(2 * G + 1, s1, p1, st[1], tk, lh, sc2);                               \
-    __builtin_amdgcn_sched_barrier(0);                                                      \
+#define SLOT_A_STEP(G)  /* slot B asked for K0 V0 K1 V1 .. K7 in this order, and V7 follows here behind the first  \
+                           MFMA (whose going out tells that the last MFMA of slot B has read V7's registers):      \
+                           behind read n, 15 - n may still be out */                                               \
+  if (g == G) {                                                                                   \
+    if (G == 0) {                                                                                 \
+      mfma_set<14>(s0, kfr[G], qf[0][G]);                                                         \
+      vfr[7] = lds_frag<4096 + 3072>(va);                                                         \
+    } else {                                                                                      \
+      mfma_add<15 - 2 * G>(s0, kfr[G], qf[0][G]);                                                 \
+    }                                                                                             \
+    soft_any<MODE>(2 * G, s1, p1, st[1], tk, lh, sc2);                                            \
+    __builtin_amdgcn_sched_barrier(0);                                                            \
+    mfma_acc<14 - 2 * G>(o[0][G % 4], vfr[G], p0[G / 4]);                                         \
+    soft_any<MODE>(2 * G + 1, s1, p1, st[1], tk, lh, sc2);                                        \
+    __builtin_amdgcn_sched_barrier(0);                                                            \
   }
           SLOT_A_STEP(0) SLOT_A_STEP(1) SLOT_A_STEP(2) SLOT_A_STEP(3)
           SLOT_A_STEP(4) SLOT_A_STEP(5) SLOT_A_STEP(6) SLOT_A_STEP(7)
 #undef SLOT_A_STEP
         }
       }
-      {  // slot B: every fragment is in registers
-        const int tk = t0 + KT + kh * 32;
-#pragma unroll
-        for (int g = 0; g < 8; ++g) {
-          if (g == 0) mfma_set<NO_WAIT>(s1, kfr[g], qf[1][g]);
-          else mfma_add<NO_WAIT>(s1, kfr[g], qf[1][g]);
-          soft_step<MASKED>(2 * g, s0, p0, st[0], tk, lh, sc2);
-          __builtin_amdgcn_sched_barrier(0);
-          mfma_acc<NO_WAIT>(o[1][g % 4], vfr[g], p1[g / 4]);
-          soft_step<MASKED>(2 * g + 1, s0, p0, st[0], tk, lh, sc2);
-          __builtin_amdgcn_sched_barrier(0);
+      // The middle of the pass: K(i + 2) and V(i + 1), whose fragments slot B reads, are in LDS for every wave; every
+      // wave has read K(i + 1) and V(i) (in slot B of the pass before), so the direct loads of K(i + 5) and V(i + 4) may
+      // fill their stages.
+      CLK(1);
+      wait_loads_but<2 * LOADS_PER_TILE>();
+      CLK(2);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      CLK(3);
+      if constexpr (MASKED) {
+        if (at_edge(i + 1)) {
+          clear_unseen(i + 1);
+          __syncthreads();
         }
+      }
+      if constexpr (MASKED) {  // this kind of pass has no registers to spare for keeping the loads' operands through slot B
+        k_load(i + 5, kpg);
+        v_load(i + 4, vpg);
+        vpg = kpg;
+        kpg = page_of(i + 6);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      CLK(4);
+      {  // slot B; a fragment's registers take the next pass's fragment as soon as its MFMA has gone out
+        const int tk = t0 + KT + kh * 32;
+        const int stage_k = ((i + 2) % STG) * K_STAGE;
+        const int va = lds0 + vaddr + ((i + 1) % STG) * V_STAGE;
+#define SLOT_B_STEP(G)  /* a fragment's registers are free once the MFMA behind the one that read them has gone out; \
+                           the direct loads of K(i + 5) and V(i + 4) go out one a step */                          \
+  {                                                                                                 \
+    if (G == 0) mfma_set<NO_WAIT>(s1, kfr[G], qf[1][G]);                                            \
+    else mfma_add<NO_WAIT>(s1, kfr[G], qf[1][G]);                                                   \
+    if (G > 0) vfr[(G + 7) % 8] = lds_frag<(((G + 7) % 8) / 4) * 4096 + ((G + 7) % 4) * 1024>(va);  \
+    if (!MASKED && G < 4) k_load_piece(i + 5, kpg, G);                                              \
+    if (!MASKED && G >= 4) v_load_piece(i + 4, vpg, G - 4);                                         \
+    soft_any<MODE>(2 * G, s0, p0, st[0], tk, lh, sc2);                                              \
+    __builtin_amdgcn_sched_barrier(0);                                                              \
+    mfma_acc<NO_WAIT>(o[1][G % 4], vfr[G], p1[G / 4]);                                              \
+    kfr[G] = k_frag(stage_k, G);                                                                    \
+    if (!MASKED && G == 7) {                                                                        \
+      vpg = kpg;                                                                                    \
+      kpg = page_of(i + 6);                                                                         \
+    }                                                                                               \
+    soft_any<MODE>(2 * G + 1, s0, p0, st[0], tk, lh, sc2);                                          \
+    __builtin_amdgcn_sched_barrier(0);                                                              \
+  }
+        SLOT_B_STEP(0) SLOT_B_STEP(1) SLOT_B_STEP(2) SLOT_B_STEP(3)
+        SLOT_B_STEP(4) SLOT_B_STEP(5) SLOT_B_STEP(6) SLOT_B_STEP(7)
+#undef SLOT_B_STEP
       }
       // The last MFMAs must have left the matrix cores before O is read.  The compiler does not know these
       // instructions: it reads the accumulators right behind the loop, in front of any wait that stands there.
+      CLK(5);
+#ifdef APC_WIDE_CLOCKS
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(clk_t[0]), "+s"(clk_t[1]), "+s"(clk_t[2]), "+s"(clk_t[3]), "+s"(clk_t[4]), "+s"(clk_t[5]));
+      if (clk_prev) clk_acc[0] += clk_t[0] - clk_prev;
+      for (int c = 1; c < 6; ++c) clk_acc[c] += clk_t[c] - clk_t[c - 1];
+      clk_prev = clk_t[5];
+#endif
       if (i + 1 >= n_kt) asm volatile("s_nop 15\n\ts_nop 15");
+      __builtin_amdgcn_sched_barrier(0);
     };
-    // Passes in which every row sees every key run without the masks: with a window the first passes need them, under
-    // the causal mask the last ones.
-    auto needs_mask = [&](int i) {
-      return !sees_all(1, t_begin + i * KT) || !sees_all(0, t_begin + (i + 1) * KT) || at_edge(i);
+    // Passes in which every row sees every key of both tiles in work, and has seen a key before, run the short
+    // softmax; with a window the first passes are of the other kind, under the causal mask the last ones.
+    auto all_seen = [&](int i) {
+      return sees_all(1, t_begin + i * KT) && sees_all(0, t_begin + (i + 1) * KT) && !at_edge(i + 1);
     };
-    int i_open = 0;
-    while (i_open < n_kt && needs_mask(i_open)) ++i_open;
-    int i_close = i_open;
-    while (i_close < n_kt && !needs_mask(i_close)) ++i_close;
+    // Three loops one after the other, not one loop that chooses a kind of pass each time: the compiler then moved O
+    // between two sets of registers in every pass.
     int i = 0;
-    for (; i < i_open; ++i) pass(std::true_type{}, i);
-    for (; i < i_close; ++i) pass(std::false_type{}, i);
-    for (; i < n_kt; ++i) pass(std::true_type{}, i);
+    while (i < n_kt && !(all_seen(i) && __builtin_amdgcn_ballot_w64(st[0].m == -INFINITY || st[1].m == -INFINITY) == 0)) {
+      pass(std::integral_constant<int, SOFT_MASKED>{}, i, i);
+      ++i;
+    }
+    if (i < n_kt) {
+      int i_end = i + 1;
+      while (i_end < n_kt && all_seen(i_end)) ++i_end;
+      st[0].sum = st[1].sum = 0.f;
+      for (; i < i_end; ++i) pass(std::integral_constant<int, SOFT_SEEN>{}, i, i_end - 1);
+      st[0].l += halves_sum(st[0].sum);
+      st[1].l += halves_sum(st[1].sum);
+    }
+    for (; i < n_kt; ++i) pass(std::integral_constant<int, SOFT_MASKED>{}, i, i);
+    // a sum this large (or no number at all) means that some P was: such a block computes its rows again below
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) st[rt].beyond |= st[rt].l < 0x1p90f ? 0 : 1;
 
+#ifdef APC_WIDE_CLOCKS
+    if (clk_on) {
+      for (int c = 0; c < 8; ++c) apc_wide_clocks[c] = clk_acc[c];
+      apc_wide_clocks[8] = n_kt;
+    }
+#endif
     __builtin_amdgcn_sched_barrier(0);
     wait_loads_but<0>();                    // no direct load is on its way into LDS
     __builtin_amdgcn_sched_barrier(0);
@@ -572,6 +720,11 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
 
 }  // namespace
 
+#ifdef APC_WIDE_CLOCKS
+APC_EXPORT int apc_wide_clocks_read(unsigned long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(apc_wide_clocks), sizeof(unsigned long long) * 16);
+}
+#endif
 bool attn_wide_takes(int d, int page_tokens) {
   return d == ATTN_WIDE_HEAD && page_tokens >= 16 && (page_tokens & (page_tokens - 1)) == 0;
 }
