@@ -494,6 +494,17 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
       const int tk = t_begin + kh * 32;
 #pragma unroll
       for (int hh = 0; hh < 16; ++hh) soft_step<true>(hh, s0, p0, st[0], tk, lh, sc2);
+      {  // Row tile 1 takes its references from tile 0 now (its softmax of tile 0 comes in pass 0): with every row's
+         // reference there, the passes of the short kind can begin with pass 0.
+        const int base = tk + 8 * lh, first_c = st[1].lo - base, last_c = st[1].pos - base;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int c = 16 * (r / 8) + r % 8;
+          mx = fmaxf(mx, (c >= first_c && c <= last_c) ? s1[r] : -INFINITY);
+        }
+        st[1].m = halves_max(mx) * sc2;
+      }
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave has read K(0)
       __builtin_amdgcn_s_barrier();        // every wave has: its stage may be filled again
