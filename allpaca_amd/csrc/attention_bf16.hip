@@ -1,7 +1,8 @@
 // Attention over the paged cache in bfloat16 on MFMA, float32 softmax.
 //
-//   prefill kernels  a tile of up to 64 consecutive rows of one request x one head; keys in tiles of 64
-//                    through LDS; online softmax.  Head sizes up to 128: v_mfma_f32_32x32x16_bf16, a wave takes
+//   prefill kernels  a block takes up to 64 consecutive rows of one request x one head (half of a step's tile of up to
+//                    128 rows; tiles that are mostly whole, of heads of 128, go to attention_wide_bf16.hip, which
+//                    takes a whole tile a block); keys in tiles of 64 through LDS; online softmax.  Head sizes up to 128: v_mfma_f32_32x32x16_bf16, a wave takes
 //                    32 rows x half of each tile's keys (attn_prefill32_kernel; 98 us for 2,048 rows of 32 heads
 //                    of 128, 707 TFLOP/s at 32,768 rows).  Larger heads: v_mfma_f32_16x16x32_bf16, 16 rows a wave
 //                    (attn_prefill_kernel, which was 9 % slower at 128).
@@ -904,9 +905,10 @@ APC_EXPORT int apc_attention_prefill_bf16(const void* q, int ldq, int q_off, voi
   if (ldo % 4 || ((uintptr_t)out & 7u)) return APC_ERR_UNSUPPORTED;  // outputs are stored 8 bytes at a time
   if (max_blocks <= 0 || window < 0 || (long)n_tiles * H > 0x7fffffffL) return APC_ERR_BAD_ARG;
   if (!(scale > 0.f)) return APC_ERR_UNSUPPORTED;  // the kernel takes the maximum before it scales
-  // n_rows: the rows of all tiles together.  Tiles that are mostly whole go to the kernel that takes 128 rows a block;
-  // short ones (ends of prompts, many small requests) would leave half of its waves without rows.
-  if (attn_wide_takes(d, page_tokens) && (long)n_rows * 4 >= (long)n_tiles * TILE_ROWS * 3)
+  // n_rows: the rows of all tiles together.  Tiles of 64 rows and more on average go to the kernel that takes 128 rows a
+  // block; with many short ones (many small requests) half of its waves would have no rows (measured at 8B shapes: 17-32
+  // rows a tile 2-4 % slower than the 64-row kernel, 16 rows over 128 keys 36 %; 33-128 rows a tile 1.2-1.35 times as fast).
+  if (attn_wide_takes(d, page_tokens) && (long)n_rows * 2 >= (long)n_tiles * TILE_ROWS)
     return launch_attn_prefill_wide((const bf16_t*)q, ldq, q_off, (bf16_t*)out, ldo, H, Hk, (const bf16_t*)cache,
                                     page_tokens, block_table, max_blocks, positions, row_seg, tile_row0, tile_rows,
                                     n_tiles, window, scale, stream);

@@ -11,33 +11,44 @@
 // * An operand read from LDS feeds two MFMAs (the two row tiles of the wave) instead of one: one read per MFMA is
 //   all that LDS can deliver when the matrix cores run at their full rate.
 // * Keys and values go from global memory into LDS by direct loads (no registers, no LDS store instructions, no
-//   address arithmetic: a wave's 16 keys lie in one page, whose descriptors sit in scalar registers), four tiles
+//   address arithmetic: a wave's 16 keys lie in one page, whose descriptors sit in scalar registers), three passes
 //   ahead of their use in four stages.  K rows are not padded; a piece of 16 bytes lies at (piece index XOR row
 //   index) instead, which the direct load does by fetching the piece that belongs at its lane's place, and reads of
 //   16 lanes still fall into different banks.  The rows of a K tile are stored in the order in which the first
 //   product's result registers want them (bits 2 and 3 of the key index swapped), so that a lane's 8 results of a
 //   16-key step are 8 consecutive keys and the matching values are one 16-byte piece of V^T as a page holds it.
-//   V^T lies in LDS as the page holds it for 16 positions ([element of d][16 positions]): a wave's read of 32
-//   elements x 16 keys is 1 KiB in lane order.
-// * One wave a SIMD (O of 64 rows x 128 alone takes 128 accumulation registers), so nothing overlaps by itself: a
-//   pass of the loop is two slots of 16 MFMAs each, and the vector work of one row tile's softmax stands in the
-//   issue slots between the MFMAs of the other's products:
+//   V^T lies in LDS by groups of 16 keys, [half of the keys][element of d]: a wave's read of 32 elements x 16 keys is
+//   1 KiB in lane order.
+// * One wave a SIMD (O of 64 rows x 128 alone takes 128 accumulation registers, the query rows 64 more), so
+//   nothing overlaps by itself: a pass of the loop is two slots of 16 MFMAs each, and the vector work of one row
+//   tile's softmax stands in the issue slots between the MFMAs of the other's products:
 //     slot A: S0(i + 1) = K(i + 1) Q0 and O0 += V(i) P0(i), beside the softmax of S1(i)
 //     slot B: S1(i + 1) = K(i + 1) Q1 and O1 += V(i) P1(i), beside the softmax of S0(i + 1)
-//   (0, 1: the row tiles; i: the tile of keys).  The fragments of K(i + 1) and V(i) are read from LDS in slot A and
-//   stay in registers for slot B.  Exponentials (a quarter of the rate of other vector instructions) and MFMAs take
-//   about the same time per tile; this order is what lets both run.  Each result is written in one slot and read
-//   in the next, so nothing needs a second set of registers and the loop body has no branch.
+//   (0, 1: the row tiles; i: the tile of keys).  The fragments of K(i + 1) and V(i) stay in registers through both
+//   slots; slot B asks LDS for the next pass's fragments as soon as a fragment's registers are free (the MFMA behind
+//   the one that read them has gone out), half a pass before they are used, and issues the direct loads, one a step.
+//   The block's one barrier a pass stands between the slots.  Each result is written in one slot and read in the
+//   next, so nothing needs a second set of registers and the loop body has no branch.
 // * A row's reference for the exponents is the largest score among its first keys (the first tile of its wave that
 //   it sees a key of) and stays: O lives in accumulation registers that only MFMAs touch in the loop, so it cannot
-//   shrink there.  P = 2^(score - reference) may then exceed 1: up to 2^64 is let through (sums stay far inside
-//   float32).  If a row ever meets a score beyond that, the block throws its work away and computes its rows again
-//   in a plain loop (one thing after the other, references that move, as attn_prefill32_kernel does).
+//   shrink there.  P = 2^(score - reference) may then exceed 1; sums stay far inside float32 as long as no P goes
+//   beyond 2^64 (passes that look at the maximum) or the sum beyond 2^90 (checked at the end).  A block in which that
+//   happens throws its work away and computes its rows again in a plain loop (one thing after the other, references
+//   that move, as attn_prefill32_kernel does).
+// * Passes in which every row sees every key of both tiles in work, and has its reference, take a softmax without
+//   masks and without a maximum (16 x (fma, exp), 8 x (pack, add to the sum) a row tile); the others, a block's
+//   first and last few, take the general one.  The three kinds of passes are three loops one after the other.
 // The MFMAs are written as instructions: the compiler does not know them, so it neither waits for their results
 // nor keeps reads behind them; the order of the slots keeps every read of a result at least one MFMA behind the
-// one that wrote it, and the accumulators of O are read only after the loop, behind a wait.
+// one that wrote it, and a wait stands at the end of the last pass of each loop, behind which the compiler may read
+// the accumulators (to write the rows, or to move them where the next loop keeps them).
 // Positions outside a block's view that lie in stale slots are cleared in LDS before the value product sees them
 // (only tiles at the edge of a request's keys have any).
+// Tried and not kept: O in fixed registers so that instructions written out could shrink it (the compiler then moved O
+// to the vector registers and back in every pass); one loop that chooses the kind of pass each time (two copies of O,
+// one moved into the other every pass); the direct loads of K in slot A (the general passes ran out of registers,
+// and the compiler's moves of accumulators read MFMA results too early); K and V fragments read for this pass only,
+// two steps ahead (same speed: the wave waits for LDS either way, see the counters in profiles/).
 // Formula: crates/allpaca-cpu/src/kernels.rs:293-356.  Reference kernel (contiguous K/V, no matrix cores):
 // attention_qtile_kernel hip/src/kernels.cpp:2203.
 #include "attention_wide.h"
@@ -45,13 +56,6 @@
 #include <math.h>
 #include <type_traits>
 
-// #define APC_WIDE_CLOCKS 1
-#ifdef APC_WIDE_CLOCKS
-__device__ unsigned long long apc_wide_clocks[16];
-#define CLK(n) asm volatile("s_memtime %0" : "=s"(clk_t[n]))
-#else
-#define CLK(n)
-#endif
 namespace {
 
 constexpr int KT = 64;                     // keys a tile
@@ -518,16 +522,11 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     // ---- a pass of the loop.  Before pass i: S1(i) raw in s1, P0(i) in p0, the fragments of K(i + 1) and V(i) in kfr
     // and vfr (on their way from LDS).  MASKED: some row may not see some key of tile i (row tile 1) or tile i + 1 (row
     // tile 0), or tile i + 1 has stale positions.
-#ifdef APC_WIDE_CLOCKS
-    const bool clk_on = blockIdx.x == 0 && tid == 0;
-    unsigned long long clk_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, clk_t[8], clk_prev = 0;
-#endif
     auto pass = [&](auto MODE_, int i, int i_last) {  // i_last: the last pass of this kind in a row
       constexpr int MODE = decltype(MODE_)::value;
       constexpr bool MASKED = MODE == SOFT_MASKED;
       const int t0 = t_begin + i * KT;
       __builtin_amdgcn_sched_barrier(0);
-      CLK(0);
       {  // slot A: the fragments have been asked for half a pass ago
         const int tk = t0 + kh * 32;
         const int va = lds0 + vaddr + (i % STG) * V_STAGE;
@@ -557,12 +556,9 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
       // The middle of the pass: K(i + 2) and V(i + 1), whose fragments slot B reads, are in LDS for every wave; every
       // wave has read K(i + 1) and V(i) (in slot B of the pass before), so the direct loads of K(i + 5) and V(i + 4) may
       // fill their stages.
-      CLK(1);
       wait_loads_but<2 * LOADS_PER_TILE>();
-      CLK(2);
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
-      CLK(3);
       if constexpr (MASKED) {
         if (at_edge(i + 1)) {
           clear_unseen(i + 1);
@@ -576,7 +572,6 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
         kpg = page_of(i + 6);
         __builtin_amdgcn_sched_barrier(0);
       }
-      CLK(4);
       {  // slot B; a fragment's registers take the next pass's fragment as soon as its MFMA has gone out
         const int tk = t0 + KT + kh * 32;
         const int stage_k = ((i + 2) % STG) * K_STAGE;
@@ -606,13 +601,6 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
       }
       // The last MFMAs must have left the matrix cores before O is read.  The compiler does not know these
       // instructions: it reads the accumulators right behind the loop, in front of any wait that stands there.
-      CLK(5);
-#ifdef APC_WIDE_CLOCKS
-      asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(clk_t[0]), "+s"(clk_t[1]), "+s"(clk_t[2]), "+s"(clk_t[3]), "+s"(clk_t[4]), "+s"(clk_t[5]));
-      if (clk_prev) clk_acc[0] += clk_t[0] - clk_prev;
-      for (int c = 1; c < 6; ++c) clk_acc[c] += clk_t[c] - clk_t[c - 1];
-      clk_prev = clk_t[5];
-#endif
       if (i + 1 >= n_kt) asm volatile("s_nop 15\n\ts_nop 15");
       __builtin_amdgcn_sched_barrier(0);
     };
@@ -641,12 +629,6 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) st[rt].beyond |= st[rt].l < 0x1p90f ? 0 : 1;
 
-#ifdef APC_WIDE_CLOCKS
-    if (clk_on) {
-      for (int c = 0; c < 8; ++c) apc_wide_clocks[c] = clk_acc[c];
-      apc_wide_clocks[8] = n_kt;
-    }
-#endif
     __builtin_amdgcn_sched_barrier(0);
     wait_loads_but<0>();                    // no direct load is on its way into LDS
     __builtin_amdgcn_sched_barrier(0);
@@ -731,11 +713,6 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
 
 }  // namespace
 
-#ifdef APC_WIDE_CLOCKS
-APC_EXPORT int apc_wide_clocks_read(unsigned long long* out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(apc_wide_clocks), sizeof(unsigned long long) * 16);
-}
-#endif
 bool attn_wide_takes(int d, int page_tokens) {
   return d == ATTN_WIDE_HEAD && page_tokens >= 16 && (page_tokens & (page_tokens - 1)) == 0;
 }
