@@ -522,6 +522,15 @@ def test_attention_of_whole_tiles_of_128_rows(P_):
     run_attention(H=2, Hk=1, d=128, P_=P_, lens=[2500], rows_per_seg=[2500 - 1277], seed=P_ + 2)
 
 
+def test_attention_of_whole_tiles_at_the_head_counts_of_an_8b_model():
+    # 32 heads over 8 kv heads (heads of a kv head share an XCD in the kernel's order of blocks); portions that end in
+    # a short tile, that begin at position 0 and deep inside a sequence, and one of a single tile
+    run_attention(H=32, Hk=8, d=128, P_=16, lens=[700, 129, 4100, 128], rows_per_seg=[700, 129, 300, 70], seed=3)
+    # tiles of 64 rows on average: still the 128-row kernel; one row less on average: the 64-row kernels take over
+    run_attention(H=8, Hk=2, d=128, P_=16, lens=[300, 300, 500], rows_per_seg=[64, 64, 64], seed=4)
+    run_attention(H=8, Hk=2, d=128, P_=16, lens=[300, 300, 500], rows_per_seg=[64, 63, 64], seed=5)
+
+
 @pytest.mark.parametrize("window", [1, 37, 128, 200, 1000])
 def test_attention_of_whole_tiles_with_windows(window):
     # windows that end inside the first key tile, that span several, that are wider than the keys; pages in front of
