@@ -205,17 +205,33 @@ __device__ __forceinline__ void soft_step_seen(int h, floatx16& s, Frag (&pf)[2]
   for (int r = 0; r < 16; ++r) {
     if (r == h) s[r] = exp2_neg(fmaf(s[r], sc2, -st.m));
     // a pair is packed two steps behind its second value: an exponential's result wants a wait state before its reader
-    if ((r & 1) && (r + 2 == h || (r == 15 && h == 15) || (r == 13 && h == 15))) {
+    if ((r & 1) && (r + 2 == h || (r == 15 && h == 15))) {
       const uint32_t pair = pack_bf16x2(s[r - 1], s[r]);
       pf[r / 8].w[(r % 8) / 2] = pair;
       st.sum = add_pair(st.sum, pair);
     }
   }
 }
-enum { SOFT_MASKED = 0, SOFT_SEEN = 1 };
+// The same with masks, for rows that have their reference: what a block's last passes need (a row's first keys lie
+// in its first passes).  A key that the row does not see gets the exponent -inf.
+__device__ __forceinline__ void soft_step_late(int h, floatx16& s, Frag (&pf)[2], Soft& st, int tk, int lh, float sc2) {
+  const int base = tk + 8 * lh, first = st.lo - base, last = st.pos - base;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int c = 16 * (r / 8) + r % 8;
+    if (r == h) s[r] = exp2_neg((c >= first && c <= last) ? fmaf(s[r], sc2, -st.m) : -INFINITY);
+    if ((r & 1) && (r + 2 == h || (r == 15 && h == 15))) {
+      const uint32_t pair = pack_bf16x2(s[r - 1], s[r]);
+      pf[r / 8].w[(r % 8) / 2] = pair;
+      st.sum = add_pair(st.sum, pair);
+    }
+  }
+}
+enum { SOFT_MASKED = 0, SOFT_SEEN = 1, SOFT_LATE = 2 };
 template <int MODE>
 __device__ __forceinline__ void soft_any(int h, floatx16& s, Frag (&pf)[2], Soft& st, int tk, int lh, float sc2) {
   if constexpr (MODE == SOFT_SEEN) soft_step_seen(h, s, pf, st, sc2);
+  else if constexpr (MODE == SOFT_LATE) soft_step_late(h, s, pf, st, tk, lh, sc2);
   else soft_step<true>(h, s, pf, st, tk, lh, sc2);
 }
 
@@ -524,7 +540,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     // tile 0), or tile i + 1 has stale positions.
     auto pass = [&](auto MODE_, int i, int i_last) {  // i_last: the last pass of this kind in a row
       constexpr int MODE = decltype(MODE_)::value;
-      constexpr bool MASKED = MODE == SOFT_MASKED;
+      constexpr bool MASKED = MODE != SOFT_SEEN;  // tiles at an edge, and the loads in one place
       const int t0 = t_begin + i * KT;
       __builtin_amdgcn_sched_barrier(0);
       {  // slot A: the fragments have been asked for half a pass ago
@@ -624,7 +640,12 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
       st[0].l += halves_sum(st[0].sum);
       st[1].l += halves_sum(st[1].sum);
     }
-    for (; i < n_kt; ++i) pass(std::integral_constant<int, SOFT_MASKED>{}, i, i);
+    if (i < n_kt) {  // the rest: masks, but every row has its reference (the loop above began when all had)
+      st[0].sum = st[1].sum = 0.f;
+      for (; i < n_kt; ++i) pass(std::integral_constant<int, SOFT_LATE>{}, i, n_kt - 1);
+      st[0].l += halves_sum(st[0].sum);
+      st[1].l += halves_sum(st[1].sum);
+    }
     // a sum this large (or no number at all) means that some P was: such a block computes its rows again below
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) st[rt].beyond |= st[rt].l < 0x1p90f ? 0 : 1;
