@@ -36,8 +36,9 @@
 //   happens throws its work away and computes its rows again in a plain loop (one thing after the other, references
 //   that move, as attn_prefill32_kernel does).
 // * Passes in which every row sees every key of both tiles in work, and has its reference, take a softmax without
-//   masks and without a maximum (16 x (fma, exp), 8 x (pack, add to the sum) a row tile); the others, a block's
-//   first and last few, take the general one.  The three kinds of passes are three loops one after the other.
+//   masks and without a maximum (16 x (fma, exp), 8 x (pack, add to the sum) a row tile); a block's first passes
+//   (until every row has its reference) take the general one, and the last few, under the causal mask, one with
+//   masks but no maximum.  The three kinds of passes are three loops one after the other.
 // The MFMAs are written as instructions: the compiler does not know them, so it neither waits for their results
 // nor keeps reads behind them; the order of the slots keeps every read of a result at least one MFMA behind the
 // one that wrote it, and a wait stands at the end of the last pass of each loop, behind which the compiler may read

@@ -36,7 +36,8 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_paged_attention_plain": [P, I, I, I, P, I, I, I, I, I, I, P, I, I, P, I, P, P, I, F, P],
         "apc_argmax_rows": [P, I, I, I, P, P, P],
         "apc_argmax_rows_no_alloc": [P, I, I, I, P, P],
-        "apc_sample_rows": [P, I, I, I, P, P, P, P, P, P],
+        "apc_sample_rows": [P, I, I, I, P, P, P, P, P, P, Z, I, P],
+        "apc_sample_rows_scratch_kib": [I],
     },
     "tuned": {
         "apc_gemm_bf16": [P, I, P, P, I, I, I, I, I, P],
@@ -95,7 +96,7 @@ class KernelTimer:
 _timer = None
 # entry points that launch nothing (questions about sizes): never timed
 NOT_KERNELS = {"apc_attention_decode_whole_fits", "apc_attention_decode_last_fits", "apc_attention_prefill_tile_rows",
-               "apc_gemm_direct_k_split"}
+               "apc_gemm_direct_k_split", "apc_sample_rows_scratch_kib"}
 
 
 class timing:

@@ -234,7 +234,12 @@ def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> None:
 
 
 def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-                uniform: torch.Tensor, out: torch.Tensor) -> None:
+                uniform: torch.Tensor, out: torch.Tensor, any_top_k: bool = True, any_top_p: bool = True,
+                few_after_top_k: bool = False, one_block: bool = False) -> None:
+    """One token a row by temperature / top-k / top-p with the row's uniform number.  `any_top_k`, `any_top_p`: whether
+    some row may ask for that cut; `few_after_top_k`: every row that samples has 0 < top-k <= 1,024.  A caller that
+    knows its rows saves the launches that none of them needs; a row for which its word is wrong still gets its
+    token, slowly.  `one_block`: the kernel without working memory, one block a row."""
     _gpu(logits, temperature, top_k, top_p, uniform, out)
     ld = _rows(logits, "logits")
     R, V = logits.shape
@@ -243,8 +248,13 @@ def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Te
         if not (t.dtype == torch.float32 and t.is_contiguous() and t.numel() >= R):
             raise ValueError(f"{name}: float32 [{R}]")
     L = _lib.load("plain")
+    kib = 0 if one_block else L.apc_sample_rows_scratch_kib(R)
+    scratch = torch.empty(kib * 1024, dtype=torch.uint8, device=logits.device) if kib else None
     _lib.check(L.apc_sample_rows(logits.data_ptr(), ld, R, V, temperature.data_ptr(), _i32(top_k, R, "top_k"),
-                                 top_p.data_ptr(), uniform.data_ptr(), _i32(out, R, "sample out"), _stream()),
+                                 top_p.data_ptr(), uniform.data_ptr(), _i32(out, R, "sample out"),
+                                 scratch.data_ptr() if scratch is not None else 0, kib * 1024,
+                                 (1 if any_top_k else 0) | (2 if any_top_p else 0) | (4 if few_after_top_k else 0),
+                                 _stream()),
                "sample_rows")
 
 

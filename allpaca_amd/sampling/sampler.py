@@ -97,7 +97,10 @@ class Sampler:
             ops.argmax_rows(logits, out)
         else:
             f = self._upload(params, indices)
-            ops.sample_rows(logits, f[0, :R], f[3, :R].view(torch.int32), f[1, :R], f[2, :R], out)
+            ops.sample_rows(logits, f[0, :R], f[3, :R].view(torch.int32), f[1, :R], f[2, :R], out,
+                            any_top_k=any(p.top_k > 0 for p in params),
+                            any_top_p=any(0.0 <= p.top_p < 1.0 for p in params),
+                            few_after_top_k=all(p.greedy or 0 < p.top_k <= 1024 for p in params))
         if self._pinned[self._turn] is None or self._pinned[self._turn].numel() < R:
             self._pinned[self._turn] = torch.empty(max(R, 64), dtype=torch.int32).pin_memory()
         pinned = self._pinned[self._turn]

@@ -354,6 +354,60 @@ def kernel_times(cfg_json, args, layers):
     return out
 
 
+def sampler_times(vocab: int) -> dict:
+    """Microseconds to choose the tokens of 1, 8 and 64 rows of random logits under four rules.  `gpu_us`: the
+    kernels alone, their launches queued while the GPU is busy with something else (as a serving loop queues them
+    behind the step), so that no waiting for the host is in it; `latency_us`: `Sampler.sample` from call to token ids
+    on an idle GPU (parameters up, kernels, ids back)."""
+    import torch
+    from allpaca_amd.kernels import ops
+    from allpaca_amd.sampling import GenerationParams
+    from allpaca_amd.sampling.sampler import Sampler
+    dev = torch.device("cuda:0")
+    rules = {"greedy": dict(temperature=0.0, top_k=0, top_p=1.0),
+             "temperature": dict(temperature=0.8, top_k=0, top_p=1.0),
+             "top_k_40_top_p_0.95": dict(temperature=0.8, top_k=40, top_p=0.95),
+             "top_p_0.95": dict(temperature=0.8, top_k=0, top_p=0.95)}
+    busy = torch.randn(8192, 8192, device=dev)
+    sampler = Sampler(dev, 0)
+    out = {}
+    for rows in (1, 8, 64):
+        logits = torch.randn(rows, vocab, device=dev) * 3.0
+        ids = torch.empty(rows, dtype=torch.int32, device=dev)
+        u = torch.rand(rows, device=dev)
+        for name, rule in rules.items():
+            params = [GenerationParams(max_tokens=1, **rule) for _ in range(rows)]
+            t = torch.full((rows,), rule["temperature"], device=dev)
+            k = torch.full((rows,), rule["top_k"], dtype=torch.int32, device=dev)
+            p = torch.full((rows,), rule["top_p"], device=dev)
+
+            def kernels():
+                if name == "greedy":
+                    ops.argmax_rows(logits, ids)
+                else:
+                    ops.sample_rows(logits, t, k, p, u, ids, any_top_k=rule["top_k"] > 0, any_top_p=rule["top_p"] < 1.0,
+                                    few_after_top_k=0 < rule["top_k"] <= 1024)
+            calls = 20
+            for _ in range(3):
+                kernels()
+                sampler.sample(logits, params, [0] * rows)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            for _ in range(6):
+                busy @ busy                                   # a few milliseconds for the launches to queue behind
+            e0.record()
+            for _ in range(calls):
+                kernels()
+            e1.record()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(calls):
+                sampler.sample(logits, params, [i] * rows)
+            wall = time.perf_counter() - t0
+            out[f"b{rows}_{name}"] = {"gpu_us": round(e0.elapsed_time(e1) * 1e3 / calls, 1),
+                                      "latency_us": round(wall * 1e6 / calls, 1)}
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -382,9 +436,10 @@ def main() -> int:
                     help="with --only prefill: a prompt of this many tokens in steps of --portion tokens instead of the "
                          "2,048-token prompt in one step")
     ap.add_argument("--portion", type=int, default=2048)
-    ap.add_argument("--only", choices=["decode", "prefill"], default=None,
-                    help="for profiling: only the decode steps at --batch (as --no-points), or only the 2,048-token "
-                         "prefill (prints its figures as the line's value)")
+    ap.add_argument("--only", choices=["decode", "prefill", "sampler"], default=None,
+                    help="for profiling: only the decode steps at --batch (as --no-points), only the 2,048-token "
+                         "prefill (prints its figures as the line's value), or only the sampler over the preset's "
+                         "vocabulary (microseconds a step's rows take on the GPU and on the host)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
@@ -431,6 +486,11 @@ def main() -> int:
             "dtype": args.dtype, "data": "synthetic: random N(0, 0.02) weights, uniform random token ids",
             "config": {"model": args.preset, "layers": layers, "layers_of_configuration": full_layers,
                        "chunk_tokens": args.chunk, "max_batch_tokens": 2048, "page_tokens": 16}}), flush=True)
+        return 0
+    if args.only == "sampler":
+        print(json.dumps({"metric": "microseconds to choose a step's tokens (GPU time, launches queued behind other work)",
+                          "unit": "us", "n_gpus": 1, "config": {"model": args.preset, "vocab": cfg_json["vocab_size"]},
+                          "sampler": sampler_times(cfg_json["vocab_size"])}), flush=True)
         return 0
     if args.only == "decode":
         args.no_points = True

@@ -295,7 +295,8 @@ def test_argmax_rows():
     assert want[1] == 20 and want[2] == 0 and want[4] == 1002
 
 
-def test_sample_rows_against_plain_sampler():
+@pytest.mark.parametrize("one_block", [False, True], ids=["many blocks a row", "one block a row"])
+def test_sample_rows_against_plain_sampler(one_block):
     o = ops()
     rng = np.random.default_rng(0)
     for V in (50, 1003, 5000):
@@ -312,20 +313,70 @@ def test_sample_rows_against_plain_sampler():
         us[4] = 0.99999994
         out = torch.empty(R, dtype=torch.int32, device=DEV)
         o.sample_rows(lg.to(DEV), torch.from_numpy(temps).to(DEV), torch.from_numpy(ks).to(DEV),
-                      torch.from_numpy(ps).to(DEV), torch.from_numpy(us).to(DEV), out)
-        got = out.cpu().tolist()
-        lgn = lg.numpy()
-        mismatches = []
-        for r in range(R):
-            want = P.sample(lgn[r], float(temps[r]), int(ks[r]), float(ps[r]), float(us[r]))
-            if got[r] != want:
-                # a draw that lands within rounding of a boundary between two candidates may fall either way:
-                # accept the neighbour if the plain sampler gives it for a nudged r
-                near = {P.sample(lgn[r], float(temps[r]), int(ks[r]), float(ps[r]), float(us[r]) + e)
-                        for e in (-2e-6, 2e-6)}
-                if got[r] not in near:
-                    mismatches.append((r, got[r], want, float(temps[r]), int(ks[r]), float(ps[r]), float(us[r])))
+                      torch.from_numpy(ps).to(DEV), torch.from_numpy(us).to(DEV), out, one_block=one_block)
+        mismatches = _sample_mismatches(out.cpu().tolist(), lg.numpy(), temps, ks, ps, us)
         assert not mismatches, mismatches
+
+
+def _sample_mismatches(got, lgn, temps, ks, ps, us):
+    """Rows whose token is not the plain sampler's.  A draw that lands within rounding of a boundary between two
+    candidates may fall either way: the neighbour is accepted if the plain sampler gives it for a nudged r."""
+    mismatches = []
+    for r in range(len(got)):
+        a = (lgn[r], float(temps[r]), int(ks[r]), float(ps[r]))
+        want = P.sample(*a, float(us[r]))
+        if got[r] != want:
+            near = {P.sample(*a, float(us[r]) + e) for e in (-2e-6, 2e-6)}
+            if got[r] not in near:
+                mismatches.append((r, got[r], want) + a[1:] + (float(us[r]),))
+    return mismatches
+
+
+@pytest.mark.parametrize("values", ["halves", "64ths", "bfloat16", "all equal", "half of them -inf"])
+def test_sample_rows_among_equal_values(values):
+    """Many candidates with the same value: the k-th largest, the end of the top-p prefix and the drawn candidate
+    then fall inside a run of equal values, which the order breaks by id (crates/allpaca-core/src/sampling.rs:24-67:
+    a stable sort by value).  The kernels with many blocks a row carry the id in the sort key; each row must give the
+    plain sampler's token, the same token as one block a row, the same alone as in the batch, and the same when the
+    caller's word on which cuts its rows want is wrong (such rows go the slow way)."""
+    o = ops()
+    rng = np.random.default_rng(5)
+    for V, R in ((701, 9), (4099, 33), (20011, 12)):   # primes: no top-p of the list is a whole share of equal values
+        lg = gen(R, V, seed=V + 1) * 3.0
+        if values == "halves":
+            lg = torch.round(lg * 2) / 2
+        elif values == "64ths":
+            lg = torch.round(lg * 64) / 64
+        elif values == "bfloat16":
+            lg = lg.bfloat16().float()
+        elif values == "all equal":
+            lg[:] = 0.25
+        else:
+            lg[:, V // 2:] = float("-inf")
+        temps = rng.choice([0.3, 0.7, 1.0, 1.5], size=R).astype(np.float32)
+        # (no k of the list times a p of the list is a whole number either: with equal values a prefix that ends
+        # exactly on p would be decided by rounding)
+        ks = rng.choice([0, 1, 7, 41, 1001, 1023, 1025, 3001], size=R).astype(np.int32)
+        ps = rng.choice([1.0, 0.99, 0.95, 0.5, 0.1, 0.0, -1.0], size=R).astype(np.float32)
+        us = rng.random(R).astype(np.float32)
+        d = [torch.from_numpy(a).to(DEV) for a in (temps, ks, ps, us)]
+        lgd = lg.to(DEV)
+        outs = {}
+        for name, kw in (("many blocks", {}), ("one block", {"one_block": True}),
+                         ("no cut announced", {"any_top_k": False, "any_top_p": False}),
+                         ("few survivors announced", {"few_after_top_k": True}),
+                         ("top-k only announced", {"any_top_p": False})):
+            out = torch.empty(R, dtype=torch.int32, device=DEV)
+            o.sample_rows(lgd, *d, out, **kw)
+            outs[name] = out.cpu().tolist()
+        mismatches = _sample_mismatches(outs["many blocks"], lg.numpy(), temps, ks, ps, us)
+        assert not mismatches, (V, mismatches)
+        for name, got in outs.items():
+            assert got == outs["many blocks"], (V, name, got, outs["many blocks"])
+        alone = torch.empty(R, dtype=torch.int32, device=DEV)
+        for r in range(R):
+            o.sample_rows(lgd[r:r + 1], *(t[r:r + 1] for t in d), alone[r:r + 1])
+        assert alone.cpu().tolist() == outs["many blocks"], V
 
 
 def test_sample_rows_frequencies():

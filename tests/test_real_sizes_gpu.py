@@ -92,7 +92,8 @@ def test_products_with_a_vocabulary_of_output_columns(K):
     assert torch.equal(alone[0], tog[5])
 
 
-def test_sampler_over_a_real_vocabulary():
+@pytest.mark.parametrize("one_block", [False, True], ids=["many blocks a row", "one block a row"])
+def test_sampler_over_a_real_vocabulary(one_block):
     """temperature / top-k / top-p over 128,256 logits against the plain sampler (crates/allpaca-core/src/
     sampling.rs:24-67, 215-331)."""
     o = ops()
@@ -110,7 +111,7 @@ def test_sampler_over_a_real_vocabulary():
     us[8] = 0.99999994
     out = torch.empty(R, dtype=torch.int32, device=DEV)
     o.sample_rows(lg.to(DEV), torch.from_numpy(temps).to(DEV), torch.from_numpy(ks).to(DEV),
-                  torch.from_numpy(ps).to(DEV), torch.from_numpy(us).to(DEV), out)
+                  torch.from_numpy(ps).to(DEV), torch.from_numpy(us).to(DEV), out, one_block=one_block)
     got = out.cpu().tolist()
     lgn = lg.numpy()
     bad = []
