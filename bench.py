@@ -190,7 +190,7 @@ def ids_hash(token_lists):
     return h.hexdigest()[:16]
 
 
-def requests_run(eng, cfg, n_requests, min_prompt, max_prompt, new_tokens, seed=0):
+def requests_run(eng, cfg, n_requests, min_prompt, max_prompt, new_tokens, seed=0, sampled=False):
     """`n_requests` requests with prompts of random length arrive at once and run to `new_tokens` tokens each
     through the scheduler: portions of prompts beside decoding rows.  Returns a dict of totals and mean times."""
     import numpy as np
@@ -199,7 +199,8 @@ def requests_run(eng, cfg, n_requests, min_prompt, max_prompt, new_tokens, seed=
     from allpaca_amd.sampling import GenerationParams
     rng = np.random.default_rng(seed)
     lengths = [int(x) for x in rng.integers(min_prompt, max_prompt + 1, size=n_requests)]
-    gp = GenerationParams(max_tokens=new_tokens, temperature=0.0)
+    # greedy, or the defaults of the request options (temperature 0.8, top-k 40, top-p 0.95)
+    gp = GenerationParams(max_tokens=new_tokens) if sampled else GenerationParams(max_tokens=new_tokens, temperature=0.0)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     ids = [eng.add_request(rng.integers(0, cfg.vocab_size, size=n).tolist(), gp) for n in lengths]
@@ -429,6 +430,8 @@ def main() -> int:
     ap.add_argument("--max-prompt", type=int, default=4096)
     ap.add_argument("--new-tokens", type=int, default=256)
     ap.add_argument("--chunk", type=int, default=512, help="largest portion of a prompt in a step (with --requests)")
+    ap.add_argument("--sampled", action="store_true",
+                    help="with --requests: tokens drawn with temperature 0.8, top-k 40, top-p 0.95 instead of greedy")
     ap.add_argument("--kernel-times", action="store_true",
                     help="instead of the measured steps: event timers around every kernel of a decode step, a mixed step "
                          "and a 2,048-token prefill (eager passes of their own), and the host's time to launch a mixed step")
@@ -471,10 +474,11 @@ def main() -> int:
         captured = eng.warm_up()                                                                    # decode graphs
         requests_run(eng, cfg, min(n, 4), args.min_prompt, min(args.max_prompt, 512), 8, seed=1)   # first launches
         warm = time.perf_counter() - t0
-        r = requests_run(eng, cfg, n, args.min_prompt, args.max_prompt, args.new_tokens)
+        r = requests_run(eng, cfg, n, args.min_prompt, args.max_prompt, args.new_tokens, sampled=args.sampled)
         print(json.dumps({
             "metric": f"output tok/s, {n} requests at once, prompts {args.min_prompt}-{args.max_prompt}, "
-                      f"{args.new_tokens} new tokens each, chunked prefill",
+                      f"{args.new_tokens} new tokens each, chunked prefill"
+                      + (", sampled (temperature 0.8, top-k 40, top-p 0.95)" if args.sampled else ""),
             "value": round(r["output_tokens"] / r["seconds"], 1), "unit": "tok/s", "n_gpus": 1,
             "seconds": round(r["seconds"], 3), "steps": r["steps"], "prompt_tokens": r["prompt_tokens"],
             "output_tokens": r["output_tokens"], "all_tokens_per_s": round((r["prompt_tokens"] + r["output_tokens"]) / r["seconds"], 1),
