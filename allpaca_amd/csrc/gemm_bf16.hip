@@ -296,6 +296,9 @@ static int launch_gemm(const bf16_t* A, int lda, const bf16_t* W, const bf16_t* 
   if constexpr (!PRE) {
     // many rows, K a multiple of 128: the kernel that keeps the weights out of LDS (same sums, bit for bit)
     if (gemm_direct_takes(MODE, A, lda, C, ldc, M, N, K)) return launch_gemm_direct(MODE, A, lda, W, W2, C, ldc, M, N, K, stream);
+  } else if constexpr (MODE == G_SWIGLU) {
+    if (gemm_direct_swiglu_pre_takes(A, lda, C, ldc, M, N, K, pre.parts))
+      return launch_gemm_direct_swiglu_pre(A, lda, pre.ss, pre.parts, pre.eps, W, W2, C, ldc, M, N, K, stream);
   }
   if constexpr (MODE == G_SWIGLU) {
     // From 1,024 rows on the tile of 256 rows x 128 outputs takes as many columns as make whole rounds of one tile a

@@ -27,7 +27,15 @@
 
 namespace {
 
-enum { D_STORE_BF16 = 0, D_STORE_F32 = 1, D_ACC_F32 = 2, D_SWIGLU = 3 };
+enum { D_STORE_BF16 = 0, D_STORE_F32 = 1, D_ACC_F32 = 2, D_SWIGLU = 3, D_SWIGLU_PRE = 4 };
+__host__ __device__ constexpr bool is_swiglu(int mode) { return mode == D_SWIGLU || mode == D_SWIGLU_PRE; }
+
+// the sums of squares of rows that a product into the residual left for the RMS norm (D_SWIGLU_PRE)
+struct DirectPre {
+  const float* ss;
+  int parts;
+  float eps;
+};
 
 constexpr int R = 4;           // ring slots of W fragments: loads run R - 1 steps of 32 columns ahead
 constexpr int S = 4;           // LDS stages of A, 64 columns each
@@ -70,7 +78,7 @@ __host__ __device__ constexpr int loads_behind_a() {
 template <int BMG, int NF, int MODE>
 __device__ __forceinline__ void direct_tile(int bid, const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
                                             const bf16_t* __restrict__ W2, int chunks, void* __restrict__ C, int ldc,
-                                            int M, int N, int K) {
+                                            int M, int N, int K, DirectPre pre = DirectPre{}) {
   static_assert(R % 2 == 0, "ring slots are static over two stages");
   constexpr int NP = BMG / 2;  // direct loads of A a wave and stage (BMG * 2 fragments over 4 waves)
   constexpr int G = 2 * BMG;   // groups of NF MFMAs a stage: (chunk of 32 columns, row group)
@@ -81,7 +89,7 @@ __device__ __forceinline__ void direct_tile(int bid, const bf16_t* __restrict__ 
   static_assert(NVM < 64, "the counter has 6 bits");
   __shared__ __attribute__((aligned(1024))) unsigned char As[S][BMG * 2][1024];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
-  constexpr int NOUT = MODE == D_SWIGLU ? NF / 2 : NF;  // bands of outputs a wave writes
+  constexpr int NOUT = is_swiglu(MODE) ? NF / 2 : NF;  // bands of outputs a wave writes
   constexpr int NB = 4 * NOUT * 16;                     // outputs of a block
   int mt, nt;
   {
@@ -106,7 +114,7 @@ __device__ __forceinline__ void direct_tile(int bid, const bf16_t* __restrict__ 
   const int base_band = min(band0, bands - 1);
   const BufferRsrc abuf = make_rsrc(A + (size_t)m0 * lda);
   const BufferRsrc wbuf = make_rsrc(W + (size_t)base_band * chunks * 512);
-  const BufferRsrc ubuf = make_rsrc((MODE == D_SWIGLU ? W2 : W) + (size_t)base_band * chunks * 512);
+  const BufferRsrc ubuf = make_rsrc((is_swiglu(MODE) ? W2 : W) + (size_t)base_band * chunks * 512);
   int woff[NF];  // SwiGLU: NOUT gate bands, then the same bands of up
 #pragma unroll
   for (int f = 0; f < NF; ++f) woff[f] = (min(band0 + f % NOUT, bands - 1) - base_band) * chunks * 1024 + lane * 16;
@@ -128,7 +136,7 @@ __device__ __forceinline__ void direct_tile(int bid, const bf16_t* __restrict__ 
   };
   Frag ring[R][NF];
   auto w_piece = [&](int slot, int q, int f) {  // band f of step q (32 columns)
-    ring[slot][f] = load_frag_buffer((MODE == D_SWIGLU && f >= NOUT) ? ubuf : wbuf, woff[f],
+    ring[slot][f] = load_frag_buffer((is_swiglu(MODE) && f >= NOUT) ? ubuf : wbuf, woff[f],
                                      min(q, 2 * ktiles - 1) * 1024);
   };
   // stages 0..S-2 of A and steps 0..LEAD-1 of W
@@ -188,6 +196,27 @@ __device__ __forceinline__ void direct_tile(int bid, const bf16_t* __restrict__ 
 
   // D[i][j]: i = output (lane / 16) * 4 + r within the band, j = row lane % 16 within the row group
   const int mi = lane % 16, nq = lane / 16;
+  float row_scale[BMG];
+  if constexpr (MODE == D_SWIGLU_PRE) {
+    // 1 / sqrt(mean of x^2 + eps) of the block's rows, a thread a row, through the LDS that the stages have left
+    float* scales = reinterpret_cast<float*>(&As[0][0][0]);
+    __syncthreads();
+    if (tid < BMG * 16) {
+      const float* row = pre.ss + (size_t)min(m0 + tid, M - 1) * pre.parts;
+      float sum = 0.f;
+      for (int p0 = 0; p0 < pre.parts; p0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = p0 + j < pre.parts ? row[p0 + j] : 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) sum += v[j];
+      }
+      scales[tid] = 1.0f / sqrtf(sum / (float)K + pre.eps);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int a = 0; a < BMG; ++a) row_scale[a] = scales[a * 16 + mi];
+  }
 #pragma unroll
   for (int a = 0; a < BMG; ++a) {
     const int m = m0 + a * 16 + mi;
@@ -216,7 +245,9 @@ __device__ __forceinline__ void direct_tile(int bid, const bf16_t* __restrict__ 
           float v[4];
 #pragma unroll
           for (int r = 0; r < 4; ++r)
-            v[r] = MODE == D_STORE_BF16 ? acc[a][f][r] : silu_f(acc[a][f][r]) * acc[a][NOUT + f][r];
+            v[r] = MODE == D_STORE_BF16  ? acc[a][f][r]
+                   : MODE == D_SWIGLU ? silu_f(acc[a][f][r]) * acc[a][NOUT + f][r]
+                                      : silu_f(acc[a][f][r] * row_scale[a]) * (acc[a][NOUT + f][r] * row_scale[a]);
           uint2 o;
           o.x = pack_bf16x2(v[0], v[1]);
           o.y = pack_bf16x2(v[2], v[3]);
@@ -231,8 +262,9 @@ template <int NF, int MODE>
 __global__ __launch_bounds__(256, 1) void gemm_direct_kernel(const bf16_t* __restrict__ A, int lda,
                                                              const bf16_t* __restrict__ W,
                                                              const bf16_t* __restrict__ W2, int chunks,
-                                                             void* __restrict__ C, int ldc, int M, int N, int K) {
-  direct_tile<8, NF, MODE>(blockIdx.x, A, lda, W, W2, chunks, C, ldc, M, N, K);
+                                                             void* __restrict__ C, int ldc, int M, int N, int K,
+                                                             DirectPre pre) {
+  direct_tile<8, NF, MODE>(blockIdx.x, A, lda, W, W2, chunks, C, ldc, M, N, K, pre);
 }
 
 // K in `gridDim.y` slices of k_slice columns: slice s leaves its float32 sums in partials[s][M][N] (the tiled product's
@@ -272,26 +304,26 @@ int pick_bands(int M, int N, bool swiglu, int k_split = 1, double* cost_out = nu
 
 template <int NF, int MODE>
 int launch(const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M, int N, int K,
-           hipStream_t stream) {
-  constexpr int NB = 4 * (MODE == D_SWIGLU ? NF / 2 : NF) * 16;
+           hipStream_t stream, DirectPre pre) {
+  constexpr int NB = 4 * (is_swiglu(MODE) ? NF / 2 : NF) * 16;
   const long blocks = 8L * ceil_div((long)ceil_div(N, NB) * ceil_div(M, 128), 8L);
   if (blocks > 0x7fffffffL) return APC_ERR_BAD_ARG;
   hipLaunchKernelGGL((gemm_direct_kernel<NF, MODE>), dim3((unsigned)blocks), dim3(256), 0, stream, A, lda, W, W2,
-                     ceil_div(K, 32), C, ldc, M, N, K);
+                     ceil_div(K, 32), C, ldc, M, N, K, pre);
   APC_LAUNCH_CHECK();
   return 0;
 }
 
 template <int MODE>
 int launch_mode(int nf, const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M, int N,
-                int K, hipStream_t stream) {
-  if constexpr (MODE != D_SWIGLU) {
-    if (nf == 3) return launch<3, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream);
-    if (nf == 5) return launch<5, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream);
+                int K, hipStream_t stream, DirectPre pre) {
+  if constexpr (!is_swiglu(MODE)) {
+    if (nf == 3) return launch<3, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream, pre);
+    if (nf == 5) return launch<5, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream, pre);
   }
-  if (nf == 4) return launch<4, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream);
-  if (nf == 6) return launch<6, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream);
-  return launch<8, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream);
+  if (nf == 4) return launch<4, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream, pre);
+  if (nf == 6) return launch<6, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream, pre);
+  return launch<8, MODE>(A, lda, W, W2, C, ldc, M, N, K, stream, pre);
 }
 
 }  // namespace
@@ -334,30 +366,29 @@ int launch_gemm_direct_slices(const bf16_t* A, int lda, const bf16_t* W, float* 
   return 0;
 }
 
-bool gemm_direct_takes(int mode, const void* A, int lda, const void* C, int ldc, int M, int N, int K) {
-  if (mode < 0 || mode > D_SWIGLU || M < GEMM_DIRECT_MIN_ROWS || K < 128 || K % 128 || N % 4 || ldc % 4) return false;
+namespace {
+bool direct_takes(int mode, int min_rows, const void* A, int lda, const void* C, int ldc, int M, int N, int K) {
+  if (mode < 0 || mode > D_SWIGLU_PRE || M < min_rows || K < 128 || K % 128 || N % 4 || ldc % 4) return false;
   if (((uintptr_t)A & 15u) || ((uintptr_t)C & 15u) || lda % 8) return false;
   // the lanes' byte offsets into the block's rows of A and the wave's bands of W are 32-bit
   if ((long)128 * lda * 2 >= 0x7fffffffL || (long)8 * ceil_div(K, 32) * 1024 >= 0x7fffffffL) return false;
   return true;
 }
 
-namespace {
 int launch_columns(int nf, int mode, const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M,
-                   int N, int K, hipStream_t stream) {
+                   int N, int K, hipStream_t stream, DirectPre pre) {
   switch (mode) {
-    case D_STORE_BF16: return launch_mode<D_STORE_BF16>(nf, A, lda, W, W2, C, ldc, M, N, K, stream);
-    case D_STORE_F32: return launch_mode<D_STORE_F32>(nf, A, lda, W, W2, C, ldc, M, N, K, stream);
-    case D_ACC_F32: return launch_mode<D_ACC_F32>(nf, A, lda, W, W2, C, ldc, M, N, K, stream);
-    default: return launch_mode<D_SWIGLU>(nf, A, lda, W, W2, C, ldc, M, N, K, stream);
+    case D_STORE_BF16: return launch_mode<D_STORE_BF16>(nf, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
+    case D_STORE_F32: return launch_mode<D_STORE_F32>(nf, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
+    case D_ACC_F32: return launch_mode<D_ACC_F32>(nf, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
+    case D_SWIGLU: return launch_mode<D_SWIGLU>(nf, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
+    default: return launch_mode<D_SWIGLU_PRE>(nf, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
   }
 }
-}  // namespace
 
-int launch_gemm_direct(int mode, const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M,
-                       int N, int K, hipStream_t stream) {
-  if (!gemm_direct_takes(mode, A, lda, C, ldc, M, N, K) || (mode == D_SWIGLU) != (W2 != nullptr)) return APC_ERR_UNSUPPORTED;
-  const bool swiglu = mode == D_SWIGLU;
+int launch_direct(int mode, const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M, int N,
+                  int K, hipStream_t stream, DirectPre pre) {
+  const bool swiglu = is_swiglu(mode);
   double whole = 0.0;
   const int nf = pick_bands(M, N, swiglu, 1, &whole);
   // A launch whose last round is far from full (2,048 rows x 14,336 SwiGLU outputs: 3.5 rounds of tiles with 8 bands a
@@ -378,11 +409,32 @@ int launch_gemm_direct(int mode, const bf16_t* A, int lda, const bf16_t* W, cons
       if (cost < 0.97 * best) best = cost, best_nf = f, best_cols = big_cols * nb, rest_nf = rf;
     }
   }
-  if (!best_nf) return launch_columns(nf, mode, A, lda, W, W2, C, ldc, M, N, K, stream);
-  const int e = launch_columns(best_nf, mode, A, lda, W, W2, C, ldc, M, best_cols, K, stream);
+  if (!best_nf) return launch_columns(nf, mode, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
+  const int e = launch_columns(best_nf, mode, A, lda, W, W2, C, ldc, M, best_cols, K, stream, pre);
   if (e) return e;
   const size_t w_skip = (size_t)(best_cols / 16) * ceil_div(K, 32) * 512;  // whole bands of the tiled layout
   const size_t elem = (mode == D_STORE_BF16 || swiglu) ? 2 : 4;
   return launch_columns(rest_nf, mode, A, lda, W + w_skip, swiglu ? W2 + w_skip : W2, (char*)C + (size_t)best_cols * elem,
-                        ldc, M, N - best_cols, K, stream);
+                        ldc, M, N - best_cols, K, stream, pre);
+}
+}  // namespace
+
+bool gemm_direct_takes(int mode, const void* A, int lda, const void* C, int ldc, int M, int N, int K) {
+  return mode <= D_SWIGLU && direct_takes(mode, GEMM_DIRECT_MIN_ROWS, A, lda, C, ldc, M, N, K);
+}
+
+int launch_gemm_direct(int mode, const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M,
+                       int N, int K, hipStream_t stream) {
+  if (!gemm_direct_takes(mode, A, lda, C, ldc, M, N, K) || (mode == D_SWIGLU) != (W2 != nullptr)) return APC_ERR_UNSUPPORTED;
+  return launch_direct(mode, A, lda, W, W2, C, ldc, M, N, K, stream, DirectPre{});
+}
+
+bool gemm_direct_swiglu_pre_takes(const void* A, int lda, const void* C, int ldc, int M, int N, int K, int ss_parts) {
+  return ss_parts > 0 && direct_takes(D_SWIGLU_PRE, GEMM_DIRECT_PRE_MIN_ROWS, A, lda, C, ldc, M, N, K);
+}
+
+int launch_gemm_direct_swiglu_pre(const bf16_t* A, int lda, const float* ss, int ss_parts, float eps, const bf16_t* W,
+                                  const bf16_t* W2, void* C, int ldc, int M, int N, int K, hipStream_t stream) {
+  if (!ss || !W2 || !gemm_direct_swiglu_pre_takes(A, lda, C, ldc, M, N, K, ss_parts)) return APC_ERR_UNSUPPORTED;
+  return launch_direct(D_SWIGLU_PRE, A, lda, W, W2, C, ldc, M, N, K, stream, DirectPre{ss, ss_parts, eps});
 }

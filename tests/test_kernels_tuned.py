@@ -241,12 +241,16 @@ def test_product_into_the_residual_leaves_the_next_norms_row_with_more_than_16_r
                                    # K in one piece (enough tiles without slices): 224 and 192 tiles; a last row tile of 44
                                    (64, 28672, 520), (300, 8192, 264), (300, 2048, 1288),
                                    # SwiGLU on the 256-row tile with the norm's scale in its epilogue
-                                   (1024, 2 * 16640, 128)])
+                                   (1024, 2 * 16640, 128),
+                                   # SwiGLU from 384 rows on: the kernel that loads its weights straight into registers,
+                                   # the norm's scale in its epilogue (a last row tile of 116, of 128 and of 0 rows)
+                                   (500, 2 * 1200, 384), (384, 2 * 264, 128), (640, 2 * 2056, 256)])
 def test_product_of_the_normalised_row_from_what_was_left_with_17_to_1024_rows(M, N, K):
     """On the tiled kernel, with K in slices (the finishing kernel scales) or whole (the product's epilogue does)."""
     t = tuned()
     whole = t._tiled_k_split(M, N, K) == 1
-    assert whole == ((M, N, K) in [(64, 28672, 520), (300, 8192, 264), (1024, 2 * 16640, 128)])
+    assert whole == ((M, N, K) in [(64, 28672, 520), (300, 8192, 264), (1024, 2 * 16640, 128), (500, 2 * 1200, 384),
+                                   (384, 2 * 264, 128), (640, 2 * 2056, 256)])
     x = f64(gen(M, K, seed=1, scale=3.0))
     x[0, : K // 2] *= 40.0
     g = f64(1 + 0.2 * gen(K, seed=2))
