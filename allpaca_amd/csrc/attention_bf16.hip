@@ -898,7 +898,7 @@ APC_EXPORT int apc_attention_prefill_bf16(const void* q, int ldq, int q_off, voi
                                           const void* cache, int page_tokens, const int* block_table, int max_blocks,
                                           const int* positions, const int* row_seg, const int* tile_row0,
                                           const int* tile_rows, int n_tiles, int n_rows, int window, float scale,
-                                          hipStream_t stream) {
+                                          int n_splits, int part_rows, float* parts, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   int e = check_common(q, ldq, q_off, cache, H, Hk, d, page_tokens);
   if (e) return e;
@@ -911,7 +911,7 @@ APC_EXPORT int apc_attention_prefill_bf16(const void* q, int ldq, int q_off, voi
   if (attn_wide_takes(d, page_tokens) && (long)n_rows * 2 >= (long)n_tiles * TILE_ROWS)
     return launch_attn_prefill_wide((const bf16_t*)q, ldq, q_off, (bf16_t*)out, ldo, H, Hk, (const bf16_t*)cache,
                                     page_tokens, block_table, max_blocks, positions, row_seg, tile_row0, tile_rows,
-                                    n_tiles, window, scale, stream);
+                                    n_tiles, window, scale, n_splits < 1 ? 1 : n_splits, part_rows, parts, stream);
   n_tiles *= 2;  // halves
   if ((long)n_tiles * H > 0x7fffffffL) return APC_ERR_BAD_ARG;
   dim3 grid(n_tiles * H), block(256);

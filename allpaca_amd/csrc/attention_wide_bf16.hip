@@ -45,6 +45,10 @@
 // the accumulators (to write the rows, or to move them where the next loop keeps them).
 // Positions outside a block's view that lie in stale slots are cleared in LDS before the value product sees them
 // (only tiles at the edge of a request's keys have any).
+// A step of few tiles (a chunk of 512 prompt tokens is 4 tiles x 32 heads = 128 blocks for 256 compute units) may have
+// the keys of every tile cut into ranges of whole key tiles, a block each: a block then leaves its rows as float32
+// with their reference and sum, and attn_wide_merge_kernel adds the ranges (512 rows over 32,768 keys: 449 -> 288 us;
+// 128 rows: 424 -> 109 us; at 2,048 keys nothing is gained, the caller cuts from 4,096 keys on).
 // Tried and not kept: O in fixed registers so that instructions written out could shrink it (the compiler then moved O
 // to the vector registers and back in every pass); one loop that chooses the kind of pass each time (two copies of O,
 // one moved into the other every pass); the direct loads of K in slot A (the general passes ran out of registers,
@@ -240,7 +244,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     const bf16_t* __restrict__ q, int ldq, int q_off, bf16_t* __restrict__ out, int ldo, int H, int Hk,
     const bf16_t* __restrict__ cache, int lgP, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ positions, const int* __restrict__ row_seg, const int* __restrict__ tile_row0,
-    const int* __restrict__ tile_rows, int n_tiles, int window, float scale) {
+    const int* __restrict__ tile_rows, int n_tiles, int window, float scale, int n_splits, int part_rows,
+    float* __restrict__ parts) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   constexpr int d = HD;
   constexpr int DT = d / 32;
@@ -248,28 +253,49 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
   const int tid = threadIdx.x, lane = tid % WAVE, wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
   const int li = lane % 32, lh = lane / 32;
   const int rh = wave / 2, kh = wave % 2;  // half of the rows, half of each tile's keys
-  int tile, h;
+  int tile, h, split;
   {
     // heads of one kv head go to one XCD (their keys and values then lie in one L2), long tiles first
     const int id = blockIdx.x, G = H / Hk;
     if (Hk % 8 == 0) {
-      const int xcd = id % 8, slot = id / 8;
+      const int xcd = id % 8;
+      int slot = id / 8;
+      split = slot % n_splits;
+      slot /= n_splits;
       const int lhd = slot / n_tiles;
       tile = n_tiles - 1 - slot % n_tiles;
       h = (xcd + 8 * (lhd / G)) * G + lhd % G;
     } else {
-      tile = n_tiles - 1 - id % n_tiles;
-      h = id / n_tiles;
+      split = id % n_splits;
+      tile = n_tiles - 1 - (id / n_splits) % n_tiles;
+      h = id / n_splits / n_tiles;
     }
   }
   const int row0 = tile_row0[tile], nrows = tile_rows[tile];
   const int kvh = h / (H / Hk);
   const int pos0 = positions[row0];
   const int* bt = block_table + (size_t)row_seg[row0] * max_blocks;
-  const int last = pos0 + nrows - 1;
   const int first = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
   const size_t page_stride = (size_t)2 * Hk * P * d;
-  const int t_begin = (first / KT) * KT;
+  // The keys of the block: those its rows see, or with the tile's keys cut into n_splits ranges of whole key tiles,
+  // one of them: `last` is then the range's last key, the rows see nothing beyond it, and what the block leaves is a
+  // partial result that attn_wide_merge_kernel adds to the other ranges'.
+  int t_begin = (first / KT) * KT;
+  int last = pos0 + nrows - 1;
+  if (n_splits > 1) {
+    const int per = ceil_div((last - t_begin) / KT + 1, n_splits);
+    t_begin += split * per * KT;
+    last = min(last, t_begin + per * KT - 1);
+  }
+  float* part_o = parts ? parts + ((size_t)split * part_rows * H + h) * d : nullptr;           // + row * H * d
+  float* part_ml = parts ? parts + (size_t)n_splits * part_rows * H * d + ((size_t)split * part_rows * H + h) * 2 : nullptr;
+  if (t_begin > last) {  // more ranges than key tiles: nothing here
+    if (part_ml && tid < nrows) {
+      part_ml[(size_t)(row0 + tid) * H * 2] = -INFINITY;
+      part_ml[(size_t)(row0 + tid) * H * 2 + 1] = 0.f;
+    }
+    return;
+  }
   const int n_kt = (last - t_begin) / KT + 1;
   const int last16 = (last / 16) * 16;
   const bf16_t* k_head = cache + (size_t)kvh * P * d;
@@ -291,8 +317,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
       st[rt].l = 0.f;
       st[rt].mx = st[rt].sum = 0.f;
       st[rt].beyond = 0;
-      st[rt].pos = pos0 + my_row;
-      st[rt].lo = (window > 0 && st[rt].pos - window + 1 > 0) ? st[rt].pos - window + 1 : 0;
+      st[rt].pos = min(pos0 + my_row, last);
+      st[rt].lo = (window > 0 && pos0 + my_row - window + 1 > 0) ? pos0 + my_row - window + 1 : 0;
     }
     // from here on the values live in accumulation registers (left to the compiler, they are copied there in every pass)
 #pragma unroll
@@ -305,7 +331,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
   }
   // whether every row of row tile rt sees all of the wave's 32 keys of the tile that starts at t0
   auto sees_all = [&](int rt, int t0) {
-    const int tk = t0 + kh * 32, low = pos0 + rh * 64 + rt * 32, top = low + 31;
+    const int tk = t0 + kh * 32, low = min(pos0 + rh * 64 + rt * 32, last), top = pos0 + rh * 64 + rt * 32 + 31;
     const int win_lo = (window > 0 && top - window + 1 > 0) ? top - window + 1 : 0;
     return tk + 31 <= low && tk >= win_lo;
   };
@@ -436,7 +462,29 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     const float m = fmaxf(m1, m2);
     const float m_safe = m == -INFINITY ? 0.f : m;
     const float a1 = exp2_neg(m1 - m_safe), a2 = exp2_neg(m2 - m_safe);
-    const float inv = 1.0f / (l1 * a1 + l2 * a2);
+    const float l = l1 * a1 + l2 * a2;
+    if (part_o) {  // the row over this range of keys, as a float32 row with its reference and sum
+      if (lh == 0) {
+        part_ml[(size_t)(row0 + my_row) * H * 2] = l > 0.f ? m : -INFINITY;
+        part_ml[(size_t)(row0 + my_row) * H * 2 + 1] = l;
+      }
+      if (!(l > 0.f)) return;  // the row sees no key of the range
+      const float inv = 1.0f / l;
+      float* prow = part_o + (size_t)(row0 + my_row) * H * d;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          floatx4 y;
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            y[r] = (o[dt][g * 4 + r] * a1 + meet_o[(((rh * 2 + rt) * DT + dt) * 16 + g * 4 + r) * 64 + lane] * a2) * inv;
+          *reinterpret_cast<floatx4*>(prow + dt * 32 + g * 8 + lh * 4) = y;
+        }
+      }
+      return;
+    }
+    const float inv = 1.0f / l;
     bf16_t* orow = out + (size_t)(row0 + my_row) * ldo + (size_t)h * d;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
@@ -733,6 +781,40 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
   }
 }
 
+// The ranges of keys of a row added up: out = sum_s w_s O_s / sum_s w_s with w_s = l_s 2^(m_s - max m).  A block
+// takes a row of a tile, a thread four elements of a head at a time.
+__global__ __launch_bounds__(256) void attn_wide_merge_kernel(const float* __restrict__ parts, int n_splits, int part_rows,
+                                                              int H, const int* __restrict__ tile_row0,
+                                                              const int* __restrict__ tile_rows, bf16_t* __restrict__ out,
+                                                              int ldo) {
+  constexpr int d = HD;
+  const int tile = blockIdx.x / ATTN_WIDE_ROWS, r = blockIdx.x % ATTN_WIDE_ROWS;
+  if (r >= tile_rows[tile]) return;
+  const int row = tile_row0[tile] + r;
+  const float* part_ml = parts + (size_t)n_splits * part_rows * H * d;
+  const size_t plane = (size_t)part_rows * H;
+  for (int hq = threadIdx.x; hq < H * (d / 4); hq += 256) {
+    const int h = hq / (d / 4), e = (hq % (d / 4)) * 4;
+    const size_t at = (size_t)row * H + h;
+    float m = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) m = fmaxf(m, part_ml[(s * plane + at) * 2]);
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    float sum = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      const float ms = part_ml[(s * plane + at) * 2];
+      if (ms == -INFINITY) continue;
+      const float w = part_ml[(s * plane + at) * 2 + 1] * exp2_neg(ms - m);
+      acc += w * *reinterpret_cast<const floatx4*>(parts + (s * plane + at) * d + e);
+      sum += w;
+    }
+    const float inv = sum > 0.f ? 1.0f / sum : 0.f;
+    uint2 pk;
+    pk.x = pack_bf16x2(acc[0] * inv, acc[1] * inv);
+    pk.y = pack_bf16x2(acc[2] * inv, acc[3] * inv);
+    *reinterpret_cast<uint2*>(out + (size_t)row * ldo + (size_t)h * d + e) = pk;
+  }
+}
+
 }  // namespace
 
 bool attn_wide_takes(int d, int page_tokens) {
@@ -742,8 +824,12 @@ bool attn_wide_takes(int d, int page_tokens) {
 int launch_attn_prefill_wide(const bf16_t* q, int ldq, int q_off, bf16_t* out, int ldo, int H, int Hk,
                              const bf16_t* cache, int page_tokens, const int* block_table, int max_blocks,
                              const int* positions, const int* row_seg, const int* tile_row0, const int* tile_rows,
-                             int n_tiles, int window, float scale, hipStream_t stream) {
+                             int n_tiles, int window, float scale, int n_splits, int part_rows, float* parts,
+                             hipStream_t stream) {
   if (!attn_wide_takes(ATTN_WIDE_HEAD, page_tokens)) return APC_ERR_UNSUPPORTED;
+  if (n_splits < 1 || (n_splits > 1 && (!parts || part_rows <= 0)) || (long)n_tiles * H * n_splits > 0x7fffffffL)
+    return APC_ERR_BAD_ARG;
+  if (n_splits == 1) parts = nullptr;
   int lgP = 0;
   while ((1 << lgP) < page_tokens) ++lgP;
   static bool configured[64] = {};
@@ -756,9 +842,14 @@ int launch_attn_prefill_wide(const bf16_t* q, int ldq, int q_off, bf16_t* out, i
     if (e != hipSuccess) return (int)e;
     configured[dev] = true;
   }
-  hipLaunchKernelGGL(attn_prefill_wide_kernel, dim3(n_tiles * H), dim3(256), LDS_BYTES + 16, stream, q, ldq, q_off, out, ldo,
-                     H, Hk, cache, lgP, block_table, max_blocks, positions, row_seg, tile_row0, tile_rows, n_tiles,
-                     window, scale);
+  hipLaunchKernelGGL(attn_prefill_wide_kernel, dim3(n_tiles * H * n_splits), dim3(256), LDS_BYTES + 16, stream, q, ldq,
+                     q_off, out, ldo, H, Hk, cache, lgP, block_table, max_blocks, positions, row_seg, tile_row0, tile_rows,
+                     n_tiles, window, scale, n_splits, part_rows, parts);
   APC_LAUNCH_CHECK();
+  if (n_splits > 1) {
+    hipLaunchKernelGGL(attn_wide_merge_kernel, dim3(n_tiles * ATTN_WIDE_ROWS), dim3(256), 0, stream, parts, n_splits,
+                       part_rows, H, tile_row0, tile_rows, out, ldo);
+    APC_LAUNCH_CHECK();
+  }
   return 0;
 }

@@ -55,7 +55,7 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_gemm_direct_k_split": [I, I, I],
         "apc_skinny_gemm_bf16": [P, I, P, P, I, I, I, I, I, P],
         "apc_skinny_swiglu_bf16": [P, I, P, P, P, I, I, I, I, P],
-        "apc_attention_prefill_bf16": [P, I, I, P, I, I, I, I, P, I, P, I, P, P, P, P, I, I, I, F, P],
+        "apc_attention_prefill_bf16": [P, I, I, P, I, I, I, I, P, I, P, I, P, P, P, P, I, I, I, F, I, I, P, P],
         "apc_attention_decode_bf16": [P, I, I, P, I, I, I, I, I, P, I, P, I, P, P, P, I, F, I, I, P, P, P],
         "apc_attention_decode_last_fits": [I, I, I, I],
         "apc_attention_decode_whole_fits": [I, I, I],

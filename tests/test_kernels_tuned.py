@@ -441,8 +441,9 @@ def test_product_for_q_k_v_that_rotates_declines_what_it_does_not_take():
                                   torch.zeros(17, dtype=torch.int32, device=DEV), bt, cache2, P_)
 
 
-def run_attention(H, Hk, d, P_, lens, rows_per_seg, window=0, seed=0, stale=0.0, loud=None):
+def run_attention(H, Hk, d, P_, lens, rows_per_seg, window=0, seed=0, stale=0.0, loud=None, ranges=None):
     """Sequences of `lens` keys in the cache; the last `rows_per_seg[s]` positions of sequence s are the step's rows.
+    `ranges`: into how many ranges the kernel for tiles of 128 rows is expected to cut the keys of this step.
     `stale`: what lies in the slots beyond a sequence's last key and in the spare page; with a window, the pages that
     every row of the step has passed are marked as given back in the block table (the spare page stands in).
     `loud`: (sequence, position, factor) of a key whose scores dwarf all others."""
@@ -462,6 +463,8 @@ def run_attention(H, Hk, d, P_, lens, rows_per_seg, window=0, seed=0, stale=0.0,
     step = pack_step(entries, pos0, [0] * len(lens), tables, torch.device(DEV), [spare],
                      tile_rows=kernel_ops.attention_tile_rows(BF))
     T = sum(rows_per_seg)
+    if ranges is not None:
+        assert t._key_splits(step, H, window) == ranges
     # queries scaled up: scores of deviation ~2.5, so a few keys carry each row and a wrong or missing one shows
     q = gen(T, H * d + 16, seed=seed + 7, scale=2.5, dtype=BF).to(DEV)
     out = torch.zeros(T, H * d, dtype=BF, device=DEV)
@@ -550,6 +553,34 @@ def test_attention_of_whole_tiles_when_a_late_key_dwarfs_the_first(where):
     """The kernel for tiles of 128 rows keeps a row's first reference for its exponents; a key whose scores lie far
     beyond it (here by hundreds of powers of two) sends the block to its plain loop, whose references move."""
     run_attention(H=4, Hk=2, d=128, P_=16, lens=[768], rows_per_seg=[512], seed=where, loud=(0, where, 40.0))
+
+
+@pytest.mark.parametrize("range_min", [64, 192, 512])
+def test_attention_of_whole_tiles_with_the_keys_cut_into_ranges(monkeypatch, range_min):
+    """A step of few tiles over many keys: the keys of every tile are cut into ranges, a block each, and a second
+    kernel adds the ranges.  With the smallest range set low so that modest sizes are cut: requests whose tiles have
+    very different numbers of keys (some fewer key tiles than ranges: empty ranges), NaN beyond the last key, windows
+    (rows that see no key of a range), a key that dwarfs the others in the first and in a later range, 8 ranges."""
+    nan = float("nan")
+    monkeypatch.setattr(tuned(), "KEY_RANGE_MIN", range_min)
+    n = lambda keys, blocks: max(1, min(8, 256 // blocks, keys // range_min))
+    run_attention(H=4, Hk=2, d=128, P_=16, lens=[1500, 200, 128], rows_per_seg=[300, 200, 100], seed=range_min, stale=nan,
+                  ranges=n(1500, 6 * 4))
+    run_attention(H=2, Hk=1, d=128, P_=32, lens=[2500], rows_per_seg=[130], seed=range_min + 1, ranges=n(2500, 2 * 2))
+    run_attention(H=4, Hk=2, d=128, P_=16, lens=[1900, 700], rows_per_seg=[250, 128], window=700, seed=range_min + 2,
+                  stale=nan, ranges=n(828, 3 * 4))
+    run_attention(H=4, Hk=2, d=128, P_=16, lens=[1900], rows_per_seg=[128], window=150, seed=range_min + 3, stale=nan,
+                  ranges=n(278, 4))
+    for where in (3, 1100, 1499):
+        run_attention(H=4, Hk=2, d=128, P_=16, lens=[1500], rows_per_seg=[256], seed=range_min + where,
+                      loud=(0, where, 40.0), ranges=n(1500, 2 * 4))
+
+
+def test_attention_of_whole_tiles_with_the_keys_cut_into_ranges_at_the_size_from_which_it_is_done():
+    # 2,048 keys a range: 4,500 keys in 2 ranges, 17,000 in 8
+    run_attention(H=4, Hk=2, d=128, P_=16, lens=[4500], rows_per_seg=[100], seed=1, ranges=2)
+    run_attention(H=2, Hk=1, d=128, P_=64, lens=[17000], rows_per_seg=[129], seed=2, ranges=8)
+    run_attention(H=4, Hk=2, d=128, P_=16, lens=[4000], rows_per_seg=[100], seed=3, ranges=1)
 
 
 @pytest.mark.parametrize("d", [16, 64, 128, 192, 256])
