@@ -98,15 +98,17 @@ def decode_during_prefill(batch, context, chunk=2048):
     return batch * -(-context // chunk) + batch
 
 
-def decode_run(eng, cfg, batch, context, steps, warmup):
-    """Fills `batch` requests to `context` tokens, then times `steps` decode steps."""
+def decode_run(eng, cfg, batch, context, steps, warmup, sampled=False):
+    """Fills `batch` requests to `context` tokens, then times `steps` decode steps (greedy, or with `sampled` the
+    request options' defaults: temperature 0.8, top-k 40, top-p 0.95)."""
     import numpy as np
     import torch
 
     from allpaca_amd.sampling import GenerationParams
     rng = np.random.default_rng(0)
     # requests that finish their prompt first decode while the others still prefill: leave room for that
-    gp = GenerationParams(max_tokens=warmup + steps + decode_during_prefill(batch, context) + 8, temperature=0.0)
+    gp = GenerationParams(max_tokens=warmup + steps + decode_during_prefill(batch, context) + 8,
+                          **({} if sampled else {"temperature": 0.0}))
     for _ in range(batch):
         eng.add_request(rng.integers(0, cfg.vocab_size, size=context - 1).tolist(), gp)
     while any(not r.decoding for r in eng.scheduler.running) or eng.scheduler.waiting:
@@ -431,7 +433,8 @@ def main() -> int:
     ap.add_argument("--new-tokens", type=int, default=256)
     ap.add_argument("--chunk", type=int, default=512, help="largest portion of a prompt in a step (with --requests)")
     ap.add_argument("--sampled", action="store_true",
-                    help="with --requests: tokens drawn with temperature 0.8, top-k 40, top-p 0.95 instead of greedy")
+                    help="tokens drawn with temperature 0.8, top-k 40, top-p 0.95 instead of greedy (the decode steps, or "
+                         "with --requests the requests)")
     ap.add_argument("--kernel-times", action="store_true",
                     help="instead of the measured steps: event timers around every kernel of a decode step, a mixed step "
                          "and a 2,048-token prefill (eager passes of their own), and the host's time to launch a mixed step")
@@ -536,7 +539,7 @@ def main() -> int:
         extra = args.warmup + args.steps + decode_during_prefill(b, args.context) + 16
         cfg, eng = build_engine(cfg_json, args.dtype, max(b, 1), args.context, extra, layers,
                                 use_graphs=not args.no_graphs, max_context=args.max_context)
-        sec = decode_run(eng, cfg, b, args.context, args.steps, args.warmup)
+        sec = decode_run(eng, cfg, b, args.context, args.steps, args.warmup, sampled=args.sampled)
         ms[b] = sec * 1e3
         if b == args.batch:
             main_hash = decode_run.ids_hash
@@ -563,7 +566,8 @@ def main() -> int:
 
     sec = ms[args.batch] / 1e3
     out = {
-        "metric": f"decode tok/s @ batch {args.batch}, context {args.context} ({args.preset} shapes)",
+        "metric": f"decode tok/s @ batch {args.batch}, context {args.context} ({args.preset} shapes)"
+                  + (", sampled (temperature 0.8, top-k 40, top-p 0.95)" if args.sampled else ""),
         "value": round(args.batch / sec, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms[args.batch], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic: random N(0, 0.02) weights, uniform random token ids",
