@@ -240,13 +240,16 @@ __device__ __forceinline__ void soft_any(int h, floatx16& s, Frag (&pf)[2], Soft
   else soft_step<true>(h, s, pf, st, tk, lh, sc2);
 }
 
+// WIN: the rows see a window of keys (without one, a row's first key is key 0, which costs no register)
+template <bool WIN>
 __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     const bf16_t* __restrict__ q, int ldq, int q_off, bf16_t* __restrict__ out, int ldo, int H, int Hk,
     const bf16_t* __restrict__ cache, int lgP, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ positions, const int* __restrict__ row_seg, const int* __restrict__ tile_row0,
-    const int* __restrict__ tile_rows, int n_tiles, int window, float scale, int n_splits, int part_rows,
+    const int* __restrict__ tile_rows, int n_tiles, int window_arg, float scale, int n_splits, int part_rows,
     float* __restrict__ parts) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  const int window = WIN ? window_arg : 0;
   constexpr int d = HD;
   constexpr int DT = d / 32;
   const int P = 1 << lgP;
@@ -287,12 +290,18 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     t_begin += split * per * KT;
     last = min(last, t_begin + per * KT - 1);
   }
-  float* part_o = parts ? parts + ((size_t)split * part_rows * H + h) * d : nullptr;           // + row * H * d
-  float* part_ml = parts ? parts + (size_t)n_splits * part_rows * H * d + ((size_t)split * part_rows * H + h) * 2 : nullptr;
+  // Where a block with a range of keys leaves its rows: [range][row][head][d] floats, then [range][row][head][m, l].
+  // Worked out where it is needed, from the kernel's arguments, so that nothing of it lives through the loop.
+  auto part_index = [&]() {
+    const int id = blockIdx.x;
+    const int sp = (Hk % 8 == 0 ? id / 8 : id) % n_splits;
+    return (size_t)sp * part_rows * H + h;  // + row * H
+  };
   if (t_begin > last) {  // more ranges than key tiles: nothing here
-    if (part_ml && tid < nrows) {
-      part_ml[(size_t)(row0 + tid) * H * 2] = -INFINITY;
-      part_ml[(size_t)(row0 + tid) * H * 2 + 1] = 0.f;
+    if (parts && tid < nrows) {
+      float* ml = parts + (size_t)n_splits * part_rows * H * d + (part_index() + (size_t)(row0 + tid) * H) * 2;
+      ml[0] = -INFINITY;
+      ml[1] = 0.f;
     }
     return;
   }
@@ -305,8 +314,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
   // the wave's 2 x 32 query rows as second operands: row = lane % 32, 8 elements of d per lane and step of 16
   Frag qf[2][d / 16];
   Soft st[2];
+  u32x4 qv[2][d / 16];  // on their way from memory while the first keys and values are asked for
   {
-    u32x4 qv[2][d / 16];
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
       const int my_row = rh * 64 + rt * 32 + li;
@@ -320,14 +329,6 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
       st[rt].pos = min(pos0 + my_row, last);
       st[rt].lo = (window > 0 && pos0 + my_row - window + 1 > 0) ? pos0 + my_row - window + 1 : 0;
     }
-    // from here on the values live in accumulation registers (left to the compiler, they are copied there in every pass)
-#pragma unroll
-    for (int rt = 0; rt < 2; ++rt)
-#pragma unroll
-      for (int ks = 0; ks < d / 16; ++ks) {
-        asm volatile("" : "+a"(qv[rt][ks]));
-        qf[rt][ks] = __builtin_bit_cast(Frag, qv[rt][ks]);
-      }
   }
   // whether every row of row tile rt sees all of the wave's 32 keys of the tile that starts at t0
   auto sees_all = [&](int rt, int t0) {
@@ -344,13 +345,16 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
   // The 4 loads of a tile's K (and of its V) differ by 1 KiB in LDS, which the instruction's offset field gives; that
   // field counts for the address in memory too, so the lanes' offsets take it back (and 3 KiB more, which the base
   // gives back, so that none is negative).
-  int koff[4], voff[4];
+  // (The lanes' offsets of the 4 loads of V differ by the same step, which goes into the loads' scalar offset: one
+  // register instead of four.)
+  int koff[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int sw = 2 * (i & 1) + (i >> 1);
     koff[i] = (4 * sw + lane / 16) * (d * 2) + (((lane % 16) ^ (lane / 16) ^ (4 * i)) * 16) + 3072 - i * 1024;
-    voff[i] = (32 * i + lane % 32) * (P * 2) + (lane / 32) * 16 + 3072 - i * 1024;
   }
+  const int voff = (lane % 32) * (P * 2) + (lane / 32) * 16 + 3072;
+  const int vstep = 32 * P * 2 - 1024;  // load i: elements 32 i .. of a page row of 2 P bytes, 1 KiB further in LDS
   auto group_of = [&](int j) { return min(t_begin + j * KT + 16 * wave, last16); };  // first key of the wave's 16
   auto page_of = [&](int j) { return __builtin_amdgcn_readfirstlane(bt[group_of(j) >> lgP]); };
   const bf16_t* k_head_low = k_head - 1536;  // 3 KiB lower
@@ -369,10 +373,10 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     const BufferRsrc vr = make_rsrc(v_head_low + (size_t)__builtin_amdgcn_readfirstlane(page) * page_stride);
     const int soff = (group_of(j) & (P - 1)) * 2;
     const lds_ptr dst = (lds_ptr)(smem + V_BASE + (j % STG) * V_STAGE + wave * 4096);
-    if (i == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[0], soff, 0, 0);
-    if (i == 1) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[1], soff, 1024, 0);
-    if (i == 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[2], soff, 2048, 0);
-    if (i == 3) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[3], soff, 3072, 0);
+    if (i == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff, 0, 0);
+    if (i == 1) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + vstep, 1024, 0);
+    if (i == 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + 2 * vstep, 2048, 0);
+    if (i == 3) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + 3 * vstep, 3072, 0);
   };
   auto k_load = [&](int j, int page) {
     const BufferRsrc kr = make_rsrc(k_head_low + (size_t)__builtin_amdgcn_readfirstlane(page) * page_stride);
@@ -387,10 +391,32 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     const BufferRsrc vr = make_rsrc(v_head_low + (size_t)__builtin_amdgcn_readfirstlane(page) * page_stride);
     const int soff = (group_of(j) & (P - 1)) * 2;
     const lds_ptr dst = (lds_ptr)(smem + V_BASE + (j % STG) * V_STAGE + wave * 4096);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[0], soff, 0, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[1], soff, 1024, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[2], soff, 2048, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff[3], soff, 3072, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + vstep, 1024, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + 2 * vstep, 2048, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + 3 * vstep, 3072, 0);
+  };
+  // The same with the lanes' offsets worked out on the spot, for the passes that have no register to spare for them
+  // (the compiler would otherwise keep them through the loop and spill something else)
+  auto kv_load_tight = [&](int jk, int pagek, int jv, int pagev) {
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    const BufferRsrc kr = make_rsrc(k_head_low + (size_t)__builtin_amdgcn_readfirstlane(pagek) * page_stride);
+    const int ksoff = (group_of(jk) & (P - 1)) * (d * 2);
+    const lds_ptr kdst = (lds_ptr)(smem + (jk % STG) * K_STAGE + (16 * wave) * 256);
+    const int x = (ln / 16) * (d * 2) + (((ln % 16) ^ (ln / 16)) * 16);  // (row, place) of load 0; load i: place ^ 4 i
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, kdst, 16, x + 3072, ksoff, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, kdst, 16, (x ^ 64) + 8 * (d * 2) + 2048, ksoff, 1024, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, kdst, 16, (x ^ 128) + 4 * (d * 2) + 1024, ksoff, 2048, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, kdst, 16, (x ^ 192) + 12 * (d * 2), ksoff, 3072, 0);
+    const BufferRsrc vr = make_rsrc(v_head_low + (size_t)__builtin_amdgcn_readfirstlane(pagev) * page_stride);
+    const int vsoff = (group_of(jv) & (P - 1)) * 2;
+    const lds_ptr vdst = (lds_ptr)(smem + V_BASE + (jv % STG) * V_STAGE + wave * 4096);
+    const int vo = (ln % 32) * (P * 2) + (ln / 32) * 16 + 3072;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, vdst, 16, vo, vsoff, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, vdst, 16, vo, vsoff + vstep, 1024, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, vdst, 16, vo, vsoff + 2 * vstep, 2048, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, vdst, 16, vo, vsoff + 3 * vstep, 3072, 0);
   };
   // Stale positions of the V^T stage of tile j are cleared: what lies beyond the last key or in front of the first
   // one that a row of the block sees may be anything, and 0 x NaN is NaN.  (A group of 16 keys beyond the last one
@@ -463,14 +489,16 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     const float m_safe = m == -INFINITY ? 0.f : m;
     const float a1 = exp2_neg(m1 - m_safe), a2 = exp2_neg(m2 - m_safe);
     const float l = l1 * a1 + l2 * a2;
-    if (part_o) {  // the row over this range of keys, as a float32 row with its reference and sum
+    if (parts) {  // the row over this range of keys, as a float32 row with its reference and sum
+      const size_t at = part_index() + (size_t)(row0 + my_row) * H;
       if (lh == 0) {
-        part_ml[(size_t)(row0 + my_row) * H * 2] = l > 0.f ? m : -INFINITY;
-        part_ml[(size_t)(row0 + my_row) * H * 2 + 1] = l;
+        float* ml = parts + (size_t)n_splits * part_rows * H * d + at * 2;
+        ml[0] = l > 0.f ? m : -INFINITY;
+        ml[1] = l;
       }
       if (!(l > 0.f)) return;  // the row sees no key of the range
       const float inv = 1.0f / l;
-      float* prow = part_o + (size_t)(row0 + my_row) * H * d;
+      float* prow = parts + at * d;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
@@ -531,6 +559,16 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
       vpg = pg3;
       kpg = page_of(4);
     }
+    __builtin_amdgcn_sched_barrier(0);
+    // from here on the query rows live in accumulation registers (left to the compiler, they are copied there in every
+    // pass)
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int ks = 0; ks < d / 16; ++ks) {
+        asm volatile("" : "+a"(qv[rt][ks]));
+        qf[rt][ks] = __builtin_bit_cast(Frag, qv[rt][ks]);
+      }
     __builtin_amdgcn_sched_barrier(0);
     wait_loads_but<2 * LOADS_PER_TILE>();  // K(0), K(1), V(0)
     __builtin_amdgcn_s_barrier();
@@ -631,8 +669,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
         }
       }
       if constexpr (MASKED) {  // this kind of pass has no registers to spare for keeping the loads' operands through slot B
-        k_load(i + 5, kpg);
-        v_load(i + 4, vpg);
+        kv_load_tight(i + 5, kpg, i + 4, vpg);
         vpg = kpg;
         kpg = page_of(i + 6);
         __builtin_amdgcn_sched_barrier(0);
@@ -681,6 +718,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
       pass(std::integral_constant<int, SOFT_MASKED>{}, i, i);
       ++i;
     }
+    // (what the passes above saw, as one scalar: the loops below have no register to spare for the lanes' flags)
+    const bool beyond_early = __builtin_amdgcn_ballot_w64((st[0].beyond | st[1].beyond) != 0) != 0;
     if (i < n_kt) {
       int i_end = i + 1;
       while (i_end < n_kt && all_seen(i_end)) ++i_end;
@@ -696,13 +735,12 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
       st[1].l += halves_sum(st[1].sum);
     }
     // a sum this large (or no number at all) means that some P was: such a block computes its rows again below
-#pragma unroll
-    for (int rt = 0; rt < 2; ++rt) st[rt].beyond |= st[rt].l < 0x1p90f ? 0 : 1;
+    const bool beyond_late = __builtin_amdgcn_ballot_w64(!(st[0].l < 0x1p90f) || !(st[1].l < 0x1p90f)) != 0;
 
     __builtin_amdgcn_sched_barrier(0);
     wait_loads_but<0>();                    // no direct load is on its way into LDS
     __builtin_amdgcn_sched_barrier(0);
-    if (__builtin_amdgcn_ballot_w64((st[0].beyond | st[1].beyond) != 0) != 0 && lane == 0) block_beyond = 1;
+    if ((beyond_early || beyond_late) && lane == 0) block_beyond = 1;
     __syncthreads();
     if (!block_beyond) {
       leave(0, o[0], st[0].m, st[0].l);
@@ -716,7 +754,10 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
 
   // ---- the plain loop: a score outran its row's reference somewhere in the block.  One row tile after the other,
   // one thing after the other, references that move and O shrunk by vector instructions when they do.
-  for (int rt = 0; rt < 2; ++rt) {
+  // (the row tile as a constant: indexed by a variable, the query rows and the rows' state would live in memory, and
+  // the loops above would keep that memory up to date)
+  auto plain_rows = [&](auto RT_) {
+    constexpr int rt = decltype(RT_)::value;
     floatx16 o[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -778,7 +819,9 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     leave(rt, o, m_run, l_run);
     __syncthreads();
     add_and_write(rt, o, m_run, l_run);
-  }
+  };
+  plain_rows(std::integral_constant<int, 0>{});
+  plain_rows(std::integral_constant<int, 1>{});
 }
 
 // The ranges of keys of a row added up: out = sum_s w_s O_s / sum_s w_s with w_s = l_s 2^(m_s - max m).  A block
@@ -833,16 +876,19 @@ int launch_attn_prefill_wide(const bf16_t* q, int ldq, int q_off, bf16_t* out, i
   int lgP = 0;
   while ((1 << lgP) < page_tokens) ++lgP;
   static bool configured[64] = {};
+  const auto kernel = window > 0 ? attn_prefill_wide_kernel<true> : attn_prefill_wide_kernel<false>;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return (int)e;
   if (dev < 0 || dev >= 64) return APC_ERR_UNSUPPORTED;
   if (!configured[dev]) {  // more LDS than a kernel gets without asking
-    e = hipFuncSetAttribute((const void*)attn_prefill_wide_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES + 16);
-    if (e != hipSuccess) return (int)e;
+    for (const void* f : {(const void*)attn_prefill_wide_kernel<true>, (const void*)attn_prefill_wide_kernel<false>}) {
+      e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES + 16);
+      if (e != hipSuccess) return (int)e;
+    }
     configured[dev] = true;
   }
-  hipLaunchKernelGGL(attn_prefill_wide_kernel, dim3(n_tiles * H * n_splits), dim3(256), LDS_BYTES + 16, stream, q, ldq,
+  hipLaunchKernelGGL(kernel, dim3(n_tiles * H * n_splits), dim3(256), LDS_BYTES + 16, stream, q, ldq,
                      q_off, out, ldo, H, Hk, cache, lgP, block_table, max_blocks, positions, row_seg, tile_row0, tile_rows,
                      n_tiles, window, scale, n_splits, part_rows, parts);
   APC_LAUNCH_CHECK();
