@@ -126,6 +126,31 @@ def test_sampler_over_a_real_vocabulary(one_block):
     assert not bad, bad
 
 
+def test_sampler_over_more_than_a_million_logits():
+    """Beyond 2^20 logits the sort key (32 bits of value, 21 of id) takes a fifth digit of 13 bits: the sampler with many
+    blocks a row against the one with one block a row (and against the plain sampler on the rows that are cheap there:
+    top-k leaves few candidates)."""
+    o = ops()
+    V, R = (1 << 20) + 4099, 6
+    lg = gen(R, V, seed=5) * 3.0
+    lg[0, 7] = lg[0, V - 1] = lg[0, V // 2] = 25.0           # ties at the top, as far apart as ids get
+    lg[1] = torch.round(lg[1] * 4) / 4                        # runs of equal values everywhere
+    temps = np.asarray([0.7, 1.0, 0.9, 1.2, 0.8, 1.0], np.float32)
+    ks = np.asarray([0, 0, 40, 5, 0, 3000], np.int32)
+    ps = np.asarray([1.0, 0.9, 0.95, 1.0, 0.5, 0.99], np.float32)
+    us = np.random.default_rng(9).random(R).astype(np.float32)
+    d = [torch.from_numpy(a).to(DEV) for a in (temps, ks, ps, us)]
+    lgd = lg.to(DEV)
+    many = torch.empty(R, dtype=torch.int32, device=DEV)
+    one = torch.empty(R, dtype=torch.int32, device=DEV)
+    o.sample_rows(lgd, *d, many)
+    o.sample_rows(lgd, *d, one, one_block=True)
+    assert many.cpu().tolist() == one.cpu().tolist()
+    lgn = lg.numpy()
+    for r in (2, 3):
+        assert int(many[r]) == P.sample(lgn[r], float(temps[r]), int(ks[r]), float(ps[r]), float(us[r]))
+
+
 def test_a_folder_at_the_widths_of_a_3b_model_through_the_front_door(tmp_path):
     """config.json + model.safetensors of two layers at the widths of Llama-3.2-3B (hidden 3072, 24 heads over 8 of
     128, feed-forward 8192, vocabulary 128,256, tied head: 1.2 GB in bfloat16) written tensor by tensor, loaded by
