@@ -824,38 +824,49 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
   plain_rows(std::integral_constant<int, 1>{});
 }
 
-// The ranges of keys of a row added up: out = sum_s w_s O_s / sum_s w_s with w_s = l_s 2^(m_s - max m).  A block
-// takes a row of a tile, a thread four elements of a head at a time.
+// The ranges of keys of a row added up: out = sum_s w_s O_s / sum_s w_s with w_s = l_s 2^(m_s - max m).  A thread
+// takes four elements of a head of a row; blockIdx.y counts the blocks of 256 threads a row needs.
 __global__ __launch_bounds__(256) void attn_wide_merge_kernel(const float* __restrict__ parts, int n_splits, int part_rows,
                                                               int H, const int* __restrict__ tile_row0,
                                                               const int* __restrict__ tile_rows, bf16_t* __restrict__ out,
                                                               int ldo) {
   constexpr int d = HD;
   const int tile = blockIdx.x / ATTN_WIDE_ROWS, r = blockIdx.x % ATTN_WIDE_ROWS;
-  if (r >= tile_rows[tile]) return;
+  const int hq = blockIdx.y * 256 + threadIdx.x;
+  if (r >= tile_rows[tile] || hq >= H * (d / 4)) return;
   const int row = tile_row0[tile] + r;
   const float* part_ml = parts + (size_t)n_splits * part_rows * H * d;
   const size_t plane = (size_t)part_rows * H;
-  for (int hq = threadIdx.x; hq < H * (d / 4); hq += 256) {
-    const int h = hq / (d / 4), e = (hq % (d / 4)) * 4;
-    const size_t at = (size_t)row * H + h;
-    float m = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) m = fmaxf(m, part_ml[(s * plane + at) * 2]);
-    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-    float sum = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float ms = part_ml[(s * plane + at) * 2];
-      if (ms == -INFINITY) continue;
-      const float w = part_ml[(s * plane + at) * 2 + 1] * exp2_neg(ms - m);
-      acc += w * *reinterpret_cast<const floatx4*>(parts + (s * plane + at) * d + e);
+  const int h = hq / (d / 4), e = (hq % (d / 4)) * 4;
+  const size_t at = (size_t)row * H + h;
+  constexpr int MOST = 8;  // ranges (the launch code refuses more)
+  float ms[MOST], ls[MOST];
+  floatx4 os[MOST];
+  float m = -INFINITY;
+#pragma unroll
+  for (int s = 0; s < MOST; ++s) {
+    if (s < n_splits) {
+      ms[s] = part_ml[(s * plane + at) * 2];
+      ls[s] = part_ml[(s * plane + at) * 2 + 1];
+      os[s] = *reinterpret_cast<const floatx4*>(parts + (s * plane + at) * d + e);
+      m = fmaxf(m, ms[s]);
+    }
+  }
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  float sum = 0.f;
+#pragma unroll
+  for (int s = 0; s < MOST; ++s) {
+    if (s < n_splits && ms[s] != -INFINITY) {  // (a range that the row sees no key of has left no row)
+      const float w = ls[s] * exp2_neg(ms[s] - m);
+      acc += w * os[s];
       sum += w;
     }
-    const float inv = sum > 0.f ? 1.0f / sum : 0.f;
-    uint2 pk;
-    pk.x = pack_bf16x2(acc[0] * inv, acc[1] * inv);
-    pk.y = pack_bf16x2(acc[2] * inv, acc[3] * inv);
-    *reinterpret_cast<uint2*>(out + (size_t)row * ldo + (size_t)h * d + e) = pk;
   }
+  const float inv = sum > 0.f ? 1.0f / sum : 0.f;
+  uint2 pk;
+  pk.x = pack_bf16x2(acc[0] * inv, acc[1] * inv);
+  pk.y = pack_bf16x2(acc[2] * inv, acc[3] * inv);
+  *reinterpret_cast<uint2*>(out + (size_t)row * ldo + (size_t)h * d + e) = pk;
 }
 
 }  // namespace
@@ -870,7 +881,8 @@ int launch_attn_prefill_wide(const bf16_t* q, int ldq, int q_off, bf16_t* out, i
                              int n_tiles, int window, float scale, int n_splits, int part_rows, float* parts,
                              hipStream_t stream) {
   if (!attn_wide_takes(ATTN_WIDE_HEAD, page_tokens)) return APC_ERR_UNSUPPORTED;
-  if (n_splits < 1 || (n_splits > 1 && (!parts || part_rows <= 0)) || (long)n_tiles * H * n_splits > 0x7fffffffL)
+  if (n_splits < 1 || n_splits > 8 || (n_splits > 1 && (!parts || part_rows <= 0)) ||
+      (long)n_tiles * H * n_splits > 0x7fffffffL)
     return APC_ERR_BAD_ARG;
   if (n_splits == 1) parts = nullptr;
   int lgP = 0;
@@ -893,7 +905,8 @@ int launch_attn_prefill_wide(const bf16_t* q, int ldq, int q_off, bf16_t* out, i
                      n_tiles, window, scale, n_splits, part_rows, parts);
   APC_LAUNCH_CHECK();
   if (n_splits > 1) {
-    hipLaunchKernelGGL(attn_wide_merge_kernel, dim3(n_tiles * ATTN_WIDE_ROWS), dim3(256), 0, stream, parts, n_splits,
+    hipLaunchKernelGGL(attn_wide_merge_kernel, dim3(n_tiles * ATTN_WIDE_ROWS, ceil_div(H * (ATTN_WIDE_HEAD / 4), 256)),
+                       dim3(256), 0, stream, parts, n_splits,
                        part_rows, H, tile_row0, tile_rows, out, ldo);
     APC_LAUNCH_CHECK();
   }
