@@ -296,9 +296,9 @@ static int launch_gemm(const bf16_t* A, int lda, const bf16_t* W, const bf16_t* 
   if constexpr (!PRE) {
     // many rows, K a multiple of 128: the kernel that keeps the weights out of LDS (same sums, bit for bit)
     if (gemm_direct_takes(MODE, A, lda, C, ldc, M, N, K)) return launch_gemm_direct(MODE, A, lda, W, W2, C, ldc, M, N, K, stream);
-  } else if constexpr (MODE == G_SWIGLU) {
-    if (gemm_direct_swiglu_pre_takes(A, lda, C, ldc, M, N, K, pre.parts))
-      return launch_gemm_direct_swiglu_pre(A, lda, pre.ss, pre.parts, pre.eps, W, W2, C, ldc, M, N, K, stream);
+  } else if constexpr (MODE == G_SWIGLU || MODE == G_STORE_BF16) {
+    if (gemm_direct_pre_takes(MODE, A, lda, C, ldc, M, N, K, pre.parts))
+      return launch_gemm_direct_pre(MODE, A, lda, pre.ss, pre.parts, pre.eps, W, W2, C, ldc, M, N, K, stream);
   }
   if constexpr (MODE == G_SWIGLU) {
     // From 1,024 rows on the tile of 256 rows x 128 outputs takes as many columns as make whole rounds of one tile a
@@ -536,6 +536,21 @@ __global__ __launch_bounds__(256) void gemm_finish_qkv_rope_kernel(const float* 
 // How many slices of K the product of many rows (gemm_direct_bf16.hip) wants for this shape: 1, or 2 when narrow
 // tiles would be needed to fill the chip otherwise.  The caller brings the workspace for apc_gemm_splitk_bf16.
 APC_EXPORT int apc_gemm_direct_k_split(int M, int N, int K) { return gemm_direct_k_split(M, N, K); }
+
+// residual += A . W^T for more than 1,024 rows, leaving the row for the RMS norm (weight g) that reads the residual
+// next: raw [M][N] bfloat16 and ss [M][parts] (see gemm_direct.h).  apc_gemm_direct_emit_parts: the parts these sizes
+// give, 0 if this entry point does not take them.
+APC_EXPORT int apc_gemm_direct_emit_parts(const void* A, int lda, const void* residual, int ldc, int M, int N, int K) {
+  return gemm_direct_emit_parts(A, lda, residual, ldc, M, N, K);
+}
+APC_EXPORT int apc_gemm_direct_emit_bf16(const void* A, int lda, const void* W, float* residual, int ldc, int M, int N,
+                                         int K, const float* g, void* raw, int ldr, float* ss, int parts,
+                                         float* workspace, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (!aligned16(W)) return APC_ERR_UNSUPPORTED;
+  return launch_gemm_direct_emit((const bf16_t*)A, lda, (const bf16_t*)W, residual, ldc, M, N, K, g, (bf16_t*)raw, ldr, ss,
+                                 parts, workspace, stream);
+}
 
 APC_EXPORT int apc_gemm_splitk_bf16(const void* A, int lda, const void* W, const void* Wu, void* C, int ldc, int M,
                                     int N, int K, int mode, int k_split, float* workspace, hipStream_t stream) {

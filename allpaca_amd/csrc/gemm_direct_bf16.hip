@@ -27,14 +27,25 @@
 
 namespace {
 
-enum { D_STORE_BF16 = 0, D_STORE_F32 = 1, D_ACC_F32 = 2, D_SWIGLU = 3, D_SWIGLU_PRE = 4 };
+// D_..._PRE: A is a row that a product into the residual left for the RMS norm, and the sums are scaled by the row's
+// 1 / sqrt(mean of x^2 + eps).  D_ACC_EMIT: add into the residual and leave that row for the norm that reads it next.
+enum { D_STORE_BF16 = 0, D_STORE_F32 = 1, D_ACC_F32 = 2, D_SWIGLU = 3, D_SWIGLU_PRE = 4, D_ACC_EMIT = 5,
+       D_STORE_BF16_PRE = 6 };
 __host__ __device__ constexpr bool is_swiglu(int mode) { return mode == D_SWIGLU || mode == D_SWIGLU_PRE; }
+__host__ __device__ constexpr bool is_pre(int mode) { return mode == D_SWIGLU_PRE || mode == D_STORE_BF16_PRE; }
+__host__ __device__ constexpr bool is_acc(int mode) { return mode == D_ACC_F32 || mode == D_ACC_EMIT; }
 
-// the sums of squares of rows that a product into the residual left for the RMS norm (D_SWIGLU_PRE)
+// What goes with a norm folded into the product.  PRE: ss [M][parts] sums of x^2 of the rows (read), eps.
+// EMIT: g the norm's weight [N]; raw [M][ldr] takes bfloat16(x g); ss [M][parts] takes the sums of x^2 of the block's
+// columns at part0 + the block's column tile.
 struct DirectPre {
-  const float* ss;
+  float* ss;
   int parts;
   float eps;
+  const float* g;
+  bf16_t* raw;
+  int ldr;
+  int part0;
 };
 
 constexpr int R = 4;           // ring slots of W fragments: loads run R - 1 steps of 32 columns ahead
@@ -197,7 +208,7 @@ __device__ __forceinline__ void direct_tile(int bid, const bf16_t* __restrict__ 
   // D[i][j]: i = output (lane / 16) * 4 + r within the band, j = row lane % 16 within the row group
   const int mi = lane % 16, nq = lane / 16;
   float row_scale[BMG];
-  if constexpr (MODE == D_SWIGLU_PRE) {
+  if constexpr (is_pre(MODE)) {
     // 1 / sqrt(mean of x^2 + eps) of the block's rows, a thread a row, through the LDS that the stages have left
     float* scales = reinterpret_cast<float*>(&As[0][0][0]);
     __syncthreads();
@@ -217,10 +228,38 @@ __device__ __forceinline__ void direct_tile(int bid, const bf16_t* __restrict__ 
 #pragma unroll
     for (int a = 0; a < BMG; ++a) row_scale[a] = scales[a * 16 + mi];
   }
+  float emit_sq[BMG];
 #pragma unroll
   for (int a = 0; a < BMG; ++a) {
     const int m = m0 + a * 16 + mi;
-    if constexpr (MODE == D_ACC_F32) {
+    if constexpr (MODE == D_ACC_EMIT) {
+      floatx4 cv[NOUT];
+      float sq = 0.f;
+#pragma unroll
+      for (int f = 0; f < NOUT; ++f) {
+        const int n = (band0 + f) * 16 + nq * 4;
+        cv[f] = (m < M && n < N) ? *reinterpret_cast<const floatx4*>((const float*)C + (size_t)m * ldc + n)
+                                 : floatx4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int f = 0; f < NOUT; ++f) {
+        const int n = (band0 + f) * 16 + nq * 4;
+        if (m < M && n < N) {
+          const floatx4 x = cv[f] + acc[a][f];
+          const floatx4 gv = *reinterpret_cast<const floatx4*>(pre.g + n);
+          *reinterpret_cast<floatx4*>((float*)C + (size_t)m * ldc + n) = x;
+          uint2 o;
+          o.x = pack_bf16x2(x[0] * gv[0], x[1] * gv[1]);
+          o.y = pack_bf16x2(x[2] * gv[2], x[3] * gv[3]);
+          *reinterpret_cast<uint2*>(pre.raw + (size_t)m * pre.ldr + n) = o;
+          sq += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+        }
+      }
+      // the row's sum over the wave's columns: the four lanes that hold pieces of row mi
+      sq += __shfl_xor(sq, 16, WAVE);
+      sq += __shfl_xor(sq, 32, WAVE);
+      emit_sq[a] = sq;
+    } else if constexpr (MODE == D_ACC_F32) {
       floatx4 cv[NOUT];  // all loads of the residual first: a store between two loads would make the second wait
 #pragma unroll
       for (int f = 0; f < NOUT; ++f) {
@@ -245,9 +284,10 @@ __device__ __forceinline__ void direct_tile(int bid, const bf16_t* __restrict__ 
           float v[4];
 #pragma unroll
           for (int r = 0; r < 4; ++r)
-            v[r] = MODE == D_STORE_BF16  ? acc[a][f][r]
-                   : MODE == D_SWIGLU ? silu_f(acc[a][f][r]) * acc[a][NOUT + f][r]
-                                      : silu_f(acc[a][f][r] * row_scale[a]) * (acc[a][NOUT + f][r] * row_scale[a]);
+            v[r] = MODE == D_STORE_BF16       ? acc[a][f][r]
+                   : MODE == D_STORE_BF16_PRE ? acc[a][f][r] * row_scale[a]
+                   : MODE == D_SWIGLU         ? silu_f(acc[a][f][r]) * acc[a][NOUT + f][r]
+                                              : silu_f(acc[a][f][r] * row_scale[a]) * (acc[a][NOUT + f][r] * row_scale[a]);
           uint2 o;
           o.x = pack_bf16x2(v[0], v[1]);
           o.y = pack_bf16x2(v[2], v[3]);
@@ -256,6 +296,52 @@ __device__ __forceinline__ void direct_tile(int bid, const bf16_t* __restrict__ 
       }
     }
   }
+  if constexpr (MODE == D_ACC_EMIT) {
+    // the rows' sums of squares over the block's columns: the four waves' sums added in wave order through the LDS
+    // that the stages have left
+    float* sums = reinterpret_cast<float*>(&As[0][0][0]);  // [wave][BMG * 16]
+    __syncthreads();
+    if (nq == 0) {
+#pragma unroll
+      for (int a = 0; a < BMG; ++a) sums[wave * (BMG * 16) + a * 16 + mi] = emit_sq[a];
+    }
+    __syncthreads();
+    if (tid < BMG * 16 && m0 + tid < M) {
+      float sum = sums[tid];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) sum += sums[w * (BMG * 16) + tid];
+      pre.ss[(size_t)(m0 + tid) * pre.parts + pre.part0 + nt] = sum;
+    }
+  }
+}
+
+// What follows a product with K in slices when the row goes on to an RMS norm: the slices are added in order, then
+// added into the residual, and the row for the norm is left (as D_ACC_EMIT does).  A block has 1,024 columns of a row,
+// a thread four of them; ss is [M][ceil(N / 1024)].
+__global__ __launch_bounds__(256) void gemm_direct_finish_emit_kernel(const float* __restrict__ partials, int k_split, int M,
+                                                                      int N, float* __restrict__ C, int ldc,
+                                                                      const float* __restrict__ g, bf16_t* __restrict__ raw,
+                                                                      int ldr, float* __restrict__ ss) {
+  __shared__ float red[4];
+  const int m = blockIdx.y, n = (blockIdx.x * 256 + threadIdx.x) * 4;
+  float sq = 0.f;
+  if (n < N) {
+    const size_t plane = (size_t)M * N;
+    const float* src = partials + (size_t)m * N + n;
+    floatx4 x = *reinterpret_cast<const floatx4*>(src);
+    for (int s = 1; s < k_split; ++s) x += *reinterpret_cast<const floatx4*>(src + s * plane);
+    floatx4* dst = reinterpret_cast<floatx4*>(C + (size_t)m * ldc + n);
+    x += *dst;
+    *dst = x;
+    const floatx4 gv = *reinterpret_cast<const floatx4*>(g + n);
+    uint2 o;
+    o.x = pack_bf16x2(x[0] * gv[0], x[1] * gv[1]);
+    o.y = pack_bf16x2(x[2] * gv[2], x[3] * gv[3]);
+    *reinterpret_cast<uint2*>(raw + (size_t)m * ldr + n) = o;
+    sq = x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+  }
+  const float total = block_sum<256>(sq, red);
+  if (threadIdx.x == 0) ss[(size_t)m * gridDim.x + blockIdx.x] = total;
 }
 
 template <int NF, int MODE>
@@ -368,7 +454,7 @@ int launch_gemm_direct_slices(const bf16_t* A, int lda, const bf16_t* W, float* 
 
 namespace {
 bool direct_takes(int mode, int min_rows, const void* A, int lda, const void* C, int ldc, int M, int N, int K) {
-  if (mode < 0 || mode > D_SWIGLU_PRE || M < min_rows || K < 128 || K % 128 || N % 4 || ldc % 4) return false;
+  if (mode < 0 || mode > D_STORE_BF16_PRE || M < min_rows || K < 128 || K % 128 || N % 4 || ldc % 4) return false;
   if (((uintptr_t)A & 15u) || ((uintptr_t)C & 15u) || lda % 8) return false;
   // the lanes' byte offsets into the block's rows of A and the wave's bands of W are 32-bit
   if ((long)128 * lda * 2 >= 0x7fffffffL || (long)8 * ceil_div(K, 32) * 1024 >= 0x7fffffffL) return false;
@@ -382,20 +468,24 @@ int launch_columns(int nf, int mode, const bf16_t* A, int lda, const bf16_t* W, 
     case D_STORE_F32: return launch_mode<D_STORE_F32>(nf, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
     case D_ACC_F32: return launch_mode<D_ACC_F32>(nf, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
     case D_SWIGLU: return launch_mode<D_SWIGLU>(nf, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
-    default: return launch_mode<D_SWIGLU_PRE>(nf, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
+    case D_SWIGLU_PRE: return launch_mode<D_SWIGLU_PRE>(nf, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
+    case D_ACC_EMIT: return launch_mode<D_ACC_EMIT>(nf, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
+    default: return launch_mode<D_STORE_BF16_PRE>(nf, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
   }
 }
 
-int launch_direct(int mode, const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M, int N,
-                  int K, hipStream_t stream, DirectPre pre) {
-  const bool swiglu = is_swiglu(mode);
+// How a product's columns go out: one launch of tiles with nf1 bands a wave, or, where the last round of blocks would
+// be far from full (2,048 rows x 14,336 SwiGLU outputs: 3.5 rounds of tiles with 8 bands a wave), the first cols1
+// columns, which make whole rounds, on nf1 and the rest on whatever tile fills a round best (there: 4 bands, a round
+// of 0.72 of the time).  3 time units for the second launch.
+struct ColumnPlan {
+  int nf1, cols1, nf2;  // cols1 == 0: one launch
+};
+ColumnPlan plan_columns(int M, int N, bool swiglu) {
   double whole = 0.0;
   const int nf = pick_bands(M, N, swiglu, 1, &whole);
-  // A launch whose last round is far from full (2,048 rows x 14,336 SwiGLU outputs: 3.5 rounds of tiles with 8 bands a
-  // wave) in two: the columns that make whole rounds, then the rest on whatever tile fills a round best (there: 4
-  // bands, a round of 0.72 of the time).  3 time units for the second launch.
   const int mt = ceil_div(M, 128);
-  int best_nf = 0, best_cols = 0, rest_nf = 0;
+  ColumnPlan plan{nf, 0, 0};
   double best = whole;
   if (mt <= 256) {
     for (int f : {3, 4, 5, 6, 8}) {
@@ -406,16 +496,34 @@ int launch_direct(int mode, const bf16_t* A, int lda, const bf16_t* W, const bf1
       double rest = 0.0;
       const int rf = pick_bands(M, N - big_cols * nb, swiglu, 1, &rest);
       const double cost = (double)ceil_div((long)big_cols * mt, 256L) * round_cost(f) + rest + 3.0;
-      if (cost < 0.97 * best) best = cost, best_nf = f, best_cols = big_cols * nb, rest_nf = rf;
+      if (cost < 0.97 * best) best = cost, plan = ColumnPlan{f, big_cols * nb, rf};
     }
   }
-  if (!best_nf) return launch_columns(nf, mode, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
-  const int e = launch_columns(best_nf, mode, A, lda, W, W2, C, ldc, M, best_cols, K, stream, pre);
+  return plan;
+}
+int tile_columns(int nf, bool swiglu) { return 4 * (swiglu ? nf / 2 : nf) * 16; }
+// column tiles of the plan's launches together (the parts of the sums of squares that D_ACC_EMIT leaves)
+int column_tiles(const ColumnPlan& plan, int N, bool swiglu) {
+  if (!plan.cols1) return ceil_div(N, tile_columns(plan.nf1, swiglu));
+  return plan.cols1 / tile_columns(plan.nf1, swiglu) + ceil_div(N - plan.cols1, tile_columns(plan.nf2, swiglu));
+}
+
+int launch_direct(int mode, const bf16_t* A, int lda, const bf16_t* W, const bf16_t* W2, void* C, int ldc, int M, int N,
+                  int K, hipStream_t stream, DirectPre pre) {
+  const bool swiglu = is_swiglu(mode);
+  const ColumnPlan plan = plan_columns(M, N, swiglu);
+  if (!plan.cols1) return launch_columns(plan.nf1, mode, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
+  const int e = launch_columns(plan.nf1, mode, A, lda, W, W2, C, ldc, M, plan.cols1, K, stream, pre);
   if (e) return e;
-  const size_t w_skip = (size_t)(best_cols / 16) * ceil_div(K, 32) * 512;  // whole bands of the tiled layout
-  const size_t elem = (mode == D_STORE_BF16 || swiglu) ? 2 : 4;
-  return launch_columns(rest_nf, mode, A, lda, W + w_skip, swiglu ? W2 + w_skip : W2, (char*)C + (size_t)best_cols * elem,
-                        ldc, M, N - best_cols, K, stream, pre);
+  const size_t w_skip = (size_t)(plan.cols1 / 16) * ceil_div(K, 32) * 512;  // whole bands of the tiled layout
+  const size_t elem = (mode == D_STORE_BF16 || mode == D_STORE_BF16_PRE || swiglu) ? 2 : 4;
+  if (mode == D_ACC_EMIT) {
+    pre.g += plan.cols1;
+    pre.raw += plan.cols1;
+    pre.part0 += plan.cols1 / tile_columns(plan.nf1, swiglu);
+  }
+  return launch_columns(plan.nf2, mode, A, lda, W + w_skip, swiglu ? W2 + w_skip : W2, (char*)C + (size_t)plan.cols1 * elem,
+                        ldc, M, N - plan.cols1, K, stream, pre);
 }
 }  // namespace
 
@@ -429,12 +537,54 @@ int launch_gemm_direct(int mode, const bf16_t* A, int lda, const bf16_t* W, cons
   return launch_direct(mode, A, lda, W, W2, C, ldc, M, N, K, stream, DirectPre{});
 }
 
-bool gemm_direct_swiglu_pre_takes(const void* A, int lda, const void* C, int ldc, int M, int N, int K, int ss_parts) {
-  return ss_parts > 0 && direct_takes(D_SWIGLU_PRE, GEMM_DIRECT_PRE_MIN_ROWS, A, lda, C, ldc, M, N, K);
+bool gemm_direct_pre_takes(int mode, const void* A, int lda, const void* C, int ldc, int M, int N, int K, int ss_parts) {
+  if (ss_parts <= 0 || (mode != D_STORE_BF16 && mode != D_SWIGLU)) return false;
+  // SwiGLU's many outputs fill a round of 128-row tiles from 384 rows on; other products only where the direct kernel
+  // takes them without a folded norm too
+  const int min_rows = mode == D_SWIGLU ? GEMM_DIRECT_PRE_MIN_ROWS : GEMM_DIRECT_MIN_ROWS;
+  return direct_takes(mode, min_rows, A, lda, C, ldc, M, N, K);
 }
 
-int launch_gemm_direct_swiglu_pre(const bf16_t* A, int lda, const float* ss, int ss_parts, float eps, const bf16_t* W,
-                                  const bf16_t* W2, void* C, int ldc, int M, int N, int K, hipStream_t stream) {
-  if (!ss || !W2 || !gemm_direct_swiglu_pre_takes(A, lda, C, ldc, M, N, K, ss_parts)) return APC_ERR_UNSUPPORTED;
-  return launch_direct(D_SWIGLU_PRE, A, lda, W, W2, C, ldc, M, N, K, stream, DirectPre{ss, ss_parts, eps});
+int launch_gemm_direct_pre(int mode, const bf16_t* A, int lda, const float* ss, int ss_parts, float eps, const bf16_t* W,
+                           const bf16_t* W2, void* C, int ldc, int M, int N, int K, hipStream_t stream) {
+  if (!ss || !gemm_direct_pre_takes(mode, A, lda, C, ldc, M, N, K, ss_parts) || (mode == D_SWIGLU) != (W2 != nullptr))
+    return APC_ERR_UNSUPPORTED;
+  DirectPre pre{};
+  pre.ss = const_cast<float*>(ss);
+  pre.parts = ss_parts;
+  pre.eps = eps;
+  return launch_direct(mode == D_SWIGLU ? D_SWIGLU_PRE : D_STORE_BF16_PRE, A, lda, W, W2, C, ldc, M, N, K, stream, pre);
+}
+
+int gemm_direct_emit_parts(const void* A, int lda, const void* C, int ldc, int M, int N, int K) {
+  if (!direct_takes(D_ACC_EMIT, GEMM_DIRECT_MIN_ROWS, A, lda, C, ldc, M, N, K) || M > 65535) return 0;
+  if (gemm_direct_k_split(M, N, K) > 1) return ceil_div(N, 1024);
+  return column_tiles(plan_columns(M, N, false), N, false);
+}
+
+int launch_gemm_direct_emit(const bf16_t* A, int lda, const bf16_t* W, float* C, int ldc, int M, int N, int K,
+                            const float* g, bf16_t* raw, int ldr, float* ss, int ss_parts, float* workspace,
+                            hipStream_t stream) {
+  const int parts = gemm_direct_emit_parts(A, lda, C, ldc, M, N, K);
+  if (!parts || parts != ss_parts || !g || !raw || !ss || ldr < N || ldr % 4 || ((uintptr_t)raw & 7u) ||
+      ((uintptr_t)g & 15u))
+    return APC_ERR_UNSUPPORTED;
+  const int k_split = gemm_direct_k_split(M, N, K);
+  if (k_split > 1) {
+    if (!workspace) return APC_ERR_BAD_ARG;
+    const int e = launch_gemm_direct_slices(A, lda, W, workspace, M, N, K, k_split, stream);
+    if (e) return e;
+    hipLaunchKernelGGL(gemm_direct_finish_emit_kernel, dim3(parts, M), dim3(256), 0, stream, workspace, k_split, M, N, C,
+                       ldc, g, raw, ldr, ss);
+    APC_LAUNCH_CHECK();
+    return 0;
+  }
+  DirectPre pre{};
+  pre.ss = ss;
+  pre.parts = parts;
+  pre.g = g;
+  pre.raw = raw;
+  pre.ldr = ldr;
+  pre.part0 = 0;
+  return launch_direct(D_ACC_EMIT, A, lda, W, nullptr, C, ldc, M, N, K, stream, pre);
 }

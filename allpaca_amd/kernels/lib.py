@@ -53,6 +53,8 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_gemm_splitk_pre_bf16": [P, I, P, I, F, P, P, P, I, I, I, I, I, I, P, P],
         "apc_gemm_splitk_bf16": [P, I, P, P, P, I, I, I, I, I, I, P, P],
         "apc_gemm_direct_k_split": [I, I, I],
+        "apc_gemm_direct_emit_parts": [P, I, P, I, I, I, I],
+        "apc_gemm_direct_emit_bf16": [P, I, P, P, I, I, I, I, P, P, I, P, I, P, P],
         "apc_skinny_gemm_bf16": [P, I, P, P, I, I, I, I, I, P],
         "apc_skinny_swiglu_bf16": [P, I, P, P, P, I, I, I, I, P],
         "apc_attention_prefill_bf16": [P, I, I, P, I, I, I, I, P, I, P, I, P, P, P, P, I, I, I, F, I, I, P, P],
@@ -96,7 +98,7 @@ class KernelTimer:
 _timer = None
 # entry points that launch nothing (questions about sizes): never timed
 NOT_KERNELS = {"apc_attention_decode_whole_fits", "apc_attention_decode_last_fits", "apc_attention_prefill_tile_rows",
-               "apc_gemm_direct_k_split", "apc_sample_rows_scratch_kib"}
+               "apc_gemm_direct_k_split", "apc_gemm_direct_emit_parts", "apc_sample_rows_scratch_kib"}
 
 
 class timing:

@@ -134,6 +134,21 @@ def gemm_emit_bf16(a: torch.Tensor, w: PackedWeight, residual: torch.Tensor, g: 
         raise ValueError(f"gemm: a [{M}, {K}], w {w.shape}, residual {tuple(residual.shape)}")
     L = _lib.load("tuned")
     lda, ldc = _ops._rows(a, "a"), _ops._rows(residual, "residual")
+    if M > MANY_ROWS_SPLIT_MAX:
+        # the product of many rows: its own epilogue leaves the row, or with K in two slices the kernel that adds them
+        # (sums of squares per tile of columns, or per 1,024 columns)
+        parts = L.apc_gemm_direct_emit_parts(a.data_ptr(), lda, residual.data_ptr(), ldc, M, N, K)
+        if not parts:
+            return None
+        raw = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
+        ss = torch.empty((M, parts), dtype=torch.float32, device=a.device)
+        ks = L.apc_gemm_direct_k_split(M, N, K)
+        ws = torch.empty(ks * M * N, dtype=torch.float32, device=a.device) if ks > 1 else None
+        _lib.check(L.apc_gemm_direct_emit_bf16(a.data_ptr(), lda, w.data.data_ptr(), residual.data_ptr(), ldc, M, N, K,
+                                               g.data_ptr(), raw.data_ptr(), N, ss.data_ptr(), parts,
+                                               ws.data_ptr() if ws is not None else 0, _ops._stream()),
+                   "gemm_direct_emit_bf16")
+        return raw, ss
     if M > SKINNY_MAX_ROWS:   # the tiled kernel: only where K is cut into slices (the finishing kernel leaves the row)
         ks = _tiled_k_split(M, N, K)
         if ks == 1:

@@ -240,7 +240,7 @@ _PRODUCTS = {
     "apc_skinny_gemm_bf16": ((2, 3, 4), 1), "apc_skinny_gemm_emit_bf16": ((2, 3, 4), 1),
     "apc_skinny_gemm_pre_bf16": ((3, 4, 5), 1), "apc_skinny_swiglu_bf16": ((2, 3, 4), 2),
     "apc_skinny_swiglu_pre_bf16": ((3, 4, 5), 2), "apc_gemm_bf16": ((2, 3, 4), 1), "apc_gemm_swiglu_bf16": ((2, 3, 4), 2),
-    "apc_gemm_splitk_emit_bf16": ((2, 3, 4), 1),
+    "apc_gemm_splitk_emit_bf16": ((2, 3, 4), 1), "apc_gemm_direct_emit_bf16": ((2, 3, 4), 1),
 }
 
 

@@ -237,6 +237,51 @@ def test_product_into_the_residual_leaves_the_next_norms_row_with_more_than_16_r
     check(f64(out), (f64(raw) @ f64(w2).T) * rstd, BF)
 
 
+@pytest.mark.parametrize("M,D,K,slices", [
+    # K in one piece: a part per tile of columns (tiles of 3 to 8 bands a wave; many columns in two launches, whole
+    # rounds of wide tiles and the rest), a last row tile of 76 and of 6 rows, columns that end inside a tile
+    (1100, 520, 1280, 1), (1030, 4096, 256, 1), (1100, 15000, 128, 1), (2048, 1028, 384, 1), (2048, 14336, 128, 1),
+    # K in two slices: a part per 1,024 columns
+    (1100, 1024, 4096, 2), (1030, 2500, 4608, 2)])
+def test_product_into_the_residual_leaves_the_next_norms_row_with_more_than_1024_rows(M, D, K, slices):
+    """From the product that loads its weights straight into registers: its epilogue adds into the residual, writes the
+    row times the next norm's weight and the rows' sums of squares over its tile of columns; with K in two slices the
+    kernel that adds the slices does.  Then the products behind the norm take what was left: one that stores, and
+    SwiGLU."""
+    t = tuned()
+    a, w = gen(M, K, seed=1, dtype=BF).to(DEV), gen(D, K, seed=2, dtype=BF).to(DEV)
+    res = gen(M, D, seed=3, scale=2.0).to(DEV)
+    res[0] *= 30.0
+    g = (1 + 0.2 * gen(D, seed=4)).to(DEV)
+    x, raw_want, ss_want = emit_reference(a, w, f64(res), g)
+    left = t.gemm_emit_bf16(a, pack(w), res, g)
+    assert left is not None
+    raw, ss = left
+    check(f64(res), x, torch.float32)
+    from allpaca_amd.kernels import lib
+    assert lib.load("tuned").apc_gemm_direct_k_split(M, D, K) == slices
+    assert ss.shape[0] == M and 1 <= ss.shape[1] <= 256 and tuple(raw.shape) == (M, D)
+    if slices > 1:
+        assert ss.shape[1] == -(-D // 1024)
+    assert np.allclose(f64(ss).sum(axis=1), (x ** 2).sum(axis=1), rtol=1e-5)
+    d = np.abs(f64(raw) - raw_want)
+    assert (d <= 2.0 ** -7 * np.abs(raw_want) + 1.5e-5 * np.abs(x).max()).all() and (d > 0).mean() < 0.01
+    if D % 128:
+        return       # no K for the product with the weights in registers
+    eps = 1e-5
+    rstd = 1.0 / np.sqrt((x ** 2).mean(axis=1, keepdims=True) + eps)
+    N2 = 264
+    w2 = gen(N2, D, seed=5, dtype=BF).to(DEV)
+    out = torch.empty(M, N2, dtype=BF, device=DEV)
+    assert t.gemm_pre_bf16(raw, ss, eps, pack(w2), out)
+    check(f64(out), (f64(raw) @ f64(w2).T) * rstd, BF)
+    F = 136
+    w3 = gen(2 * F, D, seed=6, dtype=BF).to(DEV)
+    out = torch.empty(M, F, dtype=BF, device=DEV)
+    assert t.swiglu_pre_bf16(raw, ss, eps, pack(w3[:F].contiguous()), pack(w3[F:].contiguous()), out)
+    check(f64(out), P.silu(f64(raw) @ f64(w3[:F]).T * rstd) * (f64(raw) @ f64(w3[F:]).T * rstd), BF)
+
+
 @pytest.mark.parametrize("M,N,K", [(40, 200, 1208), (64, 6144, 4096), (100, 96, 520), (128, 130, 2048),
                                    # K in one piece (enough tiles without slices): 224 and 192 tiles; a last row tile of 44
                                    (64, 28672, 520), (300, 8192, 264), (300, 2048, 1288),
