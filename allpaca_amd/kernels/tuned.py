@@ -331,9 +331,11 @@ KEY_RANGE_MIN = 2048
 def _key_splits(step, n_heads: int, window: int) -> int:
     """Into how many ranges of keys the 128-row attention kernel cuts every tile of this step: a block per (tile, head)
     leaves compute units idle when a step has few tiles (a chunk of 512 prompt tokens at 32 heads: 128 blocks for 256
-    units), so the keys are shared out until the chip has a block a unit, as long as a range keeps 2,048 keys
-    (measured at 8B shapes, 512 rows: 1.2 times as fast at 4,096 keys, 1.56 at 32,768, no gain at 2,048: a block's
-    start and the kernel that adds the ranges cost a few tiles of 64 keys).  1: no cutting."""
+    units), so the keys are shared out until the chip has a block a unit, as long as a range keeps KEY_RANGE_MIN keys
+    (measured at 8B shapes, 512 rows: 1.2 times as fast at 4,096 keys, 1.56 at 32,768, a loss at 2,048: a block's
+    start and the kernel that adds the ranges cost a few tiles of 64 keys), or half as many while the chip stays at
+    most half full (a block alone on its compute unit and its neighbours' runs at the pace of its own chain of loads:
+    128 rows over 2,048 keys in 2 ranges 1.27 times as fast, over 4,096 keys in 4 ranges 1.9 times).  1: no cutting."""
     blocks = step.n_tiles * n_heads
     pos0 = getattr(step, "host_pos0", None)
     rows = getattr(step, "host_rows", None)
@@ -342,7 +344,8 @@ def _key_splits(step, n_heads: int, window: int) -> int:
     keys = max([p + n for p, n in zip(pos0, rows) if n > 1] or [0])     # of the longest prompt in the step
     if window:
         keys = min(keys, window + 128)
-    return max(1, min(KEY_SPLITS_MAX, 256 // blocks, keys // KEY_RANGE_MIN))
+    few = min(keys // max(1, KEY_RANGE_MIN // 2), 128 // blocks)
+    return max(1, min(KEY_SPLITS_MAX, 256 // blocks, max(keys // KEY_RANGE_MIN, few)))
 
 
 def _pair_counters(device: torch.device, pairs: int) -> torch.Tensor:

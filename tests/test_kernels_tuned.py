@@ -608,7 +608,7 @@ def test_attention_of_whole_tiles_with_the_keys_cut_into_ranges(monkeypatch, ran
     (rows that see no key of a range), a key that dwarfs the others in the first and in a later range, 8 ranges."""
     nan = float("nan")
     monkeypatch.setattr(tuned(), "KEY_RANGE_MIN", range_min)
-    n = lambda keys, blocks: max(1, min(8, 256 // blocks, keys // range_min))
+    n = lambda keys, blocks: max(1, min(8, 256 // blocks, max(keys // range_min, min(keys // (range_min // 2), 128 // blocks))))
     run_attention(H=4, Hk=2, d=128, P_=16, lens=[1500, 200, 128], rows_per_seg=[300, 200, 100], seed=range_min, stale=nan,
                   ranges=n(1500, 6 * 4))
     run_attention(H=2, Hk=1, d=128, P_=32, lens=[2500], rows_per_seg=[130], seed=range_min + 1, ranges=n(2500, 2 * 2))
@@ -622,10 +622,13 @@ def test_attention_of_whole_tiles_with_the_keys_cut_into_ranges(monkeypatch, ran
 
 
 def test_attention_of_whole_tiles_with_the_keys_cut_into_ranges_at_the_size_from_which_it_is_done():
-    # 2,048 keys a range: 4,500 keys in 2 ranges, 17,000 in 8
-    run_attention(H=4, Hk=2, d=128, P_=16, lens=[4500], rows_per_seg=[100], seed=1, ranges=2)
+    # 1,024 keys a range while the cut leaves the chip at most half full: 4,500 keys in 4 ranges, 17,000 in 8, 1,000 whole;
+    # 2,048 keys a range where it fills the chip: 32 heads x 4 tiles over 4,200 keys in 2 ranges, over 4,000 whole
+    run_attention(H=4, Hk=2, d=128, P_=16, lens=[4500], rows_per_seg=[100], seed=1, ranges=4)
     run_attention(H=2, Hk=1, d=128, P_=64, lens=[17000], rows_per_seg=[129], seed=2, ranges=8)
-    run_attention(H=4, Hk=2, d=128, P_=16, lens=[4000], rows_per_seg=[100], seed=3, ranges=1)
+    run_attention(H=4, Hk=2, d=128, P_=16, lens=[1000], rows_per_seg=[100], seed=3, ranges=1)
+    run_attention(H=32, Hk=8, d=128, P_=16, lens=[4200], rows_per_seg=[512], seed=4, ranges=2)
+    run_attention(H=32, Hk=8, d=128, P_=16, lens=[4000], rows_per_seg=[512], seed=5, ranges=1)
 
 
 @pytest.mark.parametrize("d", [16, 64, 128, 192, 256])
