@@ -41,8 +41,9 @@
 //   masks but no maximum.  The three kinds of passes are three loops one after the other.
 // The MFMAs are written as instructions: the compiler does not know them, so it neither waits for their results
 // nor keeps reads behind them; the order of the slots keeps every read of a result at least one MFMA behind the
-// one that wrote it, and a wait stands at the end of the last pass of each loop, behind which the compiler may read
-// the accumulators (to write the rows, or to move them where the next loop keeps them).
+// one that wrote it, and a wait stands at the end of a block's last pass, behind which the compiler may read the
+// accumulators to write the rows (between the loops it leaves them where they are: no loop and no place between two
+// loops has a move of an accumulator, which is worth checking in the compiler's output after a change).
 // Positions outside a block's view that lie in stale slots are cleared in LDS before the value product sees them
 // (only tiles at the edge of a request's keys have any).
 // A step of few tiles (a chunk of 512 prompt tokens is 4 tiles x 32 heads = 128 blocks for 256 compute units) may have
@@ -625,7 +626,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     // ---- a pass of the loop.  Before pass i: S1(i) raw in s1, P0(i) in p0, the fragments of K(i + 1) and V(i) in kfr
     // and vfr (on their way from LDS).  MASKED: some row may not see some key of tile i (row tile 1) or tile i + 1 (row
     // tile 0), or tile i + 1 has stale positions.
-    auto pass = [&](auto MODE_, int i, int i_last) {  // i_last: the last pass of this kind in a row
+    auto pass = [&](auto MODE_, int i) {
       constexpr int MODE = decltype(MODE_)::value;
       constexpr bool MASKED = MODE != SOFT_SEEN;  // tiles at an edge, and the loads in one place
       const int t0 = t_begin + i * KT;
@@ -715,7 +716,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     // between two sets of registers in every pass.
     int i = 0;
     while (i < n_kt && !(all_seen(i) && __builtin_amdgcn_ballot_w64(st[0].m == -INFINITY || st[1].m == -INFINITY) == 0)) {
-      pass(std::integral_constant<int, SOFT_MASKED>{}, i, i);
+      pass(std::integral_constant<int, SOFT_MASKED>{}, i);
       ++i;
     }
     // (what the passes above saw, as one scalar: the loops below have no register to spare for the lanes' flags)
@@ -724,13 +725,13 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
       int i_end = i + 1;
       while (i_end < n_kt && all_seen(i_end)) ++i_end;
       st[0].sum = st[1].sum = 0.f;
-      for (; i < i_end; ++i) pass(std::integral_constant<int, SOFT_SEEN>{}, i, i_end - 1);
+      for (; i < i_end; ++i) pass(std::integral_constant<int, SOFT_SEEN>{}, i);
       st[0].l += halves_sum(st[0].sum);
       st[1].l += halves_sum(st[1].sum);
     }
     if (i < n_kt) {  // the rest: masks, but every row has its reference (the loop above began when all had)
       st[0].sum = st[1].sum = 0.f;
-      for (; i < n_kt; ++i) pass(std::integral_constant<int, SOFT_LATE>{}, i, n_kt - 1);
+      for (; i < n_kt; ++i) pass(std::integral_constant<int, SOFT_LATE>{}, i);
       st[0].l += halves_sum(st[0].sum);
       st[1].l += halves_sum(st[1].sum);
     }

@@ -33,7 +33,6 @@ enum { D_STORE_BF16 = 0, D_STORE_F32 = 1, D_ACC_F32 = 2, D_SWIGLU = 3, D_SWIGLU_
        D_STORE_BF16_PRE = 6 };
 __host__ __device__ constexpr bool is_swiglu(int mode) { return mode == D_SWIGLU || mode == D_SWIGLU_PRE; }
 __host__ __device__ constexpr bool is_pre(int mode) { return mode == D_SWIGLU_PRE || mode == D_STORE_BF16_PRE; }
-__host__ __device__ constexpr bool is_acc(int mode) { return mode == D_ACC_F32 || mode == D_ACC_EMIT; }
 
 // What goes with a norm folded into the product.  PRE: ss [M][parts] sums of x^2 of the rows (read), eps.
 // EMIT: g the norm's weight [N]; raw [M][ldr] takes bfloat16(x g); ss [M][parts] takes the sums of x^2 of the block's
