@@ -60,6 +60,7 @@
 #include "attention_wide.h"
 #include "mfma.h"
 #include <math.h>
+#include <mutex>
 #include <type_traits>
 
 namespace {
@@ -889,17 +890,21 @@ int launch_attn_prefill_wide(const bf16_t* q, int ldq, int q_off, bf16_t* out, i
   int lgP = 0;
   while ((1 << lgP) < page_tokens) ++lgP;
   static bool configured[64] = {};
+  static std::mutex configured_lock;
   const auto kernel = window > 0 ? attn_prefill_wide_kernel<true> : attn_prefill_wide_kernel<false>;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return (int)e;
   if (dev < 0 || dev >= 64) return APC_ERR_UNSUPPORTED;
-  if (!configured[dev]) {  // more LDS than a kernel gets without asking
-    for (const void* f : {(const void*)attn_prefill_wide_kernel<true>, (const void*)attn_prefill_wide_kernel<false>}) {
-      e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES + 16);
-      if (e != hipSuccess) return (int)e;
+  {  // more LDS than a kernel gets without asking: once per device
+    std::lock_guard<std::mutex> hold(configured_lock);
+    if (!configured[dev]) {
+      for (const void* f : {(const void*)attn_prefill_wide_kernel<true>, (const void*)attn_prefill_wide_kernel<false>}) {
+        e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES + 16);
+        if (e != hipSuccess) return (int)e;
+      }
+      configured[dev] = true;
     }
-    configured[dev] = true;
   }
   hipLaunchKernelGGL(kernel, dim3(n_tiles * H * n_splits), dim3(256), LDS_BYTES + 16, stream, q, ldq,
                      q_off, out, ldo, H, Hk, cache, lgP, block_table, max_blocks, positions, row_seg, tile_row0, tile_rows,
