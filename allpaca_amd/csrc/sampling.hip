@@ -1015,7 +1015,8 @@ APC_EXPORT int apc_sample_rows(const float* logits, int ldl, int n_rows, int V, 
     const hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;
   }
-  if (!scratch || n_rows > 65535 || dev < 0 || dev >= 64) {
+  // (a row's weights add up in 64 bits: 2^40 a candidate at most, so 2^22 candidates stay far inside)
+  if (!scratch || n_rows > 65535 || dev < 0 || dev >= 64 || V > (1 << 22)) {
     hipLaunchKernelGGL(sample_rows_kernel, dim3(n_rows), dim3(SNT), 0, stream, logits, ldl, V, temperature, top_k,
                        top_p, uniform, out);
     APC_LAUNCH_CHECK();
