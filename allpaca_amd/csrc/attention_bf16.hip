@@ -1,7 +1,7 @@
 // Attention over the paged cache in bfloat16 on MFMA, float32 softmax.
 //
 //   prefill kernels  a block takes up to 64 consecutive rows of one request x one head (half of a step's tile of up to
-//                    128 rows; tiles that are mostly whole, of heads of 128, go to attention_wide_bf16.hip, which
+//                    128 rows; tiles that are mostly whole, of heads of 128 or 64, go to attention_wide_bf16.hip, which
 //                    takes a whole tile a block); keys in tiles of 64 through LDS; online softmax.  Head sizes up to 128: v_mfma_f32_32x32x16_bf16, a wave takes
 //                    32 rows x half of each tile's keys (attn_prefill32_kernel; 98 us for 2,048 rows of 32 heads
 //                    of 128, 707 TFLOP/s at 32,768 rows).  Larger heads: v_mfma_f32_16x16x32_bf16, 16 rows a wave
@@ -911,7 +911,7 @@ APC_EXPORT int apc_attention_prefill_bf16(const void* q, int ldq, int q_off, voi
   if (attn_wide_takes(d, page_tokens) && (long)n_rows * 2 >= (long)n_tiles * TILE_ROWS)
     return launch_attn_prefill_wide((const bf16_t*)q, ldq, q_off, (bf16_t*)out, ldo, H, Hk, (const bf16_t*)cache,
                                     page_tokens, block_table, max_blocks, positions, row_seg, tile_row0, tile_rows,
-                                    n_tiles, window, scale, n_splits < 1 ? 1 : n_splits, part_rows, parts, stream);
+                                    n_tiles, window, scale, n_splits < 1 ? 1 : n_splits, part_rows, parts, d, stream);
   n_tiles *= 2;  // halves
   if ((long)n_tiles * H > 0x7fffffffL) return APC_ERR_BAD_ARG;
   dim3 grid(n_tiles * H), block(256);

@@ -1,5 +1,6 @@
-// Attention of prompt portions over the paged cache for a head size of 128: tiles of 128 rows, keys and values
-// straight from global memory into LDS, softmax and matrix products of one wave woven together by hand.
+// Attention of prompt portions over the paged cache for head sizes of 128 and 64: tiles of 128 rows, keys and values
+// straight from global memory into LDS, softmax and matrix products of one wave woven together by hand.  (The text
+// below gives the figures of a head size of 128; what a head size of 64 changes stands at its end.)
 //
 // A block of 4 waves takes up to 128 consecutive rows of one request and one head: wave (rh, kh) owns the rows
 // rh * 64 .. + 63 (two MFMA tiles of 32 rows, "row tiles") and the keys kh * 32 .. + 31 of every tile of 64 keys, with a
@@ -55,6 +56,14 @@
 // one moved into the other every pass); the direct loads of K in slot A (the general passes ran out of registers,
 // and the compiler's moves of accumulators read MFMA results too early); K and V fragments read for this pass only,
 // two steps ahead (same speed: the wave waits for LDS either way, see the counters in profiles/).
+// Heads of 64 (the kernel's parameter HD): half the fragments, MFMAs and direct loads a slot for the same softmax, whose
+// 16 steps a slot stand four to a pair of MFMAs instead of two; a row of K is 128 bytes, so a direct load brings 8 rows
+// and a piece lies at (piece index XOR (row / 2) % 8).  The registers and the 64 KiB of stages would let two blocks
+// share a compute unit; they must not: the kernel's waits are counted by hand for a wave that has its SIMD to itself,
+// and with two blocks a compute unit some heads' rows differed from run to run (2,048 rows over 8,192 keys: every run),
+// so the launch asks for more than half of a compute unit's LDS.  Measured at 32 heads, 2,048 rows over 32,768 keys:
+// 742 us (718 TFLOP/s; the 64-row kernels: 543), 2,048 rows over 2,048 keys 56 us; the softmax's vector instructions
+// bound it (118 of them beside 16 MFMAs in the short pass).
 // Formula: crates/allpaca-cpu/src/kernels.rs:293-356.  Reference kernel (contiguous K/V, no matrix cores):
 // attention_qtile_kernel hip/src/kernels.cpp:2203.
 #include "attention_wide.h"
@@ -62,19 +71,22 @@
 #include <math.h>
 #include <mutex>
 #include <type_traits>
+#include <utility>
 
 namespace {
 
 constexpr int KT = 64;                     // keys a tile
-constexpr int HD = ATTN_WIDE_HEAD;         // head size
 constexpr int STG = 4;                     // stages of K and of V in LDS
-constexpr int K_STAGE = KT * HD * 2;       // bytes: [64 rows][256]
-constexpr int V_STAGE = HD * KT * 2;       // bytes: [4 groups of 16 keys][128 elements][32]
-constexpr int V_BASE = STG * K_STAGE;
-constexpr int LDS_BYTES = STG * (K_STAGE + V_STAGE);  // of the stages; the block asks for 16 more
+// bytes of the stages for a head size of hd (the block asks for 16 more): K [64 rows][2 hd], V^T [4 groups of 16
+// keys][hd elements][32]
+constexpr int lds_bytes(int hd) { return STG * (KT * hd * 2 + hd * KT * 2); }
+// What a launch asks for: the stages, a flag behind them, and never less than 88 KiB, more than half of a compute
+// unit's 160 KiB, so that a block has its compute unit to itself.  The waits between the kernel's MFMAs and the
+// instructions around them are counted by hand for a wave that is alone on its SIMD: with two blocks of heads of 64 a
+// compute unit (their 64 KiB and registers would allow it) some heads' rows came out different from run to run.
+constexpr int lds_request(int hd) { return lds_bytes(hd) + 16 > 88 * 1024 ? lds_bytes(hd) + 16 : 88 * 1024; }
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float RISE = 64.f;               // by how much (in powers of 2) a score may exceed its row's reference
-constexpr int LOADS_PER_TILE = 8;          // a wave's direct loads per pass of the loop: 4 of K, 4 of V
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void* lds_ptr;
@@ -243,7 +255,8 @@ __device__ __forceinline__ void soft_any(int h, floatx16& s, Frag (&pf)[2], Soft
 }
 
 // WIN: the rows see a window of keys (without one, a row's first key is key 0, which costs no register)
-template <bool WIN>
+// HD: the head size, 128 or 64 (half the MFMAs a pass for the same softmax)
+template <int HD, bool WIN>
 __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     const bf16_t* __restrict__ q, int ldq, int q_off, bf16_t* __restrict__ out, int ldo, int H, int Hk,
     const bf16_t* __restrict__ cache, int lgP, const int* __restrict__ block_table, int max_blocks,
@@ -253,7 +266,12 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   const int window = WIN ? window_arg : 0;
   constexpr int d = HD;
-  constexpr int DT = d / 32;
+  constexpr int DT = d / 32;                 // tiles of 32 elements of a head; also a wave's direct loads per K or V tile
+  constexpr int NG = d / 16;                 // fragments of K, and of V, that a wave takes of a tile
+  constexpr int K_STAGE = KT * HD * 2, V_STAGE = HD * KT * 2, V_BASE = STG * K_STAGE, LDS_BYTES = lds_bytes(HD);
+  constexpr int LOADS_PER_TILE = 2 * DT;     // a wave's direct loads per pass of the loop
+  constexpr int ROW_BYTES = d * 2;           // of a row of K in LDS
+  constexpr int PPR = d / 8;                 // 16-byte pieces of such a row
   const int P = 1 << lgP;
   const int tid = threadIdx.x, lane = tid % WAVE, wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
   const int li = lane % 32, lh = lane / 32;
@@ -349,54 +367,74 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
   // gives back, so that none is negative).
   // (The lanes' offsets of the 4 loads of V differ by the same step, which goes into the loads' scalar offset: one
   // register instead of four.)
-  int koff[4];
+  // (Heads of 64: a row of K is 128 bytes, a load brings 8 of them, and a piece lies at piece ^ (row / 2) % 8, so that
+  // the rows r and r + 8, which share a place, differ in the half of the 256 bytes of banks they fall into.)
+  auto k_swizzle = [](int row) { return HD == 128 ? row % 16 : (row >> 1) & 7; };
+  int koff[DT];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int sw = 2 * (i & 1) + (i >> 1);
-    koff[i] = (4 * sw + lane / 16) * (d * 2) + (((lane % 16) ^ (lane / 16) ^ (4 * i)) * 16) + 3072 - i * 1024;
+  for (int i = 0; i < DT; ++i) {
+    if constexpr (HD == 128) {
+      const int sw = 2 * (i & 1) + (i >> 1);
+      koff[i] = (4 * sw + lane / 16) * (d * 2) + (((lane % 16) ^ (lane / 16) ^ (4 * i)) * 16) + 3072 - i * 1024;
+    } else {
+      const int row = 8 * i + lane / PPR;                       // LDS row among the wave's 16
+      const int g = row / 4, key = 4 * (2 * (g & 1) + (g >> 1)) + row % 4;
+      koff[i] = key * ROW_BYTES + (((lane % PPR) ^ k_swizzle(row)) * 16) + (DT - 1) * 1024 - i * 1024;
+    }
   }
-  const int voff = (lane % 32) * (P * 2) + (lane / 32) * 16 + 3072;
+  // (as scalars for the loads below: with the array itself named in them, the host's pass of the compiler left the
+  // kernel's launch stub out without a word)
+  const int koff0 = koff[0], koff1 = koff[1], koff2 = koff[DT > 2 ? 2 : 0], koff3 = koff[DT > 2 ? 3 : 0];
+  const int voff = (lane % 32) * (P * 2) + (lane / 32) * 16 + (DT - 1) * 1024;
   const int vstep = 32 * P * 2 - 1024;  // load i: elements 32 i .. of a page row of 2 P bytes, 1 KiB further in LDS
   auto group_of = [&](int j) { return min(t_begin + j * KT + 16 * wave, last16); };  // first key of the wave's 16
   auto page_of = [&](int j) { return __builtin_amdgcn_readfirstlane(bt[group_of(j) >> lgP]); };
-  const bf16_t* k_head_low = k_head - 1536;  // 3 KiB lower
-  const bf16_t* v_head_low = v_head - 1536;
+  const bf16_t* k_head_low = k_head - (DT - 1) * 512;  // 3 KiB lower (1 KiB with two loads a tile)
+  const bf16_t* v_head_low = v_head - (DT - 1) * 512;
   // one of the 4 loads of a tile's K or V (to stand between other work)
   auto k_load_piece = [&](int j, int page, int i) {
     const BufferRsrc kr = make_rsrc(k_head_low + (size_t)__builtin_amdgcn_readfirstlane(page) * page_stride);
     const int soff = (group_of(j) & (P - 1)) * (d * 2);
-    const lds_ptr dst = (lds_ptr)(smem + (j % STG) * K_STAGE + (16 * wave) * 256);
-    if (i == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[0], soff, 0, 0);
-    if (i == 1) __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[1], soff, 1024, 0);
-    if (i == 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[2], soff, 2048, 0);
-    if (i == 3) __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[3], soff, 3072, 0);
+    const lds_ptr dst = (lds_ptr)(smem + (j % STG) * K_STAGE + (16 * wave) * ROW_BYTES);
+    if (i == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff0, soff, 0, 0);
+    if (i == 1) __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff1, soff, 1024, 0);
+    if constexpr (DT > 2) {
+      if (i == 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff2, soff, 2048, 0);
+      if (i == 3) __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff3, soff, 3072, 0);
+    }
   };
   auto v_load_piece = [&](int j, int page, int i) {
     const BufferRsrc vr = make_rsrc(v_head_low + (size_t)__builtin_amdgcn_readfirstlane(page) * page_stride);
     const int soff = (group_of(j) & (P - 1)) * 2;
-    const lds_ptr dst = (lds_ptr)(smem + V_BASE + (j % STG) * V_STAGE + wave * 4096);
+    const lds_ptr dst = (lds_ptr)(smem + V_BASE + (j % STG) * V_STAGE + wave * (DT * 1024));
     if (i == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff, 0, 0);
     if (i == 1) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + vstep, 1024, 0);
-    if (i == 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + 2 * vstep, 2048, 0);
-    if (i == 3) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + 3 * vstep, 3072, 0);
+    if constexpr (DT > 2) {
+      if (i == 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + 2 * vstep, 2048, 0);
+      if (i == 3) __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + 3 * vstep, 3072, 0);
+    }
   };
   auto k_load = [&](int j, int page) {
     const BufferRsrc kr = make_rsrc(k_head_low + (size_t)__builtin_amdgcn_readfirstlane(page) * page_stride);
     const int soff = (group_of(j) & (P - 1)) * (d * 2);
-    const lds_ptr dst = (lds_ptr)(smem + (j % STG) * K_STAGE + (16 * wave) * 256);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[0], soff, 0, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[1], soff, 1024, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[2], soff, 2048, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff[3], soff, 3072, 0);
+    const lds_ptr dst = (lds_ptr)(smem + (j % STG) * K_STAGE + (16 * wave) * ROW_BYTES);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff0, soff, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff1, soff, 1024, 0);
+    if constexpr (DT > 2) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff2, soff, 2048, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, dst, 16, koff3, soff, 3072, 0);
+    }
   };
   auto v_load = [&](int j, int page) {
     const BufferRsrc vr = make_rsrc(v_head_low + (size_t)__builtin_amdgcn_readfirstlane(page) * page_stride);
     const int soff = (group_of(j) & (P - 1)) * 2;
-    const lds_ptr dst = (lds_ptr)(smem + V_BASE + (j % STG) * V_STAGE + wave * 4096);
+    const lds_ptr dst = (lds_ptr)(smem + V_BASE + (j % STG) * V_STAGE + wave * (DT * 1024));
     __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff, 0, 0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + vstep, 1024, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + 2 * vstep, 2048, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + 3 * vstep, 3072, 0);
+    if constexpr (DT > 2) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + 2 * vstep, 2048, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, dst, 16, voff, soff + 3 * vstep, 3072, 0);
+    }
   };
   // The same with the lanes' offsets worked out on the spot, for the passes that have no register to spare for them
   // (the compiler would otherwise keep them through the loop and spill something else)
@@ -405,20 +443,33 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     asm volatile("" : "+v"(ln));
     const BufferRsrc kr = make_rsrc(k_head_low + (size_t)__builtin_amdgcn_readfirstlane(pagek) * page_stride);
     const int ksoff = (group_of(jk) & (P - 1)) * (d * 2);
-    const lds_ptr kdst = (lds_ptr)(smem + (jk % STG) * K_STAGE + (16 * wave) * 256);
-    const int x = (ln / 16) * (d * 2) + (((ln % 16) ^ (ln / 16)) * 16);  // (row, place) of load 0; load i: place ^ 4 i
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, kdst, 16, x + 3072, ksoff, 0, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, kdst, 16, (x ^ 64) + 8 * (d * 2) + 2048, ksoff, 1024, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, kdst, 16, (x ^ 128) + 4 * (d * 2) + 1024, ksoff, 2048, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, kdst, 16, (x ^ 192) + 12 * (d * 2), ksoff, 3072, 0);
+    const lds_ptr kdst = (lds_ptr)(smem + (jk % STG) * K_STAGE + (16 * wave) * ROW_BYTES);
+    if constexpr (HD == 128) {
+      const int x = (ln / 16) * (d * 2) + (((ln % 16) ^ (ln / 16)) * 16);  // (row, place) of load 0; load i: place ^ 4 i
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, kdst, 16, x + 3072, ksoff, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, kdst, 16, (x ^ 64) + 8 * (d * 2) + 2048, ksoff, 1024, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, kdst, 16, (x ^ 128) + 4 * (d * 2) + 1024, ksoff, 2048, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, kdst, 16, (x ^ 192) + 12 * (d * 2), ksoff, 3072, 0);
+    } else {
+#pragma unroll
+      for (int i = 0; i < DT; ++i) {
+        const int row = 8 * i + ln / PPR;
+        const int g = row / 4, key = 4 * (2 * (g & 1) + (g >> 1)) + row % 4;
+        const int off = key * ROW_BYTES + (((ln % PPR) ^ k_swizzle(row)) * 16) + (DT - 1) * 1024 - i * 1024;
+        if (i == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, kdst, 16, off, ksoff, 0, 0);
+        else __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, kdst, 16, off, ksoff, 1024, 0);
+      }
+    }
     const BufferRsrc vr = make_rsrc(v_head_low + (size_t)__builtin_amdgcn_readfirstlane(pagev) * page_stride);
     const int vsoff = (group_of(jv) & (P - 1)) * 2;
-    const lds_ptr vdst = (lds_ptr)(smem + V_BASE + (jv % STG) * V_STAGE + wave * 4096);
-    const int vo = (ln % 32) * (P * 2) + (ln / 32) * 16 + 3072;
+    const lds_ptr vdst = (lds_ptr)(smem + V_BASE + (jv % STG) * V_STAGE + wave * (DT * 1024));
+    const int vo = (ln % 32) * (P * 2) + (ln / 32) * 16 + (DT - 1) * 1024;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, vdst, 16, vo, vsoff, 0, 0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, vdst, 16, vo, vsoff + vstep, 1024, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, vdst, 16, vo, vsoff + 2 * vstep, 2048, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, vdst, 16, vo, vsoff + 3 * vstep, 3072, 0);
+    if constexpr (DT > 2) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, vdst, 16, vo, vsoff + 2 * vstep, 2048, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, vdst, 16, vo, vsoff + 3 * vstep, 3072, 0);
+    }
   };
   // Stale positions of the V^T stage of tile j are cleared: what lies beyond the last key or in front of the first
   // one that a row of the block sees may be anything, and 0 x NaN is NaN.  (A group of 16 keys beyond the last one
@@ -426,8 +477,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
   auto clear_unseen = [&](int j) {
     const int t0 = t_begin + j * KT;
     unsigned char* stage = smem + V_BASE + (j % STG) * V_STAGE;
-    for (int idx = tid; idx < HD * 8; idx += 256) {  // piece idx: group idx / 256, half (idx % 64) / 32 of an element
-      const int t16 = t0 + 16 * (idx / 256), tg = t16 + 8 * ((idx % 64) / 32);
+    for (int idx = tid; idx < HD * 8; idx += 256) {  // piece idx: group idx / (2 HD), half (idx % 64) / 32 of an element
+      const int t16 = t0 + 16 * (idx / (HD * 2)), tg = t16 + 8 * ((idx % 64) / 32);
       Frag* piece = reinterpret_cast<Frag*>(stage + idx * 16);
       if (t16 > last16) {
         *piece = zero_frag();
@@ -449,23 +500,25 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
   const int lds0 = (int)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
   int kaddr[d / 16];
 #pragma unroll
-  for (int ks = 0; ks < d / 16; ++ks) kaddr[ks] = (kh * 32 + li) * 256 + ((((2 * ks) | lh) ^ (li % 16)) * 16);
-  const int vaddr = V_BASE + 2 * kh * 4096 + lane * 16;
+  for (int ks = 0; ks < d / 16; ++ks) kaddr[ks] = (kh * 32 + li) * ROW_BYTES + ((((2 * ks) | lh) ^ k_swizzle(li)) * 16);
+  const int vaddr = V_BASE + 2 * kh * (DT * 1024) + lane * 16;
   auto k_frag = [&](int stage_bytes, int ks) { return lds_frag<0>(lds0 + kaddr[ks] + stage_bytes); };
-  auto read_v_frags = [&](Frag (&vf)[8], int va) {
+  auto read_v_frags = [&](Frag (&vf)[NG], int va) {  // fragment g: the group of 16 keys g / DT, the elements 32 (g % DT) ..
     vf[0] = lds_frag<0>(va);
     vf[1] = lds_frag<1024>(va);
     vf[2] = lds_frag<2048>(va);
     vf[3] = lds_frag<3072>(va);
-    vf[4] = lds_frag<4096>(va);
-    vf[5] = lds_frag<5120>(va);
-    vf[6] = lds_frag<6144>(va);
-    vf[7] = lds_frag<7168>(va);
+    if constexpr (NG > 4) {
+      vf[4] = lds_frag<4096>(va);
+      vf[5] = lds_frag<5120>(va);
+      vf[6] = lds_frag<6144>(va);
+      vf[7] = lds_frag<7168>(va);
+    }
   };
   // the same through the compiler's own loads (the plain loop)
   auto k_frag_plain = [&](int stage_bytes, int ks) { return *reinterpret_cast<const Frag*>(smem + kaddr[ks] + stage_bytes); };
   auto v_frag_plain = [&](int stage_bytes, int g) {
-    return *reinterpret_cast<const Frag*>(smem + vaddr + stage_bytes + (g / 4) * 4096 + (g % 4) * 1024);
+    return *reinterpret_cast<const Frag*>(smem + vaddr + stage_bytes + g * 1024);
   };
 
   // The two key halves of a row half meet: wave kh = 1 leaves its reference, sum and O^T of row tile rt in LDS, wave
@@ -579,7 +632,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
       clear_unseen(0);
       __syncthreads();
     }
-    Frag kfr[8], vfr[8];  // the fragments of K(i + 1) and V(i) of this wave, in registers through a pass
+    Frag kfr[NG], vfr[NG];  // the fragments of K(i + 1) and V(i) of this wave, in registers through a pass
     {  // S(0) of both row tiles and the softmax of row tile 0, one thing after the other
       Frag kf[d / 16];
 #pragma unroll
@@ -596,7 +649,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int g = 0; g < 8; ++g) kfr[g] = k_frag(K_STAGE, g);
+      for (int g = 0; g < NG; ++g) kfr[g] = k_frag(K_STAGE, g);
       read_v_frags(vfr, lds0 + vaddr);
       asm volatile("s_nop 15\n\ts_nop 15");  // the MFMAs have left the matrix cores: their results may be read
       __builtin_amdgcn_sched_barrier(0);
@@ -630,27 +683,31 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
     auto pass = [&](auto MODE_, int i) {
       constexpr int MODE = decltype(MODE_)::value;
       constexpr bool MASKED = MODE != SOFT_SEEN;  // tiles at an edge, and the loads in one place
+      constexpr int SPG = 16 / NG;                // softmax steps (of 16 a slot) beside the two MFMAs of a step
       const int t0 = t_begin + i * KT;
       __builtin_amdgcn_sched_barrier(0);
       {  // slot A: the fragments have been asked for half a pass ago
         const int tk = t0 + kh * 32;
         const int va = lds0 + vaddr + (i % STG) * V_STAGE;
 #pragma unroll
-        for (int g = 0; g < 8; ++g) {
-#define SLOT_A_STEP(G)  /* slot B asked for K0 V0 K1 V1 .. K7 in this order, and V7 follows here behind the first  \
-                           MFMA (whose going out tells that the last MFMA of slot B has read V7's registers):      \
-                           behind read n, 15 - n may still be out */                                               \
-  if (g == G) {                                                                                   \
+        for (int g = 0; g < NG; ++g) {
+#define SOFT_STEPS(G, HALF, S_, P_, ST_) /* half of the SPG softmax steps that stand beside the two MFMAs of step G */ \
+  _Pragma("unroll") for (int q_ = 0; q_ < SPG / 2; ++q_)                                          \
+    soft_any<MODE>(SPG * G + HALF * (SPG / 2) + q_, S_, P_, ST_, tk, lh, sc2);
+#define SLOT_A_STEP(G)  /* slot B asked for K0 V0 K1 V1 .. K7 in this order (NG = 8), and V7 follows here behind the \
+                           first MFMA (whose going out tells that the last MFMA of slot B has read V7's           \
+                           registers): behind read n, 2 NG - 1 - n may still be out */                             \
+  if constexpr (G < NG) if (g == G) {                                                             \
     if (G == 0) {                                                                                 \
-      mfma_set<14>(s0, kfr[G], qf[0][G]);                                                         \
-      vfr[7] = lds_frag<4096 + 3072>(va);                                                         \
+      mfma_set<2 * NG - 2>(s0, kfr[G], qf[0][G]);                                                 \
+      vfr[NG - 1] = lds_frag<(NG - 1) * 1024>(va);                                                \
     } else {                                                                                      \
-      mfma_add<15 - 2 * G>(s0, kfr[G], qf[0][G]);                                                 \
+      mfma_add<2 * NG - 1 - 2 * G>(s0, kfr[G], qf[0][G]);                                         \
     }                                                                                             \
-    soft_any<MODE>(2 * G, s1, p1, st[1], tk, lh, sc2);                                            \
+    SOFT_STEPS(G, 0, s1, p1, st[1])                                                               \
     __builtin_amdgcn_sched_barrier(0);                                                            \
-    mfma_acc<14 - 2 * G>(o[0][G % 4], vfr[G], p0[G / 4]);                                         \
-    soft_any<MODE>(2 * G + 1, s1, p1, st[1], tk, lh, sc2);                                        \
+    mfma_acc<2 * NG - 2 - 2 * G>(o[0][G % DT], vfr[G], p0[G / DT]);                               \
+    SOFT_STEPS(G, 1, s1, p1, st[1])                                                               \
     __builtin_amdgcn_sched_barrier(0);                                                            \
   }
           SLOT_A_STEP(0) SLOT_A_STEP(1) SLOT_A_STEP(2) SLOT_A_STEP(3)
@@ -682,26 +739,27 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
         const int va = lds0 + vaddr + ((i + 1) % STG) * V_STAGE;
 #define SLOT_B_STEP(G)  /* a fragment's registers are free once the MFMA behind the one that read them has gone out; \
                            the direct loads of K(i + 5) and V(i + 4) go out one a step */                          \
-  {                                                                                                 \
+  if constexpr (G < NG) {                                                                           \
     if (G == 0) mfma_set<NO_WAIT>(s1, kfr[G], qf[1][G]);                                            \
     else mfma_add<NO_WAIT>(s1, kfr[G], qf[1][G]);                                                   \
-    if (G > 0) vfr[(G + 7) % 8] = lds_frag<(((G + 7) % 8) / 4) * 4096 + ((G + 7) % 4) * 1024>(va);  \
-    if (!MASKED && G < 4) k_load_piece(i + 5, kpg, G);                                              \
-    if (!MASKED && G >= 4) v_load_piece(i + 4, vpg, G - 4);                                         \
-    soft_any<MODE>(2 * G, s0, p0, st[0], tk, lh, sc2);                                              \
+    if constexpr (G > 0) vfr[G - 1] = lds_frag<(G > 0 ? G - 1 : 0) * 1024>(va);                     \
+    if (!MASKED && G < DT) k_load_piece(i + 5, kpg, G);                                             \
+    if (!MASKED && G >= DT) v_load_piece(i + 4, vpg, G - DT);                                       \
+    SOFT_STEPS(G, 0, s0, p0, st[0])                                                                 \
     __builtin_amdgcn_sched_barrier(0);                                                              \
-    mfma_acc<NO_WAIT>(o[1][G % 4], vfr[G], p1[G / 4]);                                              \
+    mfma_acc<NO_WAIT>(o[1][G % DT], vfr[G], p1[G / DT]);                                            \
     kfr[G] = k_frag(stage_k, G);                                                                    \
-    if (!MASKED && G == 7) {                                                                        \
+    if (!MASKED && G == NG - 1) {                                                                   \
       vpg = kpg;                                                                                    \
       kpg = page_of(i + 6);                                                                         \
     }                                                                                               \
-    soft_any<MODE>(2 * G + 1, s0, p0, st[0], tk, lh, sc2);                                          \
+    SOFT_STEPS(G, 1, s0, p0, st[0])                                                                 \
     __builtin_amdgcn_sched_barrier(0);                                                              \
   }
         SLOT_B_STEP(0) SLOT_B_STEP(1) SLOT_B_STEP(2) SLOT_B_STEP(3)
         SLOT_B_STEP(4) SLOT_B_STEP(5) SLOT_B_STEP(6) SLOT_B_STEP(7)
 #undef SLOT_B_STEP
+#undef SOFT_STEPS
       }
       // The last MFMAs must have left the matrix cores before O is read.  The compiler does not know these
       // instructions: it reads the accumulators right behind the loop, in front of any wait that stands there.
@@ -814,7 +872,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
 #pragma unroll
         for (int w = 0; w < 4; ++w) pf.w[w] = pack_bf16x2(s[8 * jj + 2 * w], s[8 * jj + 2 * w + 1]);
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) o[dt] = mfma32(v_frag_plain(stage_v, jj * 4 + dt), pf, o[dt]);
+        for (int dt = 0; dt < DT; ++dt) o[dt] = mfma32(v_frag_plain(stage_v, jj * DT + dt), pf, o[dt]);
       }
     }
     __syncthreads();
@@ -831,8 +889,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
 __global__ __launch_bounds__(256) void attn_wide_merge_kernel(const float* __restrict__ parts, int n_splits, int part_rows,
                                                               int H, const int* __restrict__ tile_row0,
                                                               const int* __restrict__ tile_rows, bf16_t* __restrict__ out,
-                                                              int ldo) {
-  constexpr int d = HD;
+                                                              int ldo, int d) {
   const int tile = blockIdx.x / ATTN_WIDE_ROWS, r = blockIdx.x % ATTN_WIDE_ROWS;
   const int hq = blockIdx.y * 256 + threadIdx.x;
   if (r >= tile_rows[tile] || hq >= H * (d / 4)) return;
@@ -874,15 +931,15 @@ __global__ __launch_bounds__(256) void attn_wide_merge_kernel(const float* __res
 }  // namespace
 
 bool attn_wide_takes(int d, int page_tokens) {
-  return d == ATTN_WIDE_HEAD && page_tokens >= 16 && (page_tokens & (page_tokens - 1)) == 0;
+  return (d == 128 || d == 64) && page_tokens >= 16 && (page_tokens & (page_tokens - 1)) == 0;
 }
 
 int launch_attn_prefill_wide(const bf16_t* q, int ldq, int q_off, bf16_t* out, int ldo, int H, int Hk,
                              const bf16_t* cache, int page_tokens, const int* block_table, int max_blocks,
                              const int* positions, const int* row_seg, const int* tile_row0, const int* tile_rows,
                              int n_tiles, int window, float scale, int n_splits, int part_rows, float* parts,
-                             hipStream_t stream) {
-  if (!attn_wide_takes(ATTN_WIDE_HEAD, page_tokens)) return APC_ERR_UNSUPPORTED;
+                             int d, hipStream_t stream) {
+  if (!attn_wide_takes(d, page_tokens)) return APC_ERR_UNSUPPORTED;
   if (n_splits < 1 || n_splits > 8 || (n_splits > 1 && (!parts || part_rows <= 0)) ||
       (long)n_tiles * H * n_splits > 0x7fffffffL)
     return APC_ERR_BAD_ARG;
@@ -891,7 +948,9 @@ int launch_attn_prefill_wide(const bf16_t* q, int ldq, int q_off, bf16_t* out, i
   while ((1 << lgP) < page_tokens) ++lgP;
   static bool configured[64] = {};
   static std::mutex configured_lock;
-  const auto kernel = window > 0 ? attn_prefill_wide_kernel<true> : attn_prefill_wide_kernel<false>;
+  const auto kernel = d == 128 ? (window > 0 ? attn_prefill_wide_kernel<128, true> : attn_prefill_wide_kernel<128, false>)
+                               : (window > 0 ? attn_prefill_wide_kernel<64, true> : attn_prefill_wide_kernel<64, false>);
+  const int lds = lds_request(d);
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return (int)e;
@@ -899,21 +958,24 @@ int launch_attn_prefill_wide(const bf16_t* q, int ldq, int q_off, bf16_t* out, i
   {  // more LDS than a kernel gets without asking: once per device
     std::lock_guard<std::mutex> hold(configured_lock);
     if (!configured[dev]) {
-      for (const void* f : {(const void*)attn_prefill_wide_kernel<true>, (const void*)attn_prefill_wide_kernel<false>}) {
-        e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES + 16);
+      const std::pair<const void*, int> instances[] = {
+          {(const void*)attn_prefill_wide_kernel<128, true>, 128}, {(const void*)attn_prefill_wide_kernel<128, false>, 128},
+          {(const void*)attn_prefill_wide_kernel<64, true>, 64}, {(const void*)attn_prefill_wide_kernel<64, false>, 64}};
+      for (const auto& [f, hd] : instances) {
+        e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, lds_request(hd));
         if (e != hipSuccess) return (int)e;
       }
       configured[dev] = true;
     }
   }
-  hipLaunchKernelGGL(kernel, dim3(n_tiles * H * n_splits), dim3(256), LDS_BYTES + 16, stream, q, ldq,
+  hipLaunchKernelGGL(kernel, dim3(n_tiles * H * n_splits), dim3(256), lds, stream, q, ldq,
                      q_off, out, ldo, H, Hk, cache, lgP, block_table, max_blocks, positions, row_seg, tile_row0, tile_rows,
                      n_tiles, window, scale, n_splits, part_rows, parts);
   APC_LAUNCH_CHECK();
   if (n_splits > 1) {
-    hipLaunchKernelGGL(attn_wide_merge_kernel, dim3(n_tiles * ATTN_WIDE_ROWS, ceil_div(H * (ATTN_WIDE_HEAD / 4), 256)),
+    hipLaunchKernelGGL(attn_wide_merge_kernel, dim3(n_tiles * ATTN_WIDE_ROWS, ceil_div(H * (d / 4), 256)),
                        dim3(256), 0, stream, parts, n_splits,
-                       part_rows, H, tile_row0, tile_rows, out, ldo);
+                       part_rows, H, tile_row0, tile_rows, out, ldo, d);
     APC_LAUNCH_CHECK();
   }
   return 0;

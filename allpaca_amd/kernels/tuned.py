@@ -318,7 +318,7 @@ WHOLE_WAVES = 4   # waves of such a block (NW in attention_bf16.hip)
 # With fewer pairs: the blocks of a pair leave one partial result each and the one that finishes last adds them (no
 # second kernel), where the sizes allow; False: partial results per wave and a kernel that merges them.
 LAST_BLOCK_MERGES = True
-# Portions whose tiles of 128 rows are mostly whole (heads of 128, pages of a power of two from 16 on) run on the kernel
+# Portions whose tiles of 128 rows are mostly whole (heads of 128 or 64, pages of a power of two from 16 on) run on the kernel
 # that takes such a tile a block (attention_wide_bf16.hip); False sends every portion to the kernels of 64-row blocks.
 WIDE_TILES = True
 _counters: dict = {}

@@ -565,43 +565,48 @@ def test_attention_windows_with_large_heads(d, window, decode_path):
 
 
 @pytest.mark.parametrize("P_", [16, 32, 64, 128])
-def test_attention_of_whole_tiles_of_128_rows(P_):
-    """Heads of 128 in portions that fill tiles of 128 rows: the kernel that takes such a tile a block (keys and values
+@pytest.mark.parametrize("d", [128, 64])
+def test_attention_of_whole_tiles_of_128_rows(P_, d):
+    """Heads of 128 and of 64 in portions that fill tiles of 128 rows: the kernel that takes such a tile a block (keys and values
     by direct loads into LDS, one page per 16 keys).  Several requests, history in front of a portion, rows and keys
     that are no multiple of a tile, one and several key tiles, every page size it takes."""
-    run_attention(H=4, Hk=2, d=128, P_=P_, lens=[640, 300, 128], rows_per_seg=[384, 300, 128], seed=P_)
-    run_attention(H=8, Hk=8, d=128, P_=P_, lens=[1000, 257, 1], rows_per_seg=[250, 257, 1], seed=P_ + 1)
-    run_attention(H=2, Hk=1, d=128, P_=P_, lens=[2500], rows_per_seg=[2500 - 1277], seed=P_ + 2)
+    run_attention(H=4, Hk=2, d=d, P_=P_, lens=[640, 300, 128], rows_per_seg=[384, 300, 128], seed=P_)
+    run_attention(H=8, Hk=8, d=d, P_=P_, lens=[1000, 257, 1], rows_per_seg=[250, 257, 1], seed=P_ + 1)
+    run_attention(H=2, Hk=1, d=d, P_=P_, lens=[2500], rows_per_seg=[2500 - 1277], seed=P_ + 2)
 
 
-def test_attention_of_whole_tiles_at_the_head_counts_of_an_8b_model():
+@pytest.mark.parametrize("d", [128, 64])
+def test_attention_of_whole_tiles_at_the_head_counts_of_an_8b_model(d):
     # 32 heads over 8 kv heads (heads of a kv head share an XCD in the kernel's order of blocks); portions that end in
     # a short tile, that begin at position 0 and deep inside a sequence, and one of a single tile
-    run_attention(H=32, Hk=8, d=128, P_=16, lens=[700, 129, 4100, 128], rows_per_seg=[700, 129, 300, 70], seed=3)
+    run_attention(H=32, Hk=8, d=d, P_=16, lens=[700, 129, 4100, 128], rows_per_seg=[700, 129, 300, 70], seed=3)
     # tiles of 64 rows on average: still the 128-row kernel; one row less on average: the 64-row kernels take over
-    run_attention(H=8, Hk=2, d=128, P_=16, lens=[300, 300, 500], rows_per_seg=[64, 64, 64], seed=4)
-    run_attention(H=8, Hk=2, d=128, P_=16, lens=[300, 300, 500], rows_per_seg=[64, 63, 64], seed=5)
+    run_attention(H=8, Hk=2, d=d, P_=16, lens=[300, 300, 500], rows_per_seg=[64, 64, 64], seed=4)
+    run_attention(H=8, Hk=2, d=d, P_=16, lens=[300, 300, 500], rows_per_seg=[64, 63, 64], seed=5)
 
 
 @pytest.mark.parametrize("window", [1, 37, 128, 200, 1000])
-def test_attention_of_whole_tiles_with_windows(window):
+@pytest.mark.parametrize("d", [128, 64])
+def test_attention_of_whole_tiles_with_windows(window, d):
     # windows that end inside the first key tile, that span several, that are wider than the keys; pages in front of
     # the window given back (the spare page, full of NaN, stands in); NaN beyond the last key
-    run_attention(H=4, Hk=2, d=128, P_=16, lens=[900, 260], rows_per_seg=[500, 260], window=window, seed=window,
+    run_attention(H=4, Hk=2, d=d, P_=16, lens=[900, 260], rows_per_seg=[500, 260], window=window, seed=window,
                   stale=float("nan"))
-    run_attention(H=2, Hk=2, d=128, P_=32, lens=[700], rows_per_seg=[300], window=window, seed=window + 1,
+    run_attention(H=2, Hk=2, d=d, P_=32, lens=[700], rows_per_seg=[300], window=window, seed=window + 1,
                   stale=float("nan"))
 
 
 @pytest.mark.parametrize("where", [3, 200, 519, 700])
-def test_attention_of_whole_tiles_when_a_late_key_dwarfs_the_first(where):
+@pytest.mark.parametrize("d", [128, 64])
+def test_attention_of_whole_tiles_when_a_late_key_dwarfs_the_first(where, d):
     """The kernel for tiles of 128 rows keeps a row's first reference for its exponents; a key whose scores lie far
     beyond it (here by hundreds of powers of two) sends the block to its plain loop, whose references move."""
-    run_attention(H=4, Hk=2, d=128, P_=16, lens=[768], rows_per_seg=[512], seed=where, loud=(0, where, 40.0))
+    run_attention(H=4, Hk=2, d=d, P_=16, lens=[768], rows_per_seg=[512], seed=where, loud=(0, where, 40.0))
 
 
 @pytest.mark.parametrize("range_min", [64, 192, 512])
-def test_attention_of_whole_tiles_with_the_keys_cut_into_ranges(monkeypatch, range_min):
+@pytest.mark.parametrize("d", [128, 64])
+def test_attention_of_whole_tiles_with_the_keys_cut_into_ranges(monkeypatch, range_min, d):
     """A step of few tiles over many keys: the keys of every tile are cut into ranges, a block each, and a second
     kernel adds the ranges.  With the smallest range set low so that modest sizes are cut: requests whose tiles have
     very different numbers of keys (some fewer key tiles than ranges: empty ranges), NaN beyond the last key, windows
@@ -609,26 +614,53 @@ def test_attention_of_whole_tiles_with_the_keys_cut_into_ranges(monkeypatch, ran
     nan = float("nan")
     monkeypatch.setattr(tuned(), "KEY_RANGE_MIN", range_min)
     n = lambda keys, blocks: max(1, min(8, 256 // blocks, max(keys // range_min, min(keys // (range_min // 2), 128 // blocks))))
-    run_attention(H=4, Hk=2, d=128, P_=16, lens=[1500, 200, 128], rows_per_seg=[300, 200, 100], seed=range_min, stale=nan,
+    run_attention(H=4, Hk=2, d=d, P_=16, lens=[1500, 200, 128], rows_per_seg=[300, 200, 100], seed=range_min, stale=nan,
                   ranges=n(1500, 6 * 4))
-    run_attention(H=2, Hk=1, d=128, P_=32, lens=[2500], rows_per_seg=[130], seed=range_min + 1, ranges=n(2500, 2 * 2))
-    run_attention(H=4, Hk=2, d=128, P_=16, lens=[1900, 700], rows_per_seg=[250, 128], window=700, seed=range_min + 2,
+    run_attention(H=2, Hk=1, d=d, P_=32, lens=[2500], rows_per_seg=[130], seed=range_min + 1, ranges=n(2500, 2 * 2))
+    run_attention(H=4, Hk=2, d=d, P_=16, lens=[1900, 700], rows_per_seg=[250, 128], window=700, seed=range_min + 2,
                   stale=nan, ranges=n(828, 3 * 4))
-    run_attention(H=4, Hk=2, d=128, P_=16, lens=[1900], rows_per_seg=[128], window=150, seed=range_min + 3, stale=nan,
+    run_attention(H=4, Hk=2, d=d, P_=16, lens=[1900], rows_per_seg=[128], window=150, seed=range_min + 3, stale=nan,
                   ranges=n(278, 4))
     for where in (3, 1100, 1499):
-        run_attention(H=4, Hk=2, d=128, P_=16, lens=[1500], rows_per_seg=[256], seed=range_min + where,
+        run_attention(H=4, Hk=2, d=d, P_=16, lens=[1500], rows_per_seg=[256], seed=range_min + where,
                       loud=(0, where, 40.0), ranges=n(1500, 2 * 4))
 
 
-def test_attention_of_whole_tiles_with_the_keys_cut_into_ranges_at_the_size_from_which_it_is_done():
+@pytest.mark.parametrize("d", [128, 64])
+def test_attention_of_whole_tiles_with_the_keys_cut_into_ranges_at_the_size_from_which_it_is_done(d):
     # 1,024 keys a range while the cut leaves the chip at most half full: 4,500 keys in 4 ranges, 17,000 in 8, 1,000 whole;
     # 2,048 keys a range where it fills the chip: 32 heads x 4 tiles over 4,200 keys in 2 ranges, over 4,000 whole
-    run_attention(H=4, Hk=2, d=128, P_=16, lens=[4500], rows_per_seg=[100], seed=1, ranges=4)
-    run_attention(H=2, Hk=1, d=128, P_=64, lens=[17000], rows_per_seg=[129], seed=2, ranges=8)
-    run_attention(H=4, Hk=2, d=128, P_=16, lens=[1000], rows_per_seg=[100], seed=3, ranges=1)
-    run_attention(H=32, Hk=8, d=128, P_=16, lens=[4200], rows_per_seg=[512], seed=4, ranges=2)
-    run_attention(H=32, Hk=8, d=128, P_=16, lens=[4000], rows_per_seg=[512], seed=5, ranges=1)
+    run_attention(H=4, Hk=2, d=d, P_=16, lens=[4500], rows_per_seg=[100], seed=1, ranges=4)
+    run_attention(H=2, Hk=1, d=d, P_=64, lens=[17000], rows_per_seg=[129], seed=2, ranges=8)
+    run_attention(H=4, Hk=2, d=d, P_=16, lens=[1000], rows_per_seg=[100], seed=3, ranges=1)
+    run_attention(H=32, Hk=8, d=d, P_=16, lens=[4200], rows_per_seg=[512], seed=4, ranges=2)
+    run_attention(H=32, Hk=8, d=d, P_=16, lens=[4000], rows_per_seg=[512], seed=5, ranges=1)
+
+
+@pytest.mark.parametrize("d", [128, 64])
+def test_attention_of_whole_tiles_gives_the_same_bits_every_time(d):
+    """The kernel for tiles of 128 rows counts the waits around its MFMAs by hand, for a wave that has its SIMD to
+    itself; sharing a compute unit with a second block showed as rows that differ from run to run.  More blocks than
+    compute units, many times: every output equals the first bit by bit (which the other tests hold against the plain
+    implementation at smaller sizes)."""
+    from allpaca_amd.engine.batch import Entry, pack_step
+    from allpaca_amd.kernels import ops as kernel_ops
+    t = tuned()
+    H, Hk, P_, keys, rows = 32, 8, 16, 6144, 2048
+    cache, bt, ks, vs = make_cache([keys], Hk, d, P_, BF, seed=d)
+    tables = [[list(bt[0, : keys // P_].cpu().numpy())]]
+    spare = min(set(range(cache.shape[0])) - {int(p) for p in tables[0][0]})
+    step = pack_step([Entry(0, [0] * rows, [])], [keys - rows], [0], tables, torch.device(DEV), [spare],
+                     tile_rows=kernel_ops.attention_tile_rows(BF))
+    q = gen(rows, H * d, seed=d + 1, scale=2.5, dtype=BF).to(DEV)
+    outs = [torch.zeros(rows, H * d, dtype=BF, device=DEV) for _ in range(24)]
+    for o in outs:
+        assert t.attention_bf16(q, 0, o, H, Hk, d, cache, P_, step.block_tables[0], step)
+    first = outs[0].view(torch.int16)
+    differ = [i for i, o in enumerate(outs) if not torch.equal(o.view(torch.int16), first)]
+    assert not differ, f"runs {differ} differ from the first"
+    want = P.attention(f64(q[-3:]).reshape(3, H, d), f64(ks[0]), f64(vs[0]), H, Hk)
+    assert np.abs(f64(outs[0][-3:]).reshape(3, H, d) - want).max() < 2.0 ** -7 * np.abs(f64(vs[0])).max() * 0.25 + 2.0 ** -8 * np.abs(want).max()
 
 
 @pytest.mark.parametrize("d", [16, 64, 128, 192, 256])
