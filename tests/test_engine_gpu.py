@@ -316,8 +316,10 @@ def test_widths_of_an_8b_model_against_the_plain_implementation_and_between_the_
     assert worst < 0.03 and worst < 2.0 * mean, errs
 
 
-def test_a_long_prompt_at_the_widths_of_an_8b_model_in_portions_of_512_and_128():
-    """Two layers at the widths of Llama-3.1-8B, a prompt of 4,500 tokens: in steps of 2,048 rows (a block of the
+@pytest.mark.parametrize("widths", ["llama-3.1-8b", "llama-3.2-1b"])
+def test_a_long_prompt_at_the_widths_of_a_real_model_in_portions_of_512_and_128(widths):
+    """Two layers at the widths of Llama-3.1-8B (heads of 128) and of Llama-3.2-1B (heads of 64, the head tied to the
+    embedding), a prompt of 4,500 tokens: in steps of 2,048 rows (a block of the
     attention kernel per tile of 128 rows and head, but for the last step's 404 rows), in steps of 512 and of 128 rows
     (from 4,096 keys on the keys of a tile are cut into ranges for several blocks and a second kernel adds them) and
     in 32-bit: the logits of the rows
@@ -330,7 +332,7 @@ def test_a_long_prompt_at_the_widths_of_an_8b_model_in_portions_of_512_and_128()
     from allpaca_amd.parts import Runtime
     from allpaca_amd.weights import random_tensors
     V, T = 8200, 4500
-    cfg_json = dict(preset("llama-3.1-8b"), num_hidden_layers=2, vocab_size=V)
+    cfg_json = dict(preset(widths), num_hidden_layers=2, vocab_size=V)
     sharpen = (3.0 / (0.02 ** 2 * cfg_json["hidden_size"])) ** 0.5
 
     def runner(dtype):
