@@ -61,7 +61,10 @@
 // and a piece lies at (piece index XOR (row / 2) % 8).  The registers and the 64 KiB of stages would let two blocks
 // share a compute unit; they must not: the kernel's waits are counted by hand for a wave that has its SIMD to itself,
 // and with two blocks a compute unit some heads' rows differed from run to run (2,048 rows over 8,192 keys: every run),
-// so the launch asks for more than half of a compute unit's LDS.  Measured at 32 heads, 2,048 rows over 32,768 keys:
+// so the launch asks for more than half of a compute unit's LDS.  (What fails there is the wait in the middle of a
+// pass that leaves the newest direct loads on their way: with every direct load waited for, two blocks a compute
+// unit gave the same bits in 340 runs, at 657 us for the shape below.  Why the partial wait does not hold beside a
+// second block is not understood, so that is not what runs.)  Measured at 32 heads, 2,048 rows over 32,768 keys:
 // 742 us (718 TFLOP/s; the 64-row kernels: 543), 2,048 rows over 2,048 keys 56 us; the softmax's vector instructions
 // bound it (118 of them beside 16 MFMAs in the short pass).
 // Formula: crates/allpaca-cpu/src/kernels.rs:293-356.  Reference kernel (contiguous K/V, no matrix cores):
