@@ -297,10 +297,12 @@ def swiglu_pre_bf16(raw: torch.Tensor, ss: torch.Tensor, eps: float, wg: PackedW
 
 def _keys_per_part(n_rows: int, n_kv_heads: int, max_context: int, page_tokens: int = 16) -> int:
     """Keys one wave covers in the decode kernel.  A wave that walks through many keys overlaps its loads
-    with its work, so: the longest range that still leaves about a thousand waves on the chip (four per
-    compute unit), at least 64 keys, and no more pages than a wave keeps ids for (one per lane)."""
+    with its work, so: the longest range that still leaves 768 waves on the chip (three per compute unit; measured
+    at 8B shapes with 1 to 24 rows over 2,048 to 32,768 keys: the best choice of 64 .. 512 keys in every case, where
+    a thousand waves chose half the range at 12 and 24 rows and lost 9 and 12 %), at least 64 keys, and no more pages
+    than a wave keeps ids for (one per lane)."""
     kw = 64
-    while (kw < 1024 and n_rows * n_kv_heads * (-(-max_context // (kw * 2))) >= 1024
+    while (kw < 1024 and n_rows * n_kv_heads * (-(-max_context // (kw * 2))) >= 768
            and (kw * 2) // page_tokens + 2 <= 64):
         kw *= 2
     while kw > 32 and kw // page_tokens + 2 > 64:

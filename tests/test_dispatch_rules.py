@@ -69,3 +69,15 @@ def test_what_the_sampler_tells_the_kernels(monkeypatch, rules, want):
     params = [GenerationParams(max_tokens=1, temperature=t, top_k=k, top_p=p) for t, k, p in rules]
     s.launch(torch.zeros(len(rules), 16), params, [0] * len(rules))
     assert (seen["any_top_k"], seen["any_top_p"], seen["few_after_top_k"]) == want
+
+
+def test_keys_a_wave_of_the_decode_attention_takes():
+    """The longest range of keys that leaves 768 waves on the chip, from 64 keys on; never more pages than a wave
+    keeps ids for."""
+    from allpaca_amd.kernels import tuned as t
+    got = {(n, ctx): t._keys_per_part(n, 8, ctx, 16) for n, ctx in
+           [(1, 2048), (4, 2048), (8, 2048), (12, 2048), (16, 2048), (24, 2048), (8, 8192), (16, 8192), (1, 32768)]}
+    assert got == {(1, 2048): 64, (4, 2048): 64, (8, 2048): 128, (12, 2048): 256, (16, 2048): 256, (24, 2048): 512,
+                   (8, 8192): 512, (16, 8192): 512, (1, 32768): 256}
+    assert t._keys_per_part(16, 8, 1 << 20, 16) // 16 + 2 <= 64 and t._keys_per_part(16, 8, 1 << 20, 128) == 1024
+    assert t._keys_per_part(1, 1, 10, 16) == 64
