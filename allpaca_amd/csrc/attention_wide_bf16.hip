@@ -58,15 +58,14 @@
 // two steps ahead (same speed: the wave waits for LDS either way, see the counters in profiles/).
 // Heads of 64 (the kernel's parameter HD): half the fragments, MFMAs and direct loads a slot for the same softmax, whose
 // 16 steps a slot stand four to a pair of MFMAs instead of two; a row of K is 128 bytes, so a direct load brings 8 rows
-// and a piece lies at (piece index XOR (row / 2) % 8).  The registers and the 64 KiB of stages would let two blocks
-// share a compute unit; they must not: the kernel's waits are counted by hand for a wave that has its SIMD to itself,
-// and with two blocks a compute unit some heads' rows differed from run to run (2,048 rows over 8,192 keys: every run),
-// so the launch asks for more than half of a compute unit's LDS.  (What fails there is the wait in the middle of a
-// pass that leaves the newest direct loads on their way: with every direct load waited for, two blocks a compute
-// unit gave the same bits in 340 runs, at 657 us for the shape below.  Why the partial wait does not hold beside a
-// second block is not understood, so that is not what runs.)  Measured at 32 heads, 2,048 rows over 32,768 keys:
-// 742 us (718 TFLOP/s; the 64-row kernels: 543), 2,048 rows over 2,048 keys 56 us; the softmax's vector instructions
-// bound it (118 of them beside 16 MFMAs in the short pass).
+// and a piece lies at (piece index XOR (row / 2) % 8).  Its 64 KiB of stages and 256 registers a lane (the kernel is
+// compiled for two waves a SIMD at this head size) let two blocks share a compute unit, one's softmax beside the
+// other's MFMAs.  Measured at 32 heads, 2,048 rows over 32,768 keys: 643 us (828 TFLOP/s; one block a compute unit:
+// 742 us; the 64-row kernels: 543 TFLOP/s), 2,048 rows over 2,048 keys 49 us; the softmax's vector instructions bound
+// it (118 of them beside 16 MFMAs in the short pass).
+// (Two blocks a compute unit once gave rows that differed from run to run; the cause was two LDS reads without a
+// taker, see lds_frag below, not the waits on the direct loads: with those reads gone the same waits give equal
+// bits with two blocks a compute unit.)
 // Formula: crates/allpaca-cpu/src/kernels.rs:293-356.  Reference kernel (contiguous K/V, no matrix cores):
 // attention_qtile_kernel hip/src/kernels.cpp:2203.
 #include "attention_wide.h"
@@ -83,11 +82,9 @@ constexpr int STG = 4;                     // stages of K and of V in LDS
 // bytes of the stages for a head size of hd (the block asks for 16 more): K [64 rows][2 hd], V^T [4 groups of 16
 // keys][hd elements][32]
 constexpr int lds_bytes(int hd) { return STG * (KT * hd * 2 + hd * KT * 2); }
-// What a launch asks for: the stages, a flag behind them, and never less than 88 KiB, more than half of a compute
-// unit's 160 KiB, so that a block has its compute unit to itself.  The waits between the kernel's MFMAs and the
-// instructions around them are counted by hand for a wave that is alone on its SIMD: with two blocks of heads of 64 a
-// compute unit (their 64 KiB and registers would allow it) some heads' rows came out different from run to run.
-constexpr int lds_request(int hd) { return lds_bytes(hd) + 16 > 88 * 1024 ? lds_bytes(hd) + 16 : 88 * 1024; }
+// What a launch asks for: the stages and a flag behind them.  Heads of 64 leave room for two blocks a compute unit
+// (64 KiB each, and the kernel is compiled for 256 registers a lane there).
+constexpr int lds_request(int hd) { return lds_bytes(hd) + 16; }
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float RISE = 64.f;               // by how much (in powers of 2) a score may exceed its row's reference
 
@@ -98,11 +95,37 @@ typedef __attribute__((address_space(3))) void* lds_ptr;
 // waits for it by count (LDS returns in order; LGKM = how many younger LDS reads may still be out).  Left to the
 // compiler, every LDS read behind a direct load waits until all direct loads have landed: it cannot tell that the
 // loads in flight fill other stages than the one being read.
+// The compiler takes the result of such a read for finished when the instruction has gone out.  So every read's
+// registers must be taken by a statement that waits for it (an MFMA with its count, or reads_done below) while the
+// compiler still holds them for the fragment: registers of a fragment that nothing takes any more are handed to the
+// next value at once, and the fragment then arrives on top of that value, sooner or later with the load on LDS.
+// (That happened here twice: the prologue read the last V fragment, which the first pass reads again, and the
+// softmax temporaries of the first tile got its registers, 128 cycles of s_nop behind the read; and the fragments
+// that the last pass asks for the pass that never comes were still out when the rows' sums moved into their
+// registers.  With one block a compute unit LDS answered in time; with a second block's reads and direct loads on the
+// same LDS it did not always, and rows differed from run to run.  tests/test_kernel_waits.py checks the compiler's
+// output for both patterns.)
 template <int OFFSET>
 __device__ __forceinline__ Frag lds_frag(int addr) {
   u32x4 v;
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
   return __builtin_bit_cast(Frag, v);
+}
+// waits for every LDS read of this wave and holds the fragments' registers until then
+template <int N>
+__device__ __forceinline__ void reads_done(const Frag (&a)[N], const Frag (&b)[N]) {
+  static_assert(N == 4 || N == 8, "one operand a fragment");
+  u32x4 x[2 * N];
+#pragma unroll
+  for (int g = 0; g < N; ++g) {
+    x[g] = __builtin_bit_cast(u32x4, a[g]);
+    x[N + g] = __builtin_bit_cast(u32x4, b[g]);
+  }
+  if constexpr (N == 4)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::"v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "v"(x[4]), "v"(x[5]), "v"(x[6]), "v"(x[7]));
+  else
+    asm volatile("s_waitcnt lgkmcnt(0)" ::"v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "v"(x[4]), "v"(x[5]), "v"(x[6]), "v"(x[7]),
+                 "v"(x[8]), "v"(x[9]), "v"(x[10]), "v"(x[11]), "v"(x[12]), "v"(x[13]), "v"(x[14]), "v"(x[15]));
 }
 constexpr int NO_WAIT = -1;  // an operand that has been in registers for long
 // c = a . q and c += a . q with the result in vector registers and q, the wave's query rows, which only MFMAs read, in
@@ -260,7 +283,7 @@ __device__ __forceinline__ void soft_any(int h, floatx16& s, Frag (&pf)[2], Soft
 // WIN: the rows see a window of keys (without one, a row's first key is key 0, which costs no register)
 // HD: the head size, 128 or 64 (half the MFMAs a pass for the same softmax)
 template <int HD, bool WIN>
-__global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
+__global__ __launch_bounds__(256, HD == 64 ? 2 : 1) void attn_prefill_wide_kernel(
     const bf16_t* __restrict__ q, int ldq, int q_off, bf16_t* __restrict__ out, int ldo, int H, int Hk,
     const bf16_t* __restrict__ cache, int lgP, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ positions, const int* __restrict__ row_seg, const int* __restrict__ tile_row0,
@@ -506,16 +529,17 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
   for (int ks = 0; ks < d / 16; ++ks) kaddr[ks] = (kh * 32 + li) * ROW_BYTES + ((((2 * ks) | lh) ^ k_swizzle(li)) * 16);
   const int vaddr = V_BASE + 2 * kh * (DT * 1024) + lane * 16;
   auto k_frag = [&](int stage_bytes, int ks) { return lds_frag<0>(lds0 + kaddr[ks] + stage_bytes); };
-  auto read_v_frags = [&](Frag (&vf)[NG], int va) {  // fragment g: the group of 16 keys g / DT, the elements 32 (g % DT) ..
+  // fragment g: the group of 16 keys g / DT, the elements 32 (g % DT) ..  All but the last one: slot A of every pass
+  // reads that one itself, and a read whose result nobody takes must not be asked for (see lds_frag).
+  auto read_v_frags_but_last = [&](Frag (&vf)[NG], int va) {
     vf[0] = lds_frag<0>(va);
     vf[1] = lds_frag<1024>(va);
     vf[2] = lds_frag<2048>(va);
-    vf[3] = lds_frag<3072>(va);
     if constexpr (NG > 4) {
+      vf[3] = lds_frag<3072>(va);
       vf[4] = lds_frag<4096>(va);
       vf[5] = lds_frag<5120>(va);
       vf[6] = lds_frag<6144>(va);
-      vf[7] = lds_frag<7168>(va);
     }
   };
   // the same through the compiler's own loads (the plain loop)
@@ -653,7 +677,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int g = 0; g < NG; ++g) kfr[g] = k_frag(K_STAGE, g);
-      read_v_frags(vfr, lds0 + vaddr);
+      read_v_frags_but_last(vfr, lds0 + vaddr);
       asm volatile("s_nop 15\n\ts_nop 15");  // the MFMAs have left the matrix cores: their results may be read
       __builtin_amdgcn_sched_barrier(0);
       const int tk = t_begin + kh * 32;
@@ -797,6 +821,9 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_wide_kernel(
       st[0].l += halves_sum(st[0].sum);
       st[1].l += halves_sum(st[1].sum);
     }
+    // the fragments that the last pass asked for (for a pass that does not come) have arrived: their registers are free
+    reads_done(kfr, vfr);
+    __builtin_amdgcn_sched_barrier(0);
     // a sum this large (or no number at all) means that some P was: such a block computes its rows again below
     const bool beyond_late = __builtin_amdgcn_ballot_w64(!(st[0].l < 0x1p90f) || !(st[1].l < 0x1p90f)) != 0;
 

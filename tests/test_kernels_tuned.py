@@ -639,10 +639,11 @@ def test_attention_of_whole_tiles_with_the_keys_cut_into_ranges_at_the_size_from
 
 @pytest.mark.parametrize("d", [128, 64])
 def test_attention_of_whole_tiles_gives_the_same_bits_every_time(d):
-    """The kernel for tiles of 128 rows counts the waits around its MFMAs by hand, for a wave that has its SIMD to
-    itself; sharing a compute unit with a second block showed as rows that differ from run to run.  More blocks than
-    compute units, many times: every output equals the first bit by bit (which the other tests hold against the plain
-    implementation at smaller sizes)."""
+    """The kernel for tiles of 128 rows counts the waits around its MFMAs and LDS reads by hand.  A read whose
+    registers the compiler had already given to another value once showed as rows that differ from run to run when
+    two blocks shared a compute unit's LDS (heads of 64 run that way).  More blocks than compute units, many times:
+    every output equals the first bit by bit (which the other tests hold against the plain implementation at smaller
+    sizes); tests/test_kernel_waits.py looks for the pattern itself in the compiler's output."""
     from allpaca_amd.engine.batch import Entry, pack_step
     from allpaca_amd.kernels import ops as kernel_ops
     t = tuned()
