@@ -40,6 +40,12 @@ class ModelRunner:
         elif os.environ.get("ALLPACA_POISON_FREE_PAGES") == "1":
             self.storage.poison_free_pages()
         self.views = self.storage.views(model.spec.plan)
+        # The model's steps from C++ (one call a step, intermediates in a work space) if every part of it describes
+        # itself to the executor; else, or with ALLPACA_AMD_PYTHON_WALK=1, the parts are walked in Python.
+        self.native = None
+        if os.environ.get("ALLPACA_AMD_PYTHON_WALK") != "1":
+            from .native import NativeProgram
+            self.native = NativeProgram.of(model, self.views)
         self.pad_pages = [self.storage.dummy_page(g) for g in range(len(self.cache.paged_groups))]
         self.vocab_size = model.spec.vocab_size
         # decode-only steps are replayed as HIP graphs when every part of the model allows it: a single part that
@@ -105,8 +111,7 @@ class ModelRunner:
         if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] and e.positions is None for e in entries):
             logits = self.graph_step(entries)
         else:
-            info = self.pack(entries)
-            logits = self.model.forward(info, self.bind_views(info))
+            logits = self.forward(self.pack(entries))
         for e in entries:
             self.cache.commit(e.seq, len(e.tokens))
         self.steps += 1
@@ -118,6 +123,12 @@ class ModelRunner:
         tables = [[self.cache.block_table(e.seq, g) for e in entries] for g in range(len(self.cache.paged_groups))]
         return pack_step(entries, pos0, slots, tables, self.rt.device, self.pad_pages, tile_rows=self.tile_rows,
                          position_axes=self.position_axes)
+
+    def forward(self, info: StepInfo) -> Optional[torch.Tensor]:
+        """The model on a packed step: logits at the wanted rows."""
+        if self.native is not None:
+            return self.native.forward(info)
+        return self.model.forward(info, self.bind_views(info))
 
     def bind_views(self, info: StepInfo) -> list:
         for v in self.views:
@@ -265,11 +276,12 @@ class DecodeGraph:
         self.fill([])
         self.upload()
         views = runner.bind_views(self.info)
-        # one eager run on a side stream (allocations settle), then the capture
+        native = runner.native
+        # one eager run on a side stream (allocations settle, the executor's work space has its size), then the capture
         side = torch.cuda.Stream(device=dev)
         side.wait_stream(torch.cuda.current_stream(dev))
         with torch.cuda.stream(side):
-            runner.model.forward(self.info, views)
+            runner.forward(self.info)
         torch.cuda.current_stream(dev).wait_stream(side)
         torch.cuda.synchronize(dev)
         # Two graphs: a short head (the embedding and the first layers) and the rest.  Launching a graph costs the
@@ -284,16 +296,28 @@ class DecodeGraph:
         gc_was_on = gc.isenabled()
         gc.collect()
         gc.disable()
+        if native is not None:
+            self.logits = torch.empty((rows, runner.vocab_size), dtype=torch.float32, device=dev)
         try:
             with torch.cuda.graph(self.graphs[0]):
-                x = model.embed(self.info)
-                left = model.run_plan(x, self.info, views, 0, cut, None)
-                if len(self.graphs) == 1:
-                    self.logits = model.logits(x, self.info)
+                if native is not None:
+                    native.begin(self.info)
+                    native.run_range(0, cut)
+                    if len(self.graphs) == 1:
+                        native.finish(self.logits)
+                else:
+                    x = model.embed(self.info)
+                    left = model.run_plan(x, self.info, views, 0, cut, None)
+                    if len(self.graphs) == 1:
+                        self.logits = model.logits(x, self.info)
             if len(self.graphs) == 2:
                 with torch.cuda.graph(self.graphs[1], pool=self.graphs[0].pool()):
-                    model.run_plan(x, self.info, views, cut, n_plan, left)
-                    self.logits = model.logits(x, self.info)
+                    if native is not None:
+                        native.run_range(cut, n_plan)
+                        native.finish(self.logits)
+                    else:
+                        model.run_plan(x, self.info, views, cut, n_plan, left)
+                        self.logits = model.logits(x, self.info)
         finally:
             if gc_was_on:
                 gc.enable()

@@ -1,8 +1,9 @@
 """Builds the HIP kernel libraries for gfx950 with hipcc and finds them again.
 
-Two libraries, so that a run compiles only what it needs: `plain` (the whole
+Two kernel libraries, so that a run compiles only what it needs: `plain` (the whole
 float32 path and the small steps of the bfloat16 path) and `tuned` (MFMA matrix
-products and attention for bfloat16).  Objects and libraries live in
+products and attention for bfloat16); and `host`, the engine's host side in C++
+(plan executor, cache manager, step packer, scheduler), which is linked against both.  Objects and libraries live in
 `allpaca_amd/_build/` (or, if the package folder cannot be written, in a
 per-user folder under the system's temporary directory).  A library is rebuilt
 when the text of its sources or the flags change."""
@@ -25,8 +26,13 @@ LIBS: Dict[str, List[str]] = {
     "plain": ["plain_ops.hip", "plain_gemm.hip", "plain_attention.hip", "sampling.hip"],
     "tuned": ["gemm_bf16.hip", "gemm_wide_bf16.hip", "gemm_direct_bf16.hip", "skinny_gemm_bf16.hip", "attention_bf16.hip", "attention_wide_bf16.hip", "rope_bf16.hip",
               "probe.hip"],
+    "host": ["host/exec.cpp"],
 }
-HEADERS = ["common.h", "mfma.h", "gemm_wide.h", "gemm_direct.h", "attention_wide.h", "no_alloc.h"]
+HEADERS = ["common.h", "mfma.h", "gemm_wide.h", "gemm_direct.h", "attention_wide.h", "no_alloc.h",
+           "host/host.h", "host/kernels.h", "host/rules.h"]
+# libraries a library is linked against (built first; found at run time beside it)
+NEEDS: Dict[str, List[str]] = {"host": ["plain", "tuned"]}
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wno-unused-value", "-Wno-unused-result"]
 
 ARCH = "gfx950"
 # -packed-fp32-ops is switched off for device code: some packed forms have given wrong results on this hardware.
@@ -43,6 +49,8 @@ VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 
 
 def flags_for(src: str) -> List[str]:
+    if src.endswith(".cpp"):      # host code: no device pass
+        return list(HOST_FLAGS)
     if os.path.basename(src) not in ACC_REGISTER_SOURCES:
         return list(FLAGS)
     out, skip = [], 0
@@ -89,8 +97,10 @@ def _sources(name: str) -> List[str]:
 
 def source_hash(name: str) -> str:
     h = hashlib.sha256()
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(FLAGS + HOST_FLAGS).encode())
     h.update(" ".join(sorted(ACC_REGISTER_SOURCES)).encode())
+    for dep in NEEDS.get(name, []):
+        h.update(source_hash(dep).encode())
     for path in _sources(name) + [os.path.join(CSRC, f) for f in HEADERS]:
         if os.path.isfile(path):
             h.update(os.path.basename(path).encode())
@@ -120,6 +130,8 @@ def build(name: str, force: bool = False, verbose: bool = True) -> str:
     """Compile library `name`; returns the path of the .so."""
     if name not in LIBS:
         raise KernelBuildError(f"no kernel library {name!r}; known: {sorted(LIBS)}")
+    for dep in NEEDS.get(name, []):
+        build(dep, force=False, verbose=verbose)
     if not force and is_current(name):
         return lib_path(name)
     hipcc = _hipcc()
@@ -158,7 +170,10 @@ def build(name: str, force: bool = False, verbose: bool = True) -> str:
             objs = list(ex.map(compile_one, srcs))
         out = lib_path(name, d)
         tmp = out + f".tmp{os.getpid()}"
-        p = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", tmp],
+        deps = [f"-lallpaca_{dep}" for dep in NEEDS.get(name, [])]
+        if deps:
+            deps = ["-L", d, *deps, "-Wl,-rpath,$ORIGIN"]
+        p = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, *deps, "-o", tmp],
                            stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         if p.returncode != 0:
             raise KernelBuildError(f"link of {out} failed:\n{p.stdout}")
@@ -179,4 +194,4 @@ def build(name: str, force: bool = False, verbose: bool = True) -> str:
 
 
 def build_all(force: bool = True, verbose: bool = True) -> List[str]:
-    return [build(n, force=force, verbose=verbose) for n in LIBS]
+    return [build(n, force=force, verbose=verbose) for n in LIBS]   # (in the order of LIBS: what is needed comes first)

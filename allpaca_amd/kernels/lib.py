@@ -67,6 +67,11 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
     },
 }
 
+# The host library's entry points take structures (declared in `kernels/host.py`, which fills this in) and some
+# return something other than an int.
+SIGNATURES["host"] = {}
+RESTYPES: Dict[str, object] = {}
+
 _loaded: Dict[str, "Library"] = {}
 
 ERRORS = {-1: "bad argument (shape or stride the kernel does not accept)", -2: "size not supported by this kernel",
@@ -158,8 +163,8 @@ def load(name: str) -> Library:
         except AttributeError:
             raise KernelLibraryError(f"{path} lacks entry point {fn}") from None
         f.argtypes = args
-        f.restype = I
-        setattr(lib, fn, _EntryPoint(fn, f, args))
+        f.restype = RESTYPES.get(fn, I)
+        setattr(lib, fn, _EntryPoint(fn, f, args) if name != "host" else f)
     _loaded[name] = lib
     return lib
 

@@ -82,6 +82,16 @@ class Attention(Mixer):
                             cache.block_table, step, window=self.window or 0, scale=self.scale)
         ops.linear(attn, self.w_o, residual, accumulate=True, emit=emit)
 
+    def native_desc(self):
+        if type(self) is not Attention:
+            return None
+        fused = self.position.fused() if self.position is not None else (0, None)
+        if fused is None:           # an encoding that transforms q and k itself: walked in Python
+            return None
+        rot, table = fused
+        return {"kind": "attention", "w_qkv": self.w_qkv, "w_o": self.w_o, "H": self.H, "Hk": self.Hk, "d": self.d,
+                "window": self.window or 0, "scale": self.scale or 0.0, "rot": int(rot), "cos_sin": table}
+
     def forward(self, h, step, cache):
         out = torch.zeros((h.shape[0], self.D), dtype=torch.float32, device=h.device)
         self.forward_add(h, step, cache, out)

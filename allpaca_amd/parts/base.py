@@ -111,6 +111,13 @@ class Part:
         """Receives the tensors named by `param_specs` (CPU or GPU) and moves what it keeps to `rt.device`."""
         self.rt = rt
 
+    def native_desc(self):
+        """What the compiled plan executor (`engine/native.py`, `csrc/host/exec.cpp`) needs to run this part itself: a
+        dict of the part's bound tensors and constants under the names the executor knows for the part's kind, or
+        None (the default) for a part it does not know.  A model runs on the executor only if all its parts and
+        arrangements answer; otherwise its steps are walked in Python, part by part."""
+        return None
+
 
 class Norm(Part):
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:

@@ -41,6 +41,10 @@ class Block:
     def mixer(self):
         return self.parts["mixer"]
 
+    def native_desc(self):
+        describe = getattr(self.arrangement, "native_desc", None)
+        return describe(self.parts) if describe is not None else None
+
     def param_specs(self):
         out = {}
         for role, part in self.parts.items():
@@ -65,6 +69,15 @@ class PreNorm:
     @staticmethod
     def first_norm(parts):
         return parts["mixer_norm"] if parts["mixer"].takes_normed_input else None
+
+    @staticmethod
+    def native_desc(parts):
+        """The layer for the compiled executor, if it knows all four parts: a dict role -> the part's own description."""
+        out = {role: parts[role].native_desc() for role in ("mixer_norm", "mixer", "ffn_norm", "ffn")}
+        kinds = {"mixer_norm": "rmsnorm", "mixer": "attention", "ffn_norm": "rmsnorm", "ffn": "swiglu"}
+        if any(d is None or d.get("kind") != kinds[role] for role, d in out.items()):
+            return None
+        return {"kind": "pre_norm", **out}
 
     @staticmethod
     def run(parts, x: torch.Tensor, step, cache, pre=None, next_norm=None):

@@ -29,6 +29,9 @@ class TokenEmbedding(Part):
     def forward(self, tokens: torch.Tensor, out: torch.Tensor) -> None:
         ops.embed_rows(self.weight, tokens, out)
 
+    def native_desc(self):
+        return {"kind": "token_table", "weight": self.weight} if type(self) is TokenEmbedding else None
+
 
 @HEADS.register("linear")
 class LinearHead(Part):
@@ -49,3 +52,6 @@ class LinearHead(Part):
 
     def forward(self, h: torch.Tensor, out: torch.Tensor) -> None:
         ops.linear(h, self.weight, out)
+
+    def native_desc(self):
+        return {"kind": "linear", "weight": self.weight} if type(self) is LinearHead else None

@@ -48,6 +48,11 @@ class SwiGLU(FeedForward):
         h.swiglu(self.w_gate_up, act)
         ops.linear(act, self.w_down, residual, accumulate=True, emit=emit)
 
+    def native_desc(self):
+        if type(self) is not SwiGLU:
+            return None
+        return {"kind": "swiglu", "w_gate_up": self.w_gate_up, "w_down": self.w_down, "F": self.F}
+
     def forward(self, h, step):
         out = torch.zeros((h.shape[0], self.D), dtype=torch.float32, device=h.device)
         self.forward_add(h, step, out)

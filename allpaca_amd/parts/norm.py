@@ -31,3 +31,6 @@ class RMSNorm(Norm):
 
     def rms_params(self):
         return self.weight, self.eps
+
+    def native_desc(self):
+        return {"kind": "rmsnorm", "weight": self.weight, "eps": self.eps} if type(self) is RMSNorm else None

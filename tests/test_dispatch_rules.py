@@ -81,3 +81,32 @@ def test_keys_a_wave_of_the_decode_attention_takes():
                    (8, 8192): 512, (16, 8192): 512, (1, 32768): 256}
     assert t._keys_per_part(16, 8, 1 << 20, 16) // 16 + 2 <= 64 and t._keys_per_part(16, 8, 1 << 20, 128) == 1024
     assert t._keys_per_part(1, 1, 10, 16) == 64
+
+
+def test_the_executors_rules_are_the_wrappers_rules():
+    """The compiled plan executor (csrc/host/rules.h) chooses slices of K, keys a wave and ranges of keys by the same
+    rules as the Python wrappers of the kernels: held against each other over the shapes either may meet."""
+    from allpaca_amd.kernels import host, tuned
+    L = host.load()
+    for M in (17, 24, 32, 48, 64, 100, 128, 129, 200, 256, 384, 500, 512, 640, 768, 1000, 1024, 1025, 2048):
+        for N in (192, 1000, 2048, 3072, 4096, 5120, 6144, 8192, 14336, 16384, 28672, 57344, 128256):
+            for K in (120, 192, 512, 2048, 3072, 4096, 8192, 14336, 28672):
+                assert L.apc_host_rule_tiled_k_split(M, N, K) == tuned._tiled_k_split(M, N, K), (M, N, K)
+    for n in (1, 2, 3, 8, 12, 16, 24, 31, 64, 255):
+        for hk in (1, 2, 8):
+            for ctx in (1, 63, 64, 65, 2048, 2049, 8192, 32768, 131072):
+                for page in (8, 16, 24, 64, 128, 256):
+                    assert (L.apc_host_rule_keys_per_part(n, hk, ctx, page)
+                            == tuned._keys_per_part(n, hk, ctx, page)), (n, hk, ctx, page)
+    for ctx in (1, 100, 256, 257, 2048, 2049, 5000, 131072):
+        for page in (8, 16, 24, 64, 128, 256):
+            assert L.apc_host_rule_keys_per_wave_whole(ctx, page) == tuned._keys_per_wave_whole(ctx, page), (ctx, page)
+    for rows in (2, 100, 128, 129, 256, 512, 1024, 2048):
+        for pos0 in (0, 500, 1920, 3584, 8000, 32640, 130000):
+            for heads in (4, 8, 24, 32, 64):
+                for window in (0, 1000, 4096):
+                    step = _step([(pos0, rows), (7, 1)])
+                    want = tuned._key_splits(step, heads, window)
+                    got = L.apc_host_rule_key_splits(step.n_tiles, heads, pos0 + rows, window, tuned.KEY_SPLITS_MAX,
+                                                     tuned.KEY_RANGE_MIN)
+                    assert got == want, (rows, pos0, heads, window)
