@@ -17,7 +17,8 @@ crates/allpaca-core/src/kv_tier.rs:341-532); recurrent layers get no pages
 (crates/allpaca-core/src/model.rs:13392-13405)."""
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+import ctypes
+from dataclasses import dataclass
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 from ..parts.base import CacheNeed, need_kind
@@ -37,44 +38,89 @@ class OutOfSlots(CacheError):
     pass
 
 
-class PagePool:
-    """`num_pages` page ids handed out from a stack."""
+def _host():
+    from ..kernels import host
+    return host.load()
 
-    def __init__(self, num_pages: int):
+
+_POOL_ERRORS = {-22: OutOfPages, -27: CacheError, -28: CacheError, -29: CacheError}
+
+
+def _raise_pool(code: int, page=None):
+    if code == -22:
+        raise OutOfPages("no free page")
+    if code == -27:
+        raise CacheError(f"page id {page} is outside the pool")
+    if code == -28:
+        raise CacheError(f"page {page} freed twice")
+    if code == -29:
+        raise CacheError("a page was on the free list while held")
+    raise CacheError(f"page pool: error {code}")
+
+
+class PagePool:
+    """`num_pages` page ids handed out from a stack (the books are kept in `csrc/host/cache.cpp`)."""
+
+    def __init__(self, num_pages: int, _borrowed=None, _owner=None):
         if num_pages <= 0:
             raise ValueError("a page pool needs at least one page")
+        self._lib = _host()
+        self._owner = _owner             # the cache manager whose pool this is (keeps it alive), or None
+        self._p = _borrowed if _borrowed is not None else self._lib.apc_pool_new(num_pages)
         self.num_pages = num_pages
-        self._free: List[int] = list(range(num_pages - 1, -1, -1))  # page 0 goes out first
-        self._held = [False] * num_pages
-        self.allocations = 0   # how many times a page was handed out (reuse shows as allocations > num_pages)
-        self.on_free = None    # called with the id of every page that comes back (a debugging aid: see CacheStorage)
+        self._on_free = None
+
+    def __del__(self):
+        if getattr(self, "_owner", None) is None and getattr(self, "_p", None):
+            self._lib.apc_pool_free(self._p)
+            self._p = None
+
+    @property
+    def on_free(self):
+        """Called with the id of every page that comes back (a debugging aid: see CacheStorage)."""
+        return self._on_free
+
+    @on_free.setter
+    def on_free(self, fn) -> None:
+        self._on_free = fn
+        self._lib.apc_pool_log_frees(self._p, 1 if fn is not None else 0)
+
+    def _tell_frees(self) -> None:
+        if self._on_free is None:
+            return
+        buf = (ctypes.c_int * 256)()
+        while True:
+            k = self._lib.apc_pool_drain(self._p, buf, 256)
+            for i in range(k):
+                self._on_free(buf[i])
+            if k < 256:
+                return
 
     @property
     def free_count(self) -> int:
-        return len(self._free)
+        return self._lib.apc_pool_free_count(self._p)
+
+    @property
+    def allocations(self) -> int:
+        """How many times a page was handed out (reuse shows as allocations > num_pages)."""
+        return self._lib.apc_pool_allocations(self._p)
 
     def alloc(self) -> int:
-        if not self._free:
-            raise OutOfPages("no free page")
-        p = self._free.pop()
-        if self._held[p]:
-            raise CacheError(f"page {p} was on the free list while held")
-        self._held[p] = True
-        self.allocations += 1
+        p = self._lib.apc_pool_alloc(self._p)
+        if p < 0:
+            _raise_pool(p)
         return p
 
     def free(self, page: int) -> None:
-        if not (0 <= page < self.num_pages):
-            raise CacheError(f"page id {page} is outside the pool")
-        if not self._held[page]:
-            raise CacheError(f"page {page} freed twice")
-        self._held[page] = False
-        self._free.append(page)
-        if self.on_free is not None:
-            self.on_free(page)
+        code = self._lib.apc_pool_give_back(self._p, int(page))
+        if code:
+            _raise_pool(code, page)
+        self._tell_frees()
 
     def held(self) -> List[int]:
-        return [p for p, h in enumerate(self._held) if h]
+        buf = (ctypes.c_int * self.num_pages)()
+        k = self._lib.apc_pool_held(self._p, buf, self.num_pages)
+        return list(buf[:k])
 
 
 class SlotPool(PagePool):
@@ -100,15 +146,6 @@ class StateGroup:
     entries: List[int]
 
 
-@dataclass
-class _Sequence:
-    slot: int
-    length: int = 0                    # positions committed
-    reserved: int = 0                  # positions that pages exist for
-    tables: List[List[int]] = field(default_factory=list)   # per paged group: page ids, FREED where a window passed
-    version: int = 0                   # changes whenever an entry of a table was taken away or replaced
-
-
 def group_needs(needs: Sequence[CacheNeed]) -> Tuple[List[Tuple[CacheNeed, List[int]]], List[Tuple[CacheNeed, List[int]]]]:
     """Plan entries sorted by what they need: ([(need of kind "pages", entries)], [(need of kind "slot", entries)]).
     Equal needs share a group; a need is any object with the members `parts.base` lists."""
@@ -129,7 +166,9 @@ def group_needs(needs: Sequence[CacheNeed]) -> Tuple[List[Tuple[CacheNeed, List[
 class CacheManager:
     """Block tables and slots for live requests.
 
-    `num_pages`: pages of every paged group's pool (an int for all, or one per group)."""
+    `num_pages`: pages of every paged group's pool (an int for all, or one per group).  Requests are named by any
+    hashable; the books themselves are kept in C++ (`csrc/host/cache.cpp`) under ids that this class hands out, so
+    that the step packer and the scheduler there read them without coming back to Python."""
 
     def __init__(self, needs: Sequence[CacheNeed], page_tokens: int, num_pages, max_requests: int):
         if page_tokens <= 0:
@@ -140,12 +179,26 @@ class CacheManager:
             num_pages = [num_pages] * len(paged)
         if len(num_pages) != len(paged):
             raise ValueError(f"{len(paged)} paged groups but {len(num_pages)} pool sizes")
-        self.paged_groups = [PagedGroup(n, e, PagePool(np_)) for (n, e), np_ in zip(paged, num_pages)]
+        if len(paged) > 8:
+            raise ValueError(f"{len(paged)} paged groups: the cache manager keeps books for at most 8")
+        if any(n <= 0 for n in num_pages) or max_requests <= 0:
+            raise ValueError("a page pool needs at least one page")
+        self._lib = L = _host()
+        windows = [(-1 if getattr(n, "window", None) is None else int(n.window)) for n, _ in paged]
+        G = len(paged)
+        self._c = L.apc_cache_new(page_tokens, G, (ctypes.c_int * max(G, 1))(*windows),
+                                  (ctypes.c_int * max(G, 1))(*[int(n) for n in num_pages]), max_requests)
+        if not self._c:
+            raise ValueError("the cache manager could not be set up with these sizes")
+        self.paged_groups = [PagedGroup(n, e, PagePool(np_, L.apc_cache_pool(self._c, gi), self))
+                             for gi, ((n, e), np_) in enumerate(zip(paged, num_pages))]
         self.state_groups = [StateGroup(n, e) for n, e in state]
-        self.slots = SlotPool(max_requests)
+        self.slots = SlotPool(max_requests, L.apc_cache_pool(self._c, -1), self)
         self.max_requests = max_requests
-        self._seqs: Dict[Hashable, _Sequence] = {}
-        self._versions = 0
+        self._ids: Dict[Hashable, int] = {}
+        self._next_id = 0
+        self._need = (ctypes.c_int * 8)()
+        self._table = (ctypes.c_int * 64)()
         # plan entry -> ("paged", group index, index inside the group) | ("state", ...) ; filled for owners only
         self.location: Dict[int, Tuple[str, int, int]] = {}
         for gi, g in enumerate(self.paged_groups):
@@ -155,41 +208,89 @@ class CacheManager:
             for li, e in enumerate(g.entries):
                 self.location[e] = ("state", gi, li)
 
+    def __del__(self):
+        if getattr(self, "_c", None):
+            self._lib.apc_cache_free(self._c)
+            self._c = None
+
+    @property
+    def handle(self):
+        """The books' address, for the C++ step packer and scheduler."""
+        return self._c
+
+    def id_of(self, seq) -> int:
+        """The id under which the C++ side knows a live request."""
+        return self._ids[seq]
+
+    # The C++ scheduler admits and releases requests in the books itself; it tells this face afterwards.
+    def new_id(self) -> int:
+        """An id that no request has had: for a request that the C++ scheduler will admit under it."""
+        self._next_id += 1
+        return self._next_id - 1
+
+    def remember(self, seq, sid: int) -> None:
+        """`seq` was admitted in the books under id `sid`."""
+        if seq in self._ids:
+            raise CacheError(f"request {seq!r} is already live")
+        self._ids[seq] = sid
+
+    def forget(self, seq) -> None:
+        """`seq` was released in the books."""
+        self._ids.pop(seq, None)
+
+    def _fail(self, code: int, seq, what: str = ""):
+        if code == -20:
+            raise CacheError(f"request {seq!r} is already live")
+        if code == -21:
+            raise OutOfSlots("no free state slot")
+        if code == -22:
+            raise OutOfPages(f"request {seq!r} needs more pages than the pool has free{what}")
+        if code == -23:
+            raise CacheError(f"request {seq!r}: commit of positions beyond what was reserved")
+        if code == -24:
+            raise CacheError("truncate beyond the current length")
+        if code == -25:
+            raise CacheError("truncate below pages that a window has already given back")
+        if code == -26:
+            raise KeyError(seq)
+        if code == -28:
+            raise CacheError("a page was freed twice")
+        raise CacheError(f"cache manager: error {code}")
+
+    def _tell_frees(self) -> None:
+        for g in self.paged_groups:
+            if g.pool._on_free is not None:
+                g.pool._tell_frees()
+
     # ---- requests ------------------------------------------------------------
     def __contains__(self, seq) -> bool:
-        return seq in self._seqs
+        return seq in self._ids
 
     def live(self) -> List[Hashable]:
-        return list(self._seqs)
+        return list(self._ids)
 
     def admit(self, seq) -> int:
         """Registers a request and gives it a state slot (the caller zeroes the slot's state)."""
-        if seq in self._seqs:
+        if seq in self._ids:
             raise CacheError(f"request {seq!r} is already live")
-        slot = self.slots.alloc()
-        self._versions += 1
-        self._seqs[seq] = _Sequence(slot, tables=[[] for _ in self.paged_groups], version=self._versions)
+        sid = self._next_id
+        slot = self._lib.apc_cache_admit(self._c, sid)
+        if slot < 0:
+            self._fail(slot, seq)
+        self._next_id += 1
+        self._ids[seq] = sid
         return slot
 
     def slot_of(self, seq) -> int:
-        return self._seqs[seq].slot
+        return self._lib.apc_cache_slot(self._c, self._ids[seq])
 
     def length(self, seq) -> int:
-        return self._seqs[seq].length
-
-    def _first_needed(self, need: CacheNeed, next_pos: int) -> int:
-        """First position whose page a row at `next_pos` or later can still read."""
-        window = getattr(need, "window", None)
-        if window is None:
-            return 0
-        return max(0, next_pos - window + 1)
+        return self._lib.apc_cache_length(self._c, self._ids[seq])
 
     def pages_needed(self, seq, n_new: int) -> List[int]:
         """Pages each group must still take so that positions up to length + n_new exist."""
-        s = self._seqs[seq]
-        end = s.length + n_new
-        want = -(-end // self.page_tokens)
-        return [max(0, want - len(t)) for t in s.tables]
+        self._lib.apc_cache_pages_needed(self._c, self._ids[seq], int(n_new), self._need)
+        return list(self._need[:len(self.paged_groups)])
 
     def can_reserve(self, seq, n_new: int, spare: Optional[List[int]] = None) -> bool:
         """`spare`: pages per group already promised to others in the same step."""
@@ -199,64 +300,48 @@ class CacheManager:
 
     def reserve(self, seq, n_new: int) -> None:
         """Takes the pages for the next `n_new` positions, in every group or in none."""
-        s = self._seqs[seq]
-        need = self.pages_needed(seq, n_new)
-        for n, g in zip(need, self.paged_groups):
-            if n > g.pool.free_count:
-                raise OutOfPages(f"request {seq!r} needs {n} more pages, the pool has {g.pool.free_count} free")
-        for n, g, t in zip(need, self.paged_groups, s.tables):
-            for _ in range(n):
-                t.append(g.pool.alloc())
-        s.reserved = max(s.reserved, s.length + n_new)
+        code = self._lib.apc_cache_reserve(self._c, self._ids[seq], int(n_new))
+        if code:
+            what = ""
+            if code == -22:
+                what = f" ({self.pages_needed(seq, n_new)} wanted, {[g.pool.free_count for g in self.paged_groups]} free)"
+            self._fail(code, seq, what)
 
     def commit(self, seq, n_new: int) -> None:
         """The step wrote `n_new` positions; pages that every later row's window has passed go back."""
-        s = self._seqs[seq]
-        if s.length + n_new > s.reserved:
-            raise CacheError(f"request {seq!r}: commit of {n_new} positions beyond what was reserved")
-        s.length += n_new
-        for g, t in zip(self.paged_groups, s.tables):
-            first = self._first_needed(g.need, s.length)
-            for i in range(min(first // self.page_tokens, len(t))):
-                if t[i] != FREED:
-                    g.pool.free(t[i])
-                    t[i] = FREED
-                    self._versions += 1
-                    s.version = self._versions
+        code = self._lib.apc_cache_commit(self._c, self._ids[seq], int(n_new))
+        if code:
+            self._fail(code, seq)
+        self._tell_frees()
 
     def truncate(self, seq, length: int) -> None:
         """Forgets positions >= length (pages wholly beyond go back).  Not possible below a window's edge."""
-        s = self._seqs[seq]
-        if length > s.length:
-            raise CacheError("truncate beyond the current length")
-        keep = -(-length // self.page_tokens)
-        for g, t in zip(self.paged_groups, s.tables):
-            if any(p == FREED for p in t[self._first_needed(g.need, length) // self.page_tokens:keep]):
-                raise CacheError("truncate below pages that a window has already given back")
-            while len(t) > keep:
-                p = t.pop()
-                self._versions += 1
-                s.version = self._versions
-                if p != FREED:
-                    g.pool.free(p)
-        s.length = length
-        s.reserved = min(s.reserved, keep * self.page_tokens)
+        code = self._lib.apc_cache_truncate(self._c, self._ids[seq], int(length))
+        if code:
+            self._fail(code, seq)
+        self._tell_frees()
 
     def release(self, seq) -> None:
-        s = self._seqs.pop(seq)
-        for g, t in zip(self.paged_groups, s.tables):
-            for p in t:
-                if p != FREED:
-                    g.pool.free(p)
-        self.slots.free(s.slot)
+        sid = self._ids.pop(seq)
+        code = self._lib.apc_cache_release(self._c, sid)
+        self._tell_frees()
+        if code:
+            self._fail(code, seq)
 
     def block_table(self, seq, group: int) -> List[int]:
-        return self._seqs[seq].tables[group]
+        sid = self._ids[seq]
+        n = self._lib.apc_cache_table(self._c, sid, group, self._table, len(self._table))
+        if n > len(self._table):
+            self._table = (ctypes.c_int * (2 * n))()
+            n = self._lib.apc_cache_table(self._c, sid, group, self._table, len(self._table))
+        if n < 0:
+            self._fail(n, seq)
+        return list(self._table[:n])
 
     def table_version(self, seq) -> int:
         """A number that is the same as at an earlier call only if the request's block tables have only grown since
         (no page taken away or replaced, and it is the same admission of the request)."""
-        return self._seqs[seq].version
+        return self._lib.apc_cache_version(self._c, self._ids[seq])
 
     def free_pages(self, group: int = 0) -> int:
         return self.paged_groups[group].pool.free_count
@@ -267,20 +352,5 @@ class CacheManager:
     # ---- self-check (tests) ----------------------------------------------------
     def check(self) -> None:
         """No page lost, none held twice, free + held = pool."""
-        for gi, g in enumerate(self.paged_groups):
-            seen: Dict[int, Hashable] = {}
-            for sid, s in self._seqs.items():
-                for p in s.tables[gi]:
-                    if p == FREED:
-                        continue
-                    if p in seen:
-                        raise CacheError(f"group {gi}: page {p} held by {seen[p]!r} and {sid!r}")
-                    seen[p] = sid
-            held = set(g.pool.held())
-            if held != set(seen):
-                raise CacheError(f"group {gi}: pool holds {sorted(held)}, block tables hold {sorted(seen)}")
-            if len(held) + g.pool.free_count != g.pool.num_pages:
-                raise CacheError(f"group {gi}: {len(held)} held + {g.pool.free_count} free != {g.pool.num_pages}")
-        slots = [s.slot for s in self._seqs.values()]
-        if len(set(slots)) != len(slots) or set(slots) != set(self.slots.held()):
-            raise CacheError("state slots and live requests disagree")
+        if self._lib.apc_cache_check(self._c):
+            raise CacheError(self._lib.apc_cache_why(self._c).decode())

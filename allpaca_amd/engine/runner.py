@@ -9,6 +9,7 @@ mixes a prompt portion with decode rows in one of them
 (crates/allpaca-core/src/engine.rs:5451-5607); this is the one generalisation."""
 from __future__ import annotations
 
+import ctypes
 import gc
 import os
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
@@ -58,6 +59,16 @@ class ModelRunner:
         self.graphs: Dict[Tuple[int, int], "DecodeGraph"] = {}
         self.graph_replays = 0
         self.steps = 0
+        # The C++ side of a step (csrc/host/pack.cpp): entries checked against the cache's books, pages taken, the
+        # description written into one of a few pinned buffers that take turns (a buffer is written again only when
+        # the copy out of it has run).
+        from ..kernels import host as _host
+        self._host, self._hostlib = _host, _host.load()
+        self._staging: List[list] = []        # [pinned tensor, its numpy view, event of the last copy out of it]
+        self._staging_at = 0
+        self._pad_pages = np.asarray(self.pad_pages or [0], dtype=np.int32)
+        self._finding = _host.ApcStepFinding()
+        self._packed = _host.ApcPacked()
 
     # ---- requests ------------------------------------------------------------
     def admit(self, seq: Hashable) -> int:
@@ -93,10 +104,117 @@ class ModelRunner:
                 raise StepError(f"request {e.seq!r}: position {self.cache.length(e.seq) + n - 1} is beyond the "
                                 f"{self.rt.max_positions} positions this run was set up for")
 
+    # ---- a step through the C++ packer ---------------------------------------------------------------------
+    def _flatten(self, entries: Sequence[Entry]):
+        """The entries as arrays for the C++ side: (ids, tokens a request, all tokens, wanted places a request, all
+        wanted places).  Requests named twice or not admitted are refused here, where their names are known."""
+        ids, n_tok, toks, n_want, wants = [], [], [], [], []
+        known = self.cache._ids
+        seen = set()
+        for e in entries:
+            if e.seq in seen:
+                raise StepError(f"request {e.seq!r} appears twice in one step")
+            seen.add(e.seq)
+            sid = known.get(e.seq)
+            if sid is None:
+                raise StepError(f"request {e.seq!r} is not admitted")
+            ids.append(sid)
+            n_tok.append(len(e.tokens))
+            toks.extend(e.tokens)
+            n_want.append(len(e.want))
+            wants.extend(e.want)
+        t64 = np.asarray(toks, dtype=np.int64)
+        if t64.size and (int(t64.min()) < 0 or int(t64.max()) >= self.vocab_size):   # (also what int32 cannot hold)
+            at = int(np.flatnonzero((t64 < 0) | (t64 >= self.vocab_size))[0])
+            e = entries[int(np.searchsorted(np.cumsum(n_tok), at, side="right"))]
+            raise StepError(f"request {e.seq!r}: token {int(t64[at])} is outside the vocabulary of {self.vocab_size}")
+        w64 = np.asarray(wants, dtype=np.int64)
+        if w64.size and (int(w64.min()) < 0 or int(w64.max()) >= (1 << 31) - 1):
+            w64 = np.clip(w64, -1, (1 << 31) - 2)       # refused below, with its request's name
+        return (np.asarray(ids, dtype=np.int64), np.asarray(n_tok, dtype=np.int32), t64.astype(np.int32),
+                np.asarray(n_want, dtype=np.int32), w64.astype(np.int32))
+
+    def _prepare(self, entries: Sequence[Entry], flat) -> None:
+        """Checks the step and takes its pages, for all requests or for none."""
+        ids, n_tok, toks, n_want, wants = flat
+        f = self._finding
+        code = self._hostlib.apc_step_prepare(self.cache.handle, self.vocab_size, self.rt.max_positions, len(entries),
+                                              ids.ctypes.data, n_tok.ctypes.data, toks.ctypes.data, n_want.ctypes.data,
+                                              wants.ctypes.data, ctypes.byref(f))
+        if code == 0:
+            return
+        if code < 0:
+            self.cache._fail(code, None)
+        e = entries[f.entry] if f.what != 7 else None
+        if f.what == 3:
+            raise StepError(f"request {e.seq!r} brings no tokens")
+        if f.what == 4:
+            raise StepError(f"request {e.seq!r}: token {f.value} is outside the vocabulary of {self.vocab_size}")
+        if f.what == 5:
+            raise StepError(f"request {e.seq!r}: wanted place {f.value} is outside its {len(e.tokens)} tokens")
+        if f.what == 6:
+            raise StepError(f"request {e.seq!r}: position {f.value} is beyond the {self.rt.max_positions} positions "
+                            f"this run was set up for")
+        if f.what == 7:
+            raise OutOfPages(f"the step needs {f.value} new pages in group {f.entry}, {f.extra} are free")
+        raise StepError(f"the step was refused (finding {f.what} at entry {f.entry})")
+
+    def _staging_buffer(self, ints: int):
+        """A pinned buffer of at least `ints` int32 that no copy is reading any more."""
+        if len(self._staging) < 4:
+            t = torch.zeros(max(ints, 1 << 14), dtype=torch.int32).pin_memory()
+            self._staging.append([t, t.numpy(), None])
+            slot = self._staging[-1]
+        else:
+            slot = self._staging[self._staging_at]
+            self._staging_at = (self._staging_at + 1) % len(self._staging)
+            if slot[2] is not None:
+                slot[2].synchronize()
+            if slot[0].numel() < ints:
+                slot[0] = torch.zeros(max(ints, 2 * slot[0].numel()), dtype=torch.int32).pin_memory()
+                slot[1] = slot[0].numpy()
+        return slot
+
+    def _pack_flat(self, entries: Sequence[Entry], flat) -> StepInfo:
+        ids, n_tok, toks, n_want, wants = flat
+        L, c, p = self._hostlib, self.cache.handle, self._packed
+        n = len(entries)
+        L.apc_pack_layout(c, n, ids.ctypes.data, n_tok.ctypes.data, n_want.ctypes.data, self.tile_rows, 1, ctypes.byref(p))
+        slot = self._staging_buffer(p.total)
+        host, view = slot[0], slot[1]
+        code = L.apc_pack_step(c, n, ids.ctypes.data, n_tok.ctypes.data, toks.ctypes.data, n_want.ctypes.data,
+                               wants.ctypes.data, self.tile_rows, 1, self._pad_pages.ctypes.data, view.ctypes.data,
+                               view.size, ctypes.byref(p))
+        if code:
+            self._host.check(code, "packing a step")
+        dev = torch.empty(p.total, dtype=torch.int32, device=self.rt.device)
+        dev.copy_(host[:p.total], non_blocking=True)
+        if slot[2] is None:
+            slot[2] = torch.cuda.Event()
+        slot[2].record()
+        lay = StepLayout(p.T, p.S, p.R, p.n_decode, p.n_tiles, 1, list(p.table_width[:p.n_groups]))
+        o = p.off
+        return lay.info(dev, view[o[3]:o[3] + n].tolist(), n_tok.tolist(), view[o[5]:o[5] + n].tolist(),
+                        view[o[6]:o[6] + n].tolist(), p.max_decode_context, p.n_decode == p.T)
+
     def step(self, entries: Sequence[Entry]) -> Optional[torch.Tensor]:
         """Runs one batch; returns float32 logits [sum of wanted places, vocab] (device), or None."""
         if not entries:
             return None
+        if self.position_axes == 1 and all(e.positions is None for e in entries):
+            flat = self._flatten(entries)
+            self._prepare(entries, flat)
+            if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+                logits = self.graph_step(entries)
+            else:
+                logits = self.forward(self._pack_flat(entries, flat))
+            code = self._hostlib.apc_step_commit(self.cache.handle, len(entries), flat[0].ctypes.data, flat[1].ctypes.data)
+            if code:
+                self.cache._fail(code, None)
+            self.cache._tell_frees()
+            self.steps += 1
+            return logits
+        # positions on more than one axis: the step is packed in Python
         self.validate(entries)
         # pages for this step's tokens only, for all requests or for none
         need = [0] * len(self.cache.paged_groups)

@@ -28,6 +28,7 @@ crates/allpaca-core/src/scheduler.rs:607-664) by `prefill.chunk_tokens`
 so never runs out while decoding; what happens then is this engine's own rule."""
 from __future__ import annotations
 
+import ctypes
 from collections import deque
 from dataclasses import dataclass, field
 from typing import Deque, Dict, List, Optional, Tuple
@@ -114,8 +115,13 @@ class Plan:
 
 
 class Scheduler:
+    """The face of the C++ scheduler (`csrc/host/sched.cpp`): it keeps the requests themselves (their tokens, their
+    times) and mirrors what the C++ side decides into them (`status`, `computed`, `order`, `preemptions`) and into
+    `waiting` and `running`, which hold the same requests in the same order as the queues there."""
+
     def __init__(self, cache: CacheManager, max_active_requests: int, max_batch_tokens: int, chunk_tokens: int,
                  row_tile: int = 0):
+        from ..kernels import host
         self.cache = cache
         self.max_active = max_active_requests
         self.budget = max_batch_tokens
@@ -123,148 +129,93 @@ class Scheduler:
         self.row_tile = row_tile          # 0: steps are not trimmed to whole tiles of rows
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []
-        self._admissions = 0
         self.preemption_count = 0
+        self._lib = host.load()
+        self._s = self._lib.apc_sched_new(cache.handle, max_active_requests, max_batch_tokens, chunk_tokens, row_tile)
+        if not self._s:
+            raise ValueError("the scheduler needs max_active_requests, max_batch_tokens and chunk_tokens above 0")
+        self._by_cid: Dict[int, Request] = {}
+        cap = max_active_requests + 8
+        self._items = (ctypes.c_longlong * (4 * cap))()
+        self._pre = (ctypes.c_longlong * cap)()
+        self._adm = (ctypes.c_longlong * cap)()
+        self._orders = (ctypes.c_int * cap)()
+        self._n = (ctypes.c_int * 3)()
+        self._cap = cap
+
+    def __del__(self):
+        if getattr(self, "_s", None):
+            self._lib.apc_sched_free(self._s)
+            self._s = None
 
     # ---- intake ----------------------------------------------------------------
     def add(self, req: Request) -> None:
-        need = self.cache.pages_for_tokens(len(req.prompt) + req.params.max_tokens)
-        for g in self.cache.paged_groups:
-            window = getattr(g.need, "window", None)
-            window_pages = None if window is None else self.cache.pages_for_tokens(window) + 1
-            worst = need if window_pages is None else min(need, window_pages + self.cache.pages_for_tokens(self.chunk))
-            if worst > g.pool.num_pages:
-                raise RequestTooLarge(
-                    f"request {req.id}: {len(req.prompt)} prompt + {req.params.max_tokens} new tokens need {worst} "
-                    f"pages of {self.cache.page_tokens} positions, the whole pool has {g.pool.num_pages}")
+        group = ctypes.c_int(0)
+        worst = self._lib.apc_sched_too_large(self._s, len(req.prompt), req.params.max_tokens, ctypes.byref(group))
+        if worst:
+            raise RequestTooLarge(
+                f"request {req.id}: {len(req.prompt)} prompt + {req.params.max_tokens} new tokens need {worst} "
+                f"pages of {self.cache.page_tokens} positions, the whole pool has "
+                f"{self.cache.paged_groups[group.value].pool.num_pages}")
         if not req.prompt:
             raise ValueError("a request needs at least one prompt token")
         req.status = WAITING
+        req._cid = self.cache.new_id()      # its name in the cache manager's books, through every admission
+        if self._lib.apc_sched_add(self._s, req._cid, len(req.prompt), len(req.output), req.params.max_tokens):
+            raise ValueError(f"request {req.id} cannot be added")
+        self._by_cid[req._cid] = req
         self.waiting.append(req)
 
     def has_work(self) -> bool:
         return bool(self.waiting or self.running)
 
     # ---- one step's plan -------------------------------------------------------
-    def _fits(self, req: Request, n: int, promised: List[int]) -> bool:
-        need = self.cache.pages_needed(req.id, n)
-        return all(need[g] + promised[g] <= self.cache.free_pages(g) for g in range(len(need)))
-
-    def _promise(self, req: Request, n: int, promised: List[int]) -> None:
-        for g, k in enumerate(self.cache.pages_needed(req.id, n)):
-            promised[g] += k
-
-    def _preempt(self, victim: Request, plan: Plan) -> None:
-        self.cache.release(victim.id)
-        self.running.remove(victim)
-        victim.status = WAITING
-        victim.computed = 0
-        victim.preemptions += 1
-        self.preemption_count += 1
-        self.waiting.appendleft(victim)
-        plan.preempted.append(victim)
-
     def plan(self) -> Plan:
-        plan = self._plan_once(Plan())
-        while not plan.scheduled and len(self.running) > 1:
-            # Nobody can advance: the requests in their prompts hold all pages between them.  The newest gives its
-            # pages back (it is not admitted again in this step), until the oldest can go on.
-            self._preempt(max(self.running, key=lambda r: r.order), plan)
-            plan = self._plan_once(plan)
-        return plan
-
-    def _plan_once(self, plan: Plan) -> Plan:
-        """Fills `plan.scheduled` (from nothing); what `plan` lists as preempted and admitted so far stays."""
-        plan.scheduled = []
-        budget = self.budget
-        promised = [0] * len(self.cache.paged_groups)
-        # 1. decodes, oldest admission first.  If a page is missing, the newest running request that is not
-        #    yet part of this step gives way, be it the asking request itself.
-        for req in sorted([r for r in self.running if r.decoding], key=lambda r: r.order):
-            if req.status != RUNNING or budget <= 0:
-                continue
-            while req.status == RUNNING and not self._fits(req, 1, promised):
-                victims = [r for r in self.running if all(s.request is not r for s in plan.scheduled)]
-                if victims == [req] and len(self.running) == 1:
-                    raise RequestTooLarge(f"request {req.id} cannot get a page although it runs alone")
-                self._preempt(max(victims, key=lambda r: r.order), plan)
-            if req.status != RUNNING:
-                continue
-            self._promise(req, 1, promised)
-            plan.scheduled.append(Scheduled(req, req.computed, 1, True))
-            budget -= 1
-        # 2. portions of prompts that are under way
-        for req in sorted([r for r in self.running if not r.decoding], key=lambda r: r.order):
-            if budget <= 0:
-                break
-            if req.status != RUNNING:
-                continue
-            n = min(req.left, self.chunk, budget)
-            while n > 0 and not self._fits(req, n, promised):
-                n = self._shrink(req, n, promised)
-            if n <= 0:
-                continue
-            self._promise(req, n, promised)
-            plan.scheduled.append(Scheduled(req, req.computed, n, n == req.left))
-            budget -= n
-        # 3. admissions, in arrival order; the first that does not fit blocks the ones behind it
-        while self.waiting and budget > 0 and len(self.running) < self.max_active:
-            req = self.waiting[0]
-            if req in plan.preempted:
-                break  # it was just preempted for lack of pages; it comes back in a later step
-            slot_ok = self.cache.slots.free_count > 0
-            if not slot_ok:
-                break
-            self.cache.admit(req.id)
-            n = min(req.left, self.chunk, budget)
-            while n > 0 and not self._fits(req, n, promised):
-                n = self._shrink(req, n, promised)
-            if n <= 0:
-                self.cache.release(req.id)
-                break
-            self.waiting.popleft()
+        L = self._lib
+        code = L.apc_sched_plan(self._s, self._items, self._cap, self._pre, self._adm, self._orders, self._cap, self._n)
+        if code == -40:
+            raise RequestTooLarge("a request cannot get a page although it runs alone")
+        if code:
+            raise RuntimeError(f"the scheduler failed with code {code}")
+        n_sched, n_pre, n_adm = self._n[0], self._n[1], self._n[2]
+        plan = Plan()
+        for i in range(n_pre):       # in the order they gave way: each goes to the front of the queue
+            victim = self._by_cid[self._pre[i]]
+            self.cache.forget(victim.id)
+            self.running.remove(victim)
+            victim.status = WAITING
+            victim.computed = 0
+            victim.preemptions += 1
+            self.preemption_count += 1
+            self.waiting.appendleft(victim)
+            plan.preempted.append(victim)
+        for i in range(n_adm):       # from the front of the queue, in arrival order
+            req = self.waiting.popleft()
+            if req._cid != self._adm[i]:
+                raise RuntimeError("the scheduler's queue and its mirror disagree")
+            self.cache.remember(req.id, req._cid)
             req.status = RUNNING
-            self._admissions += 1
-            req.order = self._admissions
+            req.order = self._orders[i]
             self.running.append(req)
             plan.admitted.append(req)
-            self._promise(req, n, promised)
-            plan.scheduled.append(Scheduled(req, req.computed, n, n == req.left))
-            budget -= n
-        self._trim_to_tiles(plan)
+        it = self._items
+        for i in range(n_sched):
+            plan.scheduled.append(Scheduled(self._by_cid[it[4 * i]], int(it[4 * i + 1]), int(it[4 * i + 2]),
+                                            bool(it[4 * i + 3])))
+        if n_pre:
+            self.cache._tell_frees()
         return plan
-
-    def _trim_to_tiles(self, plan: Plan) -> None:
-        """Cuts the last prompt portion back when the step's rows overshoot a multiple of `row_tile` by up to a quarter
-        of a tile (two tiles or more remain, and at least half of the portion)."""
-        if not self.row_tile:
-            return
-        total = sum(s.count for s in plan.scheduled)
-        over = total % self.row_tile
-        if total < 2 * self.row_tile or not 0 < over <= self.row_tile // 4:
-            return
-        for s in reversed(plan.scheduled):
-            if not s.request.decoding and 2 * (s.count - over) >= s.count:
-                s.count -= over
-                s.samples = False
-                return
-
-    def _shrink(self, req: Request, n: int, promised: List[int]) -> int:
-        """The largest portion below n that the free pages allow (0 if none)."""
-        P = self.cache.page_tokens
-        room = min(self.cache.free_pages(g) - promised[g] for g in range(len(promised))) if promised else 0
-        have = min((len(self.cache.block_table(req.id, g)) for g in range(len(promised))), default=0)
-        can = (have + max(room, 0)) * P - self.cache.length(req.id)
-        return max(0, min(n - 1, can))
 
     # ---- after the step ----------------------------------------------------------
     def advance(self, s: Scheduled) -> None:
         s.request.computed += s.count
+        self._lib.apc_sched_advance(self._s, s.request._cid, s.count)
 
     def append_token(self, req: Request, token: int) -> Optional[str]:
         """Adds a sampled token; returns the finish reason if the request ends with it
         (stop id -> stop, `max_tokens` reached -> length; crates/allpaca-core/src/engine.rs:4607-4621)."""
         req.output.append(int(token))
+        self._lib.apc_sched_token(self._s, req._cid)
         if int(token) in req.params.stop_token_ids:
             return FinishReason.STOP
         if len(req.output) >= req.params.max_tokens:
@@ -277,8 +228,12 @@ class Scheduler:
         req.finish_reason = reason
         if req in self.running:
             self.running.remove(req)
-        if req.id in self.cache:
-            self.cache.release(req.id)
+        cid = getattr(req, "_cid", None)
+        if cid is not None and cid in self._by_cid:
+            del self._by_cid[cid]
+            self._lib.apc_sched_finish(self._s, cid)       # releases what it holds in the cache
+            self.cache.forget(req.id)
+            self.cache._tell_frees()
 
     def abort(self, req: Request) -> None:
         if req in self.waiting:

@@ -26,10 +26,10 @@ LIBS: Dict[str, List[str]] = {
     "plain": ["plain_ops.hip", "plain_gemm.hip", "plain_attention.hip", "sampling.hip"],
     "tuned": ["gemm_bf16.hip", "gemm_wide_bf16.hip", "gemm_direct_bf16.hip", "skinny_gemm_bf16.hip", "attention_bf16.hip", "attention_wide_bf16.hip", "rope_bf16.hip",
               "probe.hip"],
-    "host": ["host/exec.cpp"],
+    "host": ["host/exec.cpp", "host/cache.cpp", "host/pack.cpp", "host/sched.cpp"],
 }
 HEADERS = ["common.h", "mfma.h", "gemm_wide.h", "gemm_direct.h", "attention_wide.h", "no_alloc.h",
-           "host/host.h", "host/kernels.h", "host/rules.h"]
+           "host/host.h", "host/kernels.h", "host/rules.h", "host/cache.h"]
 # libraries a library is linked against (built first; found at run time beside it)
 NEEDS: Dict[str, List[str]] = {"host": ["plain", "tuned"]}
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wno-unused-value", "-Wno-unused-result"]

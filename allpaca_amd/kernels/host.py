@@ -37,6 +37,16 @@ class ApcStep(Structure):
                    ("max_decode_context", c_int), ("all_rows_decode", c_int), ("max_prompt_keys", c_int)])
 
 
+class ApcStepFinding(Structure):
+    _fields_ = [("what", c_int), ("entry", c_int), ("value", c_int), ("extra", c_int)]
+
+
+class ApcPacked(Structure):
+    _fields_ = [("T", c_int), ("S", c_int), ("R", c_int), ("n_decode", c_int), ("n_tiles", c_int), ("total", c_int),
+                ("off", c_int * 11), ("n_groups", c_int), ("table_off", c_int * 8), ("table_width", c_int * 8),
+                ("max_decode_context", c_int), ("max_prompt_keys", c_int), ("max_context", c_int), ("max_rows", c_int)]
+
+
 class ApcTunables(Structure):
     _fields_ = [("whole_min_pairs", c_int), ("last_block_merges", c_int), ("wide_tiles", c_int),
                 ("key_splits_max", c_int), ("key_range_min", c_int), ("force_plain", c_int)]
@@ -61,11 +71,36 @@ _lib.SIGNATURES["host"].update({
     "apc_host_rule_keys_per_part": [I, I, I, I],
     "apc_host_rule_keys_per_wave_whole": [I, I],
     "apc_host_rule_key_splits": [I, I, I, I, I, I],
+    # ---- the cache manager's books
+    "apc_pool_new": [I], "apc_pool_free": [P], "apc_pool_alloc": [P], "apc_pool_give_back": [P, I],
+    "apc_pool_free_count": [P], "apc_pool_pages": [P], "apc_pool_allocations": [P],
+    "apc_pool_held": [P, POINTER(c_int), I], "apc_pool_log_frees": [P, I], "apc_pool_drain": [P, POINTER(c_int), I],
+    "apc_cache_new": [I, I, POINTER(c_int), POINTER(c_int), I], "apc_cache_free": [P], "apc_cache_pool": [P, I],
+    "apc_cache_admit": [P, c_longlong], "apc_cache_release": [P, c_longlong],
+    "apc_cache_reserve": [P, c_longlong, I], "apc_cache_commit": [P, c_longlong, I],
+    "apc_cache_truncate": [P, c_longlong, I], "apc_cache_length": [P, c_longlong], "apc_cache_slot": [P, c_longlong],
+    "apc_cache_version": [P, c_longlong], "apc_cache_pages_needed": [P, c_longlong, I, POINTER(c_int)],
+    "apc_cache_table": [P, c_longlong, I, POINTER(c_int), I], "apc_cache_check": [P], "apc_cache_why": [P],
+    # ---- the step packer (array arguments as addresses: numpy arrays' `ctypes.data`)
+    "apc_step_prepare": [P, I, I, I, P, P, P, P, P, POINTER(ApcStepFinding)],
+    "apc_step_commit": [P, I, P, P],
+    "apc_pack_layout": [P, I, P, P, P, I, I, POINTER(ApcPacked)],
+    "apc_pack_step": [P, I, P, P, P, P, P, I, I, P, P, I, POINTER(ApcPacked)],
+    # ---- the scheduler
+    "apc_sched_new": [P, I, I, I, I], "apc_sched_free": [P], "apc_sched_too_large": [P, I, I, POINTER(c_int)],
+    "apc_sched_add": [P, c_longlong, I, I, I],
+    "apc_sched_plan": [P, POINTER(c_longlong), I, POINTER(c_longlong), POINTER(c_longlong), POINTER(c_int), I,
+                       POINTER(c_int)],
+    "apc_sched_advance": [P, c_longlong, I], "apc_sched_token": [P, c_longlong], "apc_sched_finish": [P, c_longlong],
+    "apc_sched_counts": [P, POINTER(c_int)],
 })
 _lib.RESTYPES.update({
     "apc_host_program_new": c_void_p, "apc_host_program_free": None, "apc_host_program_tunables": None,
     "apc_host_step_bytes": c_longlong, "apc_host_residual_offset": c_longlong, "apc_host_timing": None,
     "apc_host_timing_report": c_char_p,
+    "apc_pool_new": c_void_p, "apc_pool_free": None, "apc_pool_allocations": c_longlong, "apc_pool_log_frees": None,
+    "apc_cache_new": c_void_p, "apc_cache_free": None, "apc_cache_pool": c_void_p, "apc_cache_version": c_longlong,
+    "apc_cache_why": c_char_p, "apc_sched_new": c_void_p, "apc_sched_free": None,
 })
 
 ERRORS = {-10: "the work space is too small for this step", -11: "calls out of order (no step was begun)"}
