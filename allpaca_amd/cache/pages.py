@@ -149,17 +149,19 @@ class StateGroup:
 def group_needs(needs: Sequence[CacheNeed]) -> Tuple[List[Tuple[CacheNeed, List[int]]], List[Tuple[CacheNeed, List[int]]]]:
     """Plan entries sorted by what they need: ([(need of kind "pages", entries)], [(need of kind "slot", entries)]).
     Equal needs share a group; a need is any object with the members `parts.base` lists."""
-    paged: Dict[CacheNeed, List[int]] = {}
-    state: Dict[CacheNeed, List[int]] = {}
-    for i, n in enumerate(needs):
-        try:
-            kind = need_kind(n)
-        except TypeError as e:
-            raise TypeError(f"plan entry {i}: {e}") from None
-        if kind == "pages":
-            paged.setdefault(n, []).append(i)
-        elif kind == "slot":
-            state.setdefault(n, []).append(i)
+    paged: Dict[CacheNeed, list] = {}
+    state: Dict[CacheNeed, list] = {}
+    for i, asked in enumerate(needs):
+        # one need of the entry, or a dict role -> need: its parts are then stored under (entry, role)
+        for key, n in ([((i, role), n) for role, n in asked.items()] if isinstance(asked, dict) else [(i, asked)]):
+            try:
+                kind = need_kind(n)
+            except TypeError as e:
+                raise TypeError(f"plan entry {i}: {e}") from None
+            if kind == "pages":
+                paged.setdefault(n, []).append(key)
+            elif kind == "slot":
+                state.setdefault(n, []).append(key)
     return list(paged.items()), list(state.items())
 
 

@@ -95,20 +95,23 @@ class CacheStorage:
 
     def views(self, plan) -> list:
         """One view per plan entry (None for an entry without a cache)."""
+        def view(loc, writes: bool):
+            kind, gi, li = loc
+            if kind == "paged":
+                need = self.manager.paged_groups[gi].need
+                return PagedView(self.paged[gi][li], self.manager.page_tokens, getattr(need, "window", None), writes, gi)
+            return StateView(self.state[gi][li], writes, gi)
+
         out = []
         for i, e in enumerate(plan):
             owner = i if e.cache_of is None else e.cache_of
             loc = self.manager.location.get(owner)
-            if loc is None:
-                out.append(None)
+            if loc is not None:
+                out.append(view(loc, e.cache_of is None))
                 continue
-            kind, gi, li = loc
-            if kind == "paged":
-                need = self.manager.paged_groups[gi].need
-                out.append(PagedView(self.paged[gi][li], self.manager.page_tokens, getattr(need, "window", None),
-                                     e.cache_of is None, gi))
-            else:
-                out.append(StateView(self.state[gi][li], e.cache_of is None, gi))
+            # several parts of the entry keep a cache: a dict role -> view
+            roles = {k[1]: v for k, v in self.manager.location.items() if isinstance(k, tuple) and k[0] == owner}
+            out.append({role: view(loc, e.cache_of is None) for role, loc in roles.items()} or None)
         return out
 
     def zero_slot(self, slot: int) -> None:

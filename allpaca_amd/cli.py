@@ -49,6 +49,9 @@ def build_parser() -> argparse.ArgumentParser:
     g.add_argument("--max-batch-tokens", type=int)
     g.add_argument("--max-active-requests", type=int)
     g.add_argument("--json", action="store_true", help="print one JSON object per prompt")
+    g.add_argument("--dump-logits", metavar="FILE",
+                   help="append the logits every token is chosen from to FILE, a vocabulary per token as little-endian "
+                        "float32 (what ALLPACA_LOGITS_DUMP=FILE does for any program)")
     r = sub.add_parser("replay", help="trace replay (same as bin/trace_run)")
     r.add_argument("rest", nargs=argparse.REMAINDER)
     b = sub.add_parser("bench", help="decode and prefill throughput (same as bench.py)")
@@ -118,6 +121,8 @@ def cmd_generate(args) -> int:
     else:
         print("allpaca-amd: give --model DIR or --synthetic [PRESET]", file=sys.stderr)
         return 2
+    if args.dump_logits:
+        engine._dump_path = args.dump_logits
     t0 = time.time()
     outs = engine.generate(prompts, gp)
     dt = time.time() - t0
@@ -131,7 +136,9 @@ def cmd_generate(args) -> int:
             print(" ".join(str(t) for t in o.token_ids))
     n = sum(o.completion_tokens for o in outs)
     print(f"{n} tokens in {dt:.3f} s ({n / dt:.1f} tok/s), {engine.stats['steps']} steps, "
-          f"{engine.stats['preemptions']} preemptions", file=sys.stderr)
+          f"{engine.stats['preemptions']} preemptions, {engine.stats['prefill_portions']} prompt portions, "
+          f"{engine.stats['graph_replays']} graph replays, at most {engine.stats['pages_in_use_peak']} pages in use",
+          file=sys.stderr)
     return 0
 
 

@@ -4,7 +4,9 @@ the scheduler and the sampler, and offers the reference's calls
 crates/allpaca-core/src/engine.rs:2895, 3002, 3167, 3650, 3661)."""
 from __future__ import annotations
 
+import os
 import shutil
+import sys
 import tempfile
 import time
 from typing import Dict, Iterator, List, Mapping, Optional, Sequence
@@ -58,7 +60,15 @@ class Engine:
         self.requests: Dict[int, Request] = {}
         self._ahead: Optional[_AheadStep] = None
         self._next_id = 0
-        self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0}
+        # counters (the reference's: prefill chunks, forwards, batched rows, pages in use,
+        # crates/allpaca-core/src/engine.rs:4656-4679, 5099-5101, 5644-5649)
+        self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0, "prefill_portions": 0,
+                      "batched_rows": 0, "graph_replays": 0, "pages_in_use": 0, "pages_in_use_peak": 0}
+        # the logits that tokens are chosen from, kept for whoever asks (`tap_logits`), appended to a file
+        # (ALLPACA_LOGITS_DUMP=<file>) or their two largest printed (ALLPACA_LOGIT_TRACE=1)
+        self._tap: Optional[list] = None
+        self._dump_path = os.environ.get("ALLPACA_LOGITS_DUMP") or None
+        self._trace_top2 = os.environ.get("ALLPACA_LOGIT_TRACE") == "1"
 
     @staticmethod
     def pages_that_fit(model, cfg: EngineConfig) -> int:
@@ -139,6 +149,37 @@ class Engine:
     def has_unfinished(self) -> bool:
         return self.scheduler.has_work()
 
+    # ---- the logits behind the tokens ----------------------------------------------------------------------
+    def tap_logits(self, on: bool = True) -> None:
+        """Keep a copy of the logits every sampled token is chosen from (or stop and drop them), so that two runs'
+        distributions can be compared (the reference's `tap_logits`, crates/allpaca-core/src/engine.rs:1179-1183).
+        While it is on, every step waits for its logits to reach the host."""
+        self._tap = [] if on else None
+
+    def take_tapped_logits(self) -> List[tuple]:
+        """The logits tapped since the last call, in the order the tokens were chosen: (request id, index of the
+        generated token in its request, float32 array [vocab]) each (crates/allpaca-core/src/engine.rs:1185-1189)."""
+        out, self._tap = (self._tap or []), ([] if self._tap is not None else None)
+        return out
+
+    def _observe_logits(self, logits, sampled, extra: int) -> None:
+        """The tap, the dump file and the trace of the two largest logits (crates/allpaca-core/src/sampling.rs:84-127:
+        `ALLPACA_LOGIT_TRACE`, `ALLPACA_LOGITS_DUMP`, a vocabulary per sampled token as little-endian float32)."""
+        rows = logits[:len(sampled)].float().cpu().numpy()
+        for s, row in zip(sampled, rows):
+            if self._tap is not None:
+                self._tap.append((s.request.id, len(s.request.output) + extra, row.copy()))
+            if self._trace_top2:
+                top = row.argsort()[-2:][::-1] if row.size > 1 else [0, 0]
+                print(f"logit_trace {int(top[0])} {row[top[0]]:.6f} {int(top[1])} {row[top[1]]:.6f}", file=sys.stderr)
+        if self._dump_path:
+            try:
+                with open(self._dump_path, "ab") as f:
+                    f.write(rows.astype("<f4").tobytes())
+            except OSError as e:
+                print(f"ALLPACA_LOGITS_DUMP: cannot write {self._dump_path}: {e}", file=sys.stderr)
+                self._dump_path = None
+
     # ---- one tick ---------------------------------------------------------------
     def step(self) -> List[TokenEvent]:
         """One batch through the model: every decoding request advances by a token, prompts by a portion.
@@ -167,10 +208,17 @@ class Engine:
             logits = self.runner.step(entries)
             sampled_all = [s for s in scheduled if s.samples]
             pending = self._launch_sampling(logits, sampled_all, 0) if sampled_all else None
+        st = self.stats
         for s in scheduled:
             self.scheduler.advance(s)
-            self.stats["decode_tokens" if s.request.output and s.count == 1 else "prefill_tokens"] += s.count
-        self.stats["steps"] += 1
+            decode = bool(s.request.output) and s.count == 1
+            st["decode_tokens" if decode else "prefill_tokens"] += s.count
+            st["prefill_portions"] += 0 if decode else 1
+            st["batched_rows"] += s.count
+        st["steps"] += 1
+        cache = self.runner.cache
+        st["pages_in_use_peak"] = max(st["pages_in_use_peak"],
+                                      sum(g.pool.num_pages - g.pool.free_count for g in cache.paged_groups))
         events: List[TokenEvent] = []
         if pending is not None:
             if ahead is None or not ahead.dead:
@@ -189,11 +237,15 @@ class Engine:
                         self._ahead.dead.add(s.request.id)    # its row of the queued step counts for nothing
             if self._ahead is not None and all(s.request.id in self._ahead.dead for s in self._ahead.scheduled):
                 self._ahead = None
+        st["graph_replays"] = self.runner.graph_replays
+        st["pages_in_use"] = sum(g.pool.num_pages - g.pool.free_count for g in cache.paged_groups)
         return events
 
     def _launch_sampling(self, logits, sampled, extra: int):
         """Queues the choice of a token for every row; `extra`: tokens of each request that are on their way and
         not appended yet (they count for the index of the random number)."""
+        if self._tap is not None or self._dump_path or self._trace_top2:
+            self._observe_logits(logits, sampled, extra)
         return self.sampler.launch(logits, [s.request.params for s in sampled],
                                    [len(s.request.output) + extra for s in sampled])
 

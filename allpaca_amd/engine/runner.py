@@ -249,12 +249,13 @@ class ModelRunner:
         return self.model.forward(info, self.bind_views(info))
 
     def bind_views(self, info: StepInfo) -> list:
-        for v in self.views:
-            if isinstance(v, PagedView):
-                v.block_table = info.block_tables[v.group]
-            elif isinstance(v, StateView):
-                v.slots = info.state_slots
-                v.slots_host = info.host_slots
+        for entry in self.views:
+            for v in (entry.values() if isinstance(entry, dict) else (entry,)):
+                if isinstance(v, PagedView):
+                    v.block_table = info.block_tables[v.group]
+                elif isinstance(v, StateView):
+                    v.slots = info.state_slots
+                    v.slots_host = info.host_slots
         return self.views
 
     # ---- decode-only steps as HIP graphs -----------------------------------------------

@@ -57,10 +57,13 @@ class DecoderModel:
 
     # ---- cache needs, one per plan entry -------------------------------------
     def cache_needs(self) -> List[CacheNeed]:
-        """What each plan entry needs of the cache manager (None for an entry that borrows)."""
+        """What each plan entry needs of the cache manager: None (it borrows, or keeps nothing), one need (only the
+        part in the role "mixer" keeps something: the cache view goes to the arrangement as it is), or a dict
+        role -> need (the arrangement gets a dict role -> view)."""
         needs: List[CacheNeed] = []
         for e in self.spec.plan:
-            needs.append(None if e.cache_of is not None else self.blocks[e.block].mixer.cache_need())
+            asked = {} if e.cache_of is not None else self.blocks[e.block].cache_needs()
+            needs.append(None if not asked else asked["mixer"] if list(asked) == ["mixer"] else asked)
         return needs
 
     # ---- one step ------------------------------------------------------------

@@ -41,6 +41,18 @@ class Block:
     def mixer(self):
         return self.parts["mixer"]
 
+    def cache_needs(self) -> Dict[str, object]:
+        """role -> what that part needs of the cache manager, for every part of the layer that keeps something per
+        request (`cache_need()` answering other than None): attention heads beside recurrent heads are two roles with
+        a need each."""
+        out = {}
+        for role, part in self.parts.items():
+            ask = getattr(part, "cache_need", None)
+            need = ask() if callable(ask) else None
+            if need is not None:
+                out[role] = need
+        return out
+
     def native_desc(self):
         describe = getattr(self.arrangement, "native_desc", None)
         return describe(self.parts) if describe is not None else None
@@ -82,6 +94,8 @@ class PreNorm:
     @staticmethod
     def run(parts, x: torch.Tensor, step, cache, pre=None, next_norm=None):
         mixer, ffn = parts["mixer"], parts["ffn"]
+        if isinstance(cache, dict):      # a layer with several parts that keep a cache: each gets its own
+            cache = cache.get("mixer")
         rt = mixer.rt
         h = NormedInput(x, parts["mixer_norm"], rt.dtype, pre)
         emit = NormEmit.of(parts["ffn_norm"]) if mixer.emits_next_norm and ffn.takes_normed_input else None

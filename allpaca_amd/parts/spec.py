@@ -43,6 +43,10 @@ class ParamSpec:
     store: str = "compute"
     optional: bool = False
     alias_of: Optional[str] = None   # full name of another tensor to use when this one is absent by design
+    # How random weights are drawn for this tensor: "normal" (N(0, std)), "ones_plus_normal" (1 + N(0, norm_std): a
+    # norm's weight), "zeros", or a number (that constant: a bias, a decay rate).  None: by `store`, "normal" for
+    # "compute", "ones_plus_normal" for "float32", "zeros" for "int32".
+    init: Any = None
 
 
 @dataclass

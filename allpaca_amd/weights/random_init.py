@@ -5,7 +5,8 @@ The reference's synthetic model draws uniform values from one generator in a
 fixed order (crates/allpaca-core/src/model.rs:5061-5125, 13369-13387); here each
 tensor has a generator of its own keyed by (seed, tensor name), so a tensor does
 not depend on which others exist or in which order they are made.  Matrices are
-N(0, std); norm weights are 1 + N(0, norm_std)."""
+N(0, std); norm weights are 1 + N(0, norm_std); a tensor may name its own rule
+(`ParamSpec.init`: a bias that starts at zero, a rate that starts at a constant)."""
 from __future__ import annotations
 
 import hashlib
@@ -32,16 +33,23 @@ def random_tensors(specs: Mapping[str, ParamSpec], seed: int, dtype: torch.dtype
     for name, ps in specs.items():
         g = torch.Generator(device=dev)
         g.manual_seed(_tensor_seed(seed, name))
-        if ps.store == "int32":
-            out[name] = torch.zeros(ps.shape, dtype=torch.int32, device=dev)
-        elif ps.store == "float32":
+        want = stored_dtype(ps, dtype)
+        init = ps.init
+        if init is None:
+            init = {"int32": "zeros", "float32": "ones_plus_normal"}.get(ps.store, "normal")
+        if isinstance(init, (int, float)) and not isinstance(init, bool):
+            t = torch.full(ps.shape, float(init), dtype=torch.float32, device=dev)
+        elif init == "zeros":
+            t = torch.zeros(ps.shape, dtype=torch.float32, device=dev)
+        elif init == "ones_plus_normal":
             t = torch.ones(ps.shape, dtype=torch.float32, device=dev)
             if norm_std:
                 t += norm_std * torch.randn(ps.shape, generator=g, dtype=torch.float32, device=dev)
-            out[name] = t
-        else:
+        elif init == "normal":
             t = torch.randn(ps.shape, generator=g, dtype=torch.float32, device=dev) * std
-            out[name] = t.to(dtype)
+        else:
+            raise ValueError(f"tensor {name!r}: init {init!r} is not 'normal', 'ones_plus_normal', 'zeros' or a number")
+        out[name] = t.to(want)
     return out
 
 

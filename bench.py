@@ -89,8 +89,15 @@ def weight_bytes(eng):
     return total
 
 
-def kv_bytes_per_token(cfg, layers, elem=2):
-    return layers * 2 * cfg.num_key_value_heads * cfg.head_dim * elem
+def kv_bytes_per_token(eng):
+    """Bytes of cache that one more token of a request takes over all layers: what the engine's own estimate of its
+    cache says (`CacheEstimate`, from the needs that the model's parts state), a page's bytes over its positions."""
+    import torch
+    from allpaca_amd.cache import CacheEstimate
+    page = eng.config.page_tokens
+    elem = torch.empty((), dtype=eng.runner.storage.paged[0].dtype).element_size()
+    est = CacheEstimate.of(eng.model.cache_needs(), page, elem)
+    return est.bytes_per_page_of_every_group / page
 
 
 def decode_during_prefill(batch, context, chunk=2048):
@@ -317,7 +324,7 @@ def kernel_times(cfg_json, args, layers):
     with klib.timing() as t:
         for _ in range(steps):
             eng.step()
-    kv = kv_bytes_per_token(cfg, layers, 2 if args.dtype == "bf16" else 4)
+    kv = kv_bytes_per_token(eng)
     out[f"decode_b{B}_ctx{ctx}"] = kernel_table(t.totals(), steps, attention_bytes=B * (ctx + 5) * kv)
     # a mixed step: a portion of a new prompt beside the B decoding rows, as long as the scheduler makes it (a chunk of
     # 512 tokens, cut back so that the step's rows are whole tiles); host time = until the launches are queued
@@ -558,7 +565,7 @@ def main() -> int:
             main_hash = decode_run.ids_hash
             wbytes = weight_bytes(eng)
             ctx_mid = args.context + args.warmup + args.steps // 2
-            total = wbytes + b * ctx_mid * kv_bytes_per_token(cfg, layers, 2 if args.dtype == "bf16" else 4)
+            total = wbytes + b * ctx_mid * kv_bytes_per_token(eng)
             gbs = total / sec / 1e9
             roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(gbs / HBM_PEAK_GBS, 4), "measured_peak": round(measured_gbs, 1),

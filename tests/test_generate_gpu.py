@@ -375,3 +375,37 @@ def test_a_cache_larger_than_device_memory_is_refused_with_its_size():
     folder = H.model_folder("A", "float32", True)
     with pytest.raises(CacheTooLarge, match="GiB"):
         Engine(folder, dtype="float32", page_tokens=16, max_tokens=1 << 34)
+
+
+@pytest.mark.parametrize("graphs", [False, True])
+def test_the_logits_behind_the_tokens_can_be_tapped_and_dumped(tmp_path, graphs):
+    """`tap_logits` keeps the logits every token was chosen from (the reference's tap,
+    crates/allpaca-core/src/engine.rs:1179-1189); `ALLPACA_LOGITS_DUMP` / `--dump-logits` appends them to a file
+    (crates/allpaca-core/src/sampling.rs:100-127).  Greedy tokens are the first maxima of their tapped rows, the rows
+    are the plain implementation's logits, and steps queued ahead are tapped like the others."""
+    folder = H.model_folder("B", "float32", True)
+    cfg, w = H.oracle(folder)
+    prompts = [H.random_tokens(1000, n, seed=n) for n in (5, 19)]
+    eng = engine_for(folder, use_graphs=graphs)
+    eng._dump_path = str(tmp_path / "logits.f32")
+    eng.tap_logits(True)
+    outs = eng.generate(prompts, params(max_tokens=7, temperature=0.0))
+    tapped = eng.take_tapped_logits()
+    assert len(tapped) == 14 and eng.take_tapped_logits() == []
+    by_request = {}
+    for rid, index, row in tapped:
+        by_request.setdefault(rid, []).append((index, row))
+    for (rid, rows), p, o in zip(sorted(by_request.items()), prompts, outs):
+        assert [i for i, _ in rows] == list(range(7))
+        assert [int(np.argmax(r)) for _, r in rows] == o.token_ids
+        want = P.llama_forward(cfg, w, p + o.token_ids[:-1])[len(p) - 1:]
+        assert np.abs(np.stack([r for _, r in rows]) - want).max() < H.F32_ATOL
+    dumped = np.fromfile(tmp_path / "logits.f32", dtype="<f4").reshape(-1, 1000)
+    assert dumped.shape[0] == 14 and np.array_equal(dumped, np.stack([r for _, _, r in tapped]))
+    eng.tap_logits(False)
+    eng._dump_path = None
+    eng.generate(prompts[:1], params(max_tokens=2, temperature=0.0))
+    assert eng.take_tapped_logits() == []
+    st = eng.stats
+    assert st["prefill_portions"] == 3 and st["batched_rows"] == st["prefill_tokens"] + st["decode_tokens"]
+    assert st["pages_in_use"] == 0 and st["pages_in_use_peak"] >= 2 and (st["graph_replays"] > 0) == graphs

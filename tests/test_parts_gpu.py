@@ -605,3 +605,152 @@ def test_a_feed_forward_that_plans_on_the_host_keeps_the_model_out_of_graphs():
         lg = runner.step([Entry("a", [toks["a"][10 + j]], [0]), Entry("b", [toks["b"][5 + j]], [0])]).cpu().numpy()
         assert np.abs(lg[0] - want["a"][10 + j]).max() < 1e-4 and np.abs(lg[1] - want["b"][5 + j]).max() < 1e-4, j
     assert runner.graph_replays == 0
+
+
+# --------------------------------------------------------------------------------------------------
+# a third toy architecture: a layer with two parts that each keep something per request (attention heads beside a
+# decaying state, in an arrangement of the test's own), and a bias kept in 32-bit that starts at a constant
+# --------------------------------------------------------------------------------------------------
+def register_toy3():
+    from allpaca_amd.models import ARCHITECTURES, Architecture
+    from allpaca_amd.parts import (ARRANGEMENTS, FEED_FORWARDS, MIXERS, NORMS, BlockSpec, FixedState, Mixer, ModelSpec,
+                                   ParamSpec, PartSpec, PlanEntry)
+    register_toy()
+    if "toy_decay_bias" in MIXERS:
+        return
+
+    @MIXERS.register("toy_decay_bias")
+    class DecayBiasMixer(Mixer):
+        """s <- decay * s + h_row + bias, row after row; out = s W^T.  The bias is stored in 32-bit and random weights
+        start it at 0.25 (not at 1 + noise, which is what a norm's weight gets)."""
+
+        def __init__(self, hidden_size, decay):
+            self.D, self.decay = hidden_size, decay
+
+        def param_specs(self):
+            return {"mix.weight": ParamSpec((self.D, self.D), store="float32", init="normal"),
+                    "bias": ParamSpec((self.D,), store="float32", init=0.25),
+                    "gate": ParamSpec((self.D,), store="float32", init="zeros")}
+
+        def cache_need(self):
+            return FixedState((self.D,), "float32")
+
+        def bind(self, tensors, rt):
+            self.rt = rt
+            self.w = tensors["mix.weight"].to(rt.device, torch.float32)
+            self.bias = tensors["bias"].to(rt.device, torch.float32)
+            self.gate = tensors["gate"].to(rt.device, torch.float32)
+
+        def forward(self, h, step, cache):
+            out = torch.empty(h.shape[0], self.D, dtype=torch.float32, device=h.device)
+            hf = h.float()
+            for r0, n, slot in zip(step.host_row0, step.host_rows, step.host_slots):
+                s = cache.state[slot].clone()
+                for r in range(r0, r0 + n):
+                    s = self.decay * s + hf[r] + self.bias
+                    out[r] = (s * (1.0 + self.gate)) @ self.w.T
+                if cache.writes:
+                    cache.state[slot] = s
+            return out
+
+    @ARRANGEMENTS.register("toy_two_mixers")
+    class TwoMixers:
+        """x += attention(norm(x)) + recurrent(norm(x)); x += ffn(norm2(x)): two parts with a cache of their own."""
+        registries = {"norm": NORMS, "mixer": MIXERS, "recurrent": MIXERS, "ffn_norm": NORMS, "ffn": FEED_FORWARDS}
+
+        @staticmethod
+        def run(parts, x, step, cache):
+            assert set(cache) == {"mixer", "recurrent"}
+            rt = parts["mixer"].rt
+            h = torch.empty(x.shape, dtype=rt.dtype, device=x.device)
+            parts["norm"].forward(x, h)
+            parts["mixer"].forward_add(h, step, cache["mixer"], x)
+            parts["recurrent"].forward_add(h, step, cache["recurrent"], x)
+            h2 = torch.empty(x.shape, dtype=rt.dtype, device=x.device)
+            parts["ffn_norm"].forward(x, h2)
+            parts["ffn"].forward_add(h2, step, x)
+
+    def describe(c):
+        D, V = c["hidden_size"], c["vocab_size"]
+        norm = dict(size=D, eps=c["eps"])
+        block = BlockSpec("toy_two_mixers", {
+            "norm": PartSpec("rmsnorm", norm, "norm1."),
+            "mixer": PartSpec("attention", dict(hidden_size=D, num_heads=c["heads"], num_kv_heads=c["kv_heads"],
+                                                head_dim=c["head_dim"],
+                                                position=PartSpec("rope", dict(head_dim=c["head_dim"], theta=c["theta"]))),
+                              "attn."),
+            "recurrent": PartSpec("toy_decay_bias", dict(hidden_size=D, decay=c["decay"]), "rec."),
+            "ffn_norm": PartSpec("rmsnorm", norm, "norm2."),
+            "ffn": PartSpec("swiglu", dict(hidden_size=D, intermediate_size=c["ffn"]), "mlp.")}, "toy3.layers.0.")
+        return ModelSpec(D, V, c["max_positions"], PartSpec("token_table", dict(vocab_size=V, hidden_size=D), "toy3.embed."),
+                         [block], [PlanEntry(0), PlanEntry(0)], PartSpec("rmsnorm", norm, "toy3.norm."),
+                         PartSpec("linear", dict(vocab_size=V, hidden_size=D, tied=False), "toy3.head."))
+
+    ARCHITECTURES.register("Toy3ForCausalLM", Architecture("toy3", dict, describe))
+
+
+TOY3 = dict(architectures=["Toy3ForCausalLM"], vocab_size=60, hidden_size=32, heads=2, kv_heads=1, head_dim=16, ffn=40,
+            eps=1e-5, theta=10000.0, decay=0.6, max_positions=96)
+
+
+def toy3_plain(cfg, w, tokens):
+    T, D = len(tokens), cfg["hidden_size"]
+    Hh, Hk, d = cfg["heads"], cfg["kv_heads"], cfg["head_dim"]
+    x = np.asarray(w["toy3.embed.weight"], np.float64)[tokens]
+    p = "toy3.layers.0."
+    inv = P.rope_inv_freq(d, cfg["theta"])
+    for _ in range(2):      # the block runs twice, each run with caches of its own
+        h = P.rms_norm(x, w[p + "norm1.weight"], cfg["eps"])
+        q = P.rope_neox(P.linear(h, w[p + "attn.q_proj.weight"]).reshape(T, Hh, d), np.arange(T), inv)
+        k = P.rope_neox(P.linear(h, w[p + "attn.k_proj.weight"]).reshape(T, Hk, d), np.arange(T), inv)
+        v = P.linear(h, w[p + "attn.v_proj.weight"]).reshape(T, Hk, d)
+        att = P.linear(P.attention(q, k, v, Hh, Hk).reshape(T, Hh * d), w[p + "attn.o_proj.weight"])
+        s, rec = np.zeros(D), np.zeros((T, D))
+        for t in range(T):
+            s = cfg["decay"] * s + h[t] + w[p + "rec.bias"]
+            rec[t] = (s * (1.0 + w[p + "rec.gate"])) @ w[p + "rec.mix.weight"].T
+        x = x + att + rec
+        h = P.rms_norm(x, w[p + "norm2.weight"], cfg["eps"])
+        x = x + P.swiglu(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    return P.rms_norm(x, w["toy3.norm.weight"], cfg["eps"]) @ w["toy3.head.weight"].T
+
+
+def test_a_layer_with_two_parts_that_keep_a_cache_and_a_bias_in_32_bit():
+    """Defined here and nowhere in the framework: a block whose arrangement has two parts with a cache need each
+    (pages of keys and values, a state slot) and a 32-bit bias whose random start is a constant of its own."""
+    from allpaca_amd.engine.batch import Entry
+    from allpaca_amd.engine.runner import ModelRunner
+    from allpaca_amd.models import load_model
+    from allpaca_amd.weights import write_model_folder
+    register_toy3()
+    folder = os.path.join(H.tmp_root(), "toy3_model")
+    write_model_folder(folder, TOY3, seed=9, dtype=torch.float32, std=0.25, norm_std=0.1)
+    _, w = P.read_model_folder(folder)
+    p = "toy3.layers.0."
+    assert np.all(w[p + "rec.bias"] == 0.25) and np.all(w[p + "rec.gate"] == 0.0)      # ParamSpec.init
+    assert abs(float(np.std(w[p + "rec.mix.weight"])) - 0.25) < 0.05 and abs(float(np.mean(w[p + "rec.mix.weight"]))) < 0.05
+    assert abs(float(np.mean(w[p + "norm1.weight"])) - 1.0) < 0.1                       # a norm's weight: 1 + noise
+    cfg, model = load_model(folder, torch.float32, "cuda:0")
+    needs = model.cache_needs()
+    assert [sorted(n) for n in needs] == [["mixer", "recurrent"]] * 2
+    runner = ModelRunner(model, 4, 40, 3)
+    assert runner.native is None                       # the executor does not know this arrangement: walked in Python
+    assert runner.cache.paged_groups[0].entries == [(0, "mixer"), (1, "mixer")]
+    assert runner.cache.state_groups[0].entries == [(0, "recurrent"), (1, "recurrent")]
+    toks = {"a": H.random_tokens(60, 33, seed=1), "b": H.random_tokens(60, 14, seed=2)}
+    want = {k: toy3_plain(TOY3, w, t) for k, t in toks.items()}
+    got = {k: [] for k in toks}
+    at = {k: 0 for k in toks}
+    for k in toks:
+        runner.admit(k)
+    for batch in ([("a", 9), ("b", 3)], [("a", 1), ("b", 1)], [("a", 20), ("b", 1)], [("b", 9), ("a", 1)], [("a", 2)]):
+        lg = runner.step([Entry(k, toks[k][at[k]:at[k] + n], list(range(n))) for k, n in batch]).cpu().numpy()
+        r = 0
+        for k, n in batch:
+            got[k].append(lg[r:r + n])
+            r += n
+            at[k] += n
+    for k in toks:
+        assert np.abs(np.concatenate(got[k]) - want[k]).max() < 1e-4, k
+        runner.release(k)
+    runner.cache.check()
