@@ -14,11 +14,13 @@ class EngineConfig:
     num_pages: int = 0                 # pages of the cache pool; 0: sized from max_tokens
     max_tokens: int = 0                # tokens the cache pool holds when num_pages is 0; 0 too: sized from memory
     # With neither given, the pool takes `kv_bytes`, or, if that is 0, the device memory that is free once the
-    # weights are loaded minus `kv_reserve_bytes` (room for a step's activations, logits and workspaces); never more
-    # than every one of `max_active_requests` requests at the model's longest context needs
-    # (the reference's budget is `kv.vram_bytes`, crates/allpaca-core/src/engine.rs:8651-8680).
+    # weights are loaded minus `kv_reserve_bytes` (room for a step's activations, logits and workspaces; 0: worked out
+    # from `max_batch_tokens`, `max_active_requests` and the model's widths, `Engine.reserve_bytes`); never more than
+    # every one of `max_active_requests` requests at the model's longest context needs (the reference's budget is
+    # `kv.vram_bytes`, crates/allpaca-core/src/engine.rs:8651-8680).  "Free" is what the device reports when the
+    # engine is built: processes that share a GPU each see the same figure, so give each its `kv_bytes` or `max_tokens`.
     kv_bytes: int = 0
-    kv_reserve_bytes: int = 4 << 30
+    kv_reserve_bytes: int = 0
     max_active_requests: int = 64
     max_batch_tokens: int = 2048       # token budget of one step
     chunk_tokens: int = 512            # largest portion of one prompt in a step

@@ -556,6 +556,17 @@ struct KVRegs {
 // The order of additions for a row depends on its position, KW and the number of parts only.
 constexpr int NW = 4;  // waves of a block of the decode kernel
 enum { DEC_PARTS = 0, DEC_WHOLE = 1, DEC_LAST = 2 };
+// Why the hand-over of DEC_LAST holds without a release/acquire pair.  Every access to a partial result, on either
+// side, is a relaxed atomic of agent scope: on this chip such a store goes through to memory past the block's own L2
+// (sc1) and such a load is served from memory, so neither a write-back of the writer's L2 nor an invalidation of the
+// reader's is needed for these words.  What is left is order: a writer thread's stores are issued before its
+// `s_waitcnt vmcnt(0)`, which returns when memory has acknowledged them; the block's barrier behind it puts all its
+// threads' acknowledged stores before thread 0's add to the counter; the counter's adds are atomics on one word, so the
+// block that reads `nz - 1` adds after every other block's add, hence after their stores were acknowledged; its
+// loads are issued behind its own barrier, which stands behind that add.  The language's memory model does not
+// promise this for relaxed atomics; the instructions they compile to here do (the kernel is built for gfx950 alone).
+// The counters are zero before the first launch and every launch leaves them zero; a launch that dies half-way
+// would leave a count behind, so whoever owns them zeroes them when an engine is set up (engine/native.py).
 __device__ __forceinline__ void st_coh(float* p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -1008,6 +1019,12 @@ APC_EXPORT int apc_attention_decode_bf16(const void* q, int ldq, int q_off, void
 APC_EXPORT int apc_attention_decode_last_fits(int H, int Hk, int d, int n_parts) {
   if (H <= 0 || Hk <= 0 || H % Hk || d <= 0 || n_parts <= 0) return 0;
   return last_fits(H / Hk, d, n_parts) ? 1 : 0;
+}
+
+// 1 if apc_attention_prefill_bf16 sends a step of `n_tiles` tiles with `n_rows` rows in all to the kernel of 128-row
+// blocks (the only one that cuts a tile's keys into ranges and reads `parts`), else 0.
+APC_EXPORT int apc_attention_prefill_wide_takes(int d, int page_tokens, int n_tiles, int n_rows) {
+  return (n_tiles > 0 && attn_wide_takes(d, page_tokens) && (long)n_rows * 2 >= (long)n_tiles * TILE_ROWS) ? 1 : 0;
 }
 
 // Rows of a tile of the prefill kernels: the caller cuts every segment of several rows into tiles of at most this many

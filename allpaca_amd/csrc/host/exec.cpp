@@ -397,7 +397,8 @@ int attention_bf16(Program& P, const Buf& q, const Buf& out, const ApcLayer& L, 
   const int* table = s.table[E.group];
   const int width = s.table_width[E.group];
   if (s.n_tiles) {
-    const int splits = P.tun.wide_tiles
+    const bool wide = P.tun.wide_tiles && apc_attention_prefill_wide_takes(d, page, s.n_tiles, T - s.n_decode);
+    const int splits = wide
                            ? key_splits(s.n_tiles, H, s.max_prompt_keys, window, P.tun.key_splits_max,
                                         std::max(1, P.tun.key_range_min))
                            : 1;

@@ -75,4 +75,5 @@ int apc_attention_decode_bf16(const void* q, int ldq, int q_off, void* out, int 
 int apc_attention_decode_last_fits(int H, int Hk, int d, int n_parts);
 int apc_attention_decode_whole_fits(int H, int Hk, int d);
 int apc_attention_prefill_tile_rows();
+int apc_attention_prefill_wide_takes(int d, int page_tokens, int n_tiles, int n_rows);
 }

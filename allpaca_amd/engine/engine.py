@@ -83,7 +83,7 @@ class Engine:
         if not budget:
             free, _ = torch.cuda.mem_get_info(rt.device)
             free += torch.cuda.memory_reserved(rt.device) - torch.cuda.memory_allocated(rt.device)
-            budget = free - cfg.kv_reserve_bytes
+            budget = free - (cfg.kv_reserve_bytes or Engine.reserve_bytes(model, cfg))
         pages = est.pages_for_budget(budget, cfg.max_active_requests)
         most = cfg.max_active_requests * -(-rt.max_positions // cfg.page_tokens)
         pages = min(pages, most)
@@ -92,6 +92,19 @@ class Engine:
                                 f"(kv_bytes, or free device memory less kv_reserve_bytes), a page over all layers takes "
                                 f"{est.bytes_per_page_of_every_group / 2**20:.2f} MiB")
         return pages
+
+    @staticmethod
+    def reserve_bytes(model, cfg: EngineConfig) -> int:
+        """Device memory kept out of the cache pool when it is sized from what is free: a step's work space (the
+        residual stream and the widest layer's outputs for `max_batch_tokens` rows, in 32-bit terms and twice over for
+        partial sums of products with K in slices), the logits of two decode steps under way and the sampler's scratch
+        for `max_active_requests` rows, and 1 GiB for graphs, pinned staging and the allocator's slack."""
+        spec = model.spec
+        widest = max([sum(ps.shape[0] for ps in b.param_specs().values() if len(ps.shape) == 2 and ps.store == "compute")
+                      for b in model.blocks] or [0])
+        step = cfg.max_batch_tokens * (4 * spec.hidden_size + 4 * widest) * 2
+        out = cfg.max_active_requests * (3 * 4 * spec.vocab_size + (256 << 10))
+        return step + out + (1 << 30)
 
     @classmethod
     def from_model(cls, model_config, model, config: EngineConfig) -> "Engine":

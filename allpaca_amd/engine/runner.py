@@ -54,6 +54,9 @@ class ModelRunner:
         parts = [model.embedding, model.final_norm, model.head] + [p for b in model.blocks for p in b.parts.values()]
         self.use_graphs = bool(use_graphs) and all(getattr(p, "graph_safe", False) for p in parts)
         from ..kernels import ops
+        if self.rt.dtype == torch.bfloat16 and not ops.FORCE_PLAIN:
+            from ..kernels import tuned
+            tuned.check_chip(self.rt.device)
         self.tile_rows = ops.attention_tile_rows(self.rt.dtype)          # how the attention kernel wants longer segments cut
         self.position_axes = int(getattr(model.spec, "position_axes", 1))
         self.graphs: Dict[Tuple[int, int], "DecodeGraph"] = {}

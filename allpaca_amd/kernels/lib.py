@@ -62,6 +62,9 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_attention_decode_last_fits": [I, I, I, I],
         "apc_attention_decode_whole_fits": [I, I, I],
         "apc_attention_prefill_tile_rows": [],
+        "apc_attention_prefill_wide_takes": [I, I, I, I],
+    },
+    "bench": {
         "apc_probe_read": [P, Z, P, I, I, P],
         "apc_probe_mfma": [I, P, I, P],
     },
@@ -103,6 +106,7 @@ class KernelTimer:
 _timer = None
 # entry points that launch nothing (questions about sizes): never timed
 NOT_KERNELS = {"apc_attention_decode_whole_fits", "apc_attention_decode_last_fits", "apc_attention_prefill_tile_rows",
+               "apc_attention_prefill_wide_takes",
                "apc_gemm_direct_k_split", "apc_gemm_direct_emit_parts", "apc_sample_rows_scratch_kib"}
 
 

@@ -10,7 +10,7 @@ from . import ops as _ops
 
 def read_bandwidth(gib: float = 8.0, blocks: int = 256 * 8, unroll: int = 8, repeats: int = 3) -> float:
     """GB/s of reading `gib` GiB of device memory once with 16-byte loads (best of `repeats`)."""
-    L = _lib.load("tuned")
+    L = _lib.load("bench")
     n = int(gib * 2 ** 30) // 16 * 16
     buf = torch.empty(n, dtype=torch.uint8, device="cuda")
     buf.fill_(1)
@@ -30,7 +30,7 @@ def read_bandwidth(gib: float = 8.0, blocks: int = 256 * 8, unroll: int = 8, rep
 
 def mfma_rate(iters: int = 20000, blocks: int = 256 * 4, repeats: int = 2) -> float:
     """TFLOP/s of independent v_mfma_f32_32x32x16_bf16 from registers on every compute unit."""
-    L = _lib.load("tuned")
+    L = _lib.load("bench")
     out = torch.empty(blocks * 256, dtype=torch.float32, device="cuda")
     best = 0.0
     for _ in range(repeats + 1):

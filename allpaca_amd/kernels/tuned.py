@@ -54,6 +54,29 @@ def _tiled_k_split(M: int, N: int, K: int) -> int:
     return _k_split_many_rows(M, N, K) if M <= MANY_ROWS_SPLIT_MAX else 1
 
 
+# The chip these rules and the kernels' launch plans were measured on (`csrc/host/rules.h`, `gemm_direct_bf16.hip`:
+# rounds of 256 blocks over 8 XCDs; `attention_wide_bf16.hip`: 160 KiB of LDS a compute unit).
+CHIP_UNITS = 256
+CHIP_LDS_BYTES = 160 * 1024
+_chips_checked: set = set()
+
+
+def check_chip(device: torch.device) -> None:
+    """Says so, once per device, if the GPU is not the one the dispatch rules were measured on: the results stay
+    right (no kernel assumes the counts for correctness), the cuts may be badly chosen."""
+    import warnings
+    key = (device.type, device.index)
+    if device.type != "cuda" or key in _chips_checked:
+        return
+    _chips_checked.add(key)
+    prop = torch.cuda.get_device_properties(device)
+    units = getattr(prop, "multi_processor_count", CHIP_UNITS)
+    lds = getattr(prop, "shared_memory_per_block_optin", 0) or getattr(prop, "shared_memory_per_block", 0)
+    if units != CHIP_UNITS or (lds and lds < CHIP_LDS_BYTES):
+        warnings.warn(f"{prop.name}: {units} compute units and {lds} bytes of LDS a block; the bfloat16 kernels' dispatch "
+                      f"rules were measured on {CHIP_UNITS} units with {CHIP_LDS_BYTES} bytes and may be badly tuned here")
+
+
 def _aligned(*ts: torch.Tensor) -> bool:
     return all(t.data_ptr() % 16 == 0 for t in ts)
 
@@ -396,7 +419,9 @@ def attention_bf16(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int,
     L = _lib.load("tuned")
     stream = _ops._stream()
     if step.n_tiles:
-        splits = _key_splits(step, n_heads, window) if WIDE_TILES else 1
+        # (only the kernel of 128-row blocks cuts keys into ranges: no room is taken for the others)
+        wide = WIDE_TILES and L.apc_attention_prefill_wide_takes(head_dim, page_tokens, step.n_tiles, T - step.n_decode_rows)
+        splits = _key_splits(step, n_heads, window) if wide else 1
         parts = (torch.empty(splits * T * n_heads * (head_dim + 2), dtype=torch.float32, device=q.device)
                  if splits > 1 else None)
         _lib.check(L.apc_attention_prefill_bf16(

@@ -303,3 +303,33 @@ def test_random_folder_is_reproducible_and_independent_of_other_tensors(tmp_path
     assert abs(a[n].std().item() - 0.02) < 0.002 and torch.all(a["model.norm.weight"] == 1.0)
     cfg, w = P.read_model_folder(str(tmp_path / "a"))      # the plain reader reads what the writer wrote
     assert cfg["hidden_size"] == 64 and np.array_equal(w[n], a[n].double().numpy())
+
+
+def test_random_weights_are_a_function_of_seed_name_and_element():
+    """Every element is a hash of (seed, tensor name, index): the same whatever else is made, in any order, and, the
+    arithmetic being integer up to one float32 multiplication, on any device (tests/test_generate_gpu.py holds the GPU
+    against this).  A few elements against the formula written out with Python integers."""
+    import numpy as np
+    from allpaca_amd.parts import ParamSpec
+    from allpaca_amd.weights.random_init import _tensor_seed, random_tensors, unit_normal
+    M = (1 << 64) - 1
+
+    def element(base, i):
+        x = (i * 0xD6E8FEB86659FD93 + base + 0x9E3779B97F4A7C15) & M
+        z = ((x ^ (x >> 30)) * 0xBF58476D1CE4E5B9) & M
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & M
+        z ^= z >> 31
+        total = (z & 0xFFFF) + ((z >> 16) & 0xFFFF) + ((z >> 32) & 0xFFFF) + (z >> 48)
+        return np.float32(total - 131070) * np.float32((3.0 / (2 ** 32 - 1)) ** 0.5)
+
+    specs = {"a.weight": ParamSpec((33, 7)), "b.weight": ParamSpec((5, 4)), "n.weight": ParamSpec((9,), store="float32")}
+    t = random_tensors(specs, 11, torch.float32, std=0.5, norm_std=0.25)
+    base = _tensor_seed(11, "a.weight")
+    for i in (0, 1, 100, 230):
+        assert float(t["a.weight"].flatten()[i]) == float(element(base, i) * np.float32(0.5))
+    assert float(t["n.weight"][3]) == float(np.float32(1.0) + element(_tensor_seed(11, "n.weight"), 3) * np.float32(0.25))
+    alone = random_tensors({"b.weight": specs["b.weight"]}, 11, torch.float32, std=0.5)
+    assert torch.equal(alone["b.weight"], t["b.weight"])
+    assert not torch.equal(random_tensors(specs, 12, torch.float32, std=0.5)["a.weight"], t["a.weight"])
+    x = unit_normal(7, 400000, torch.device("cpu"))
+    assert abs(float(x.mean())) < 0.01 and abs(float(x.std()) - 1.0) < 0.01 and float(x.abs().max()) < 3.5

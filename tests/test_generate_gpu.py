@@ -409,3 +409,13 @@ def test_the_logits_behind_the_tokens_can_be_tapped_and_dumped(tmp_path, graphs)
     st = eng.stats
     assert st["prefill_portions"] == 3 and st["batched_rows"] == st["prefill_tokens"] + st["decode_tokens"]
     assert st["pages_in_use"] == 0 and st["pages_in_use_peak"] >= 2 and (st["graph_replays"] > 0) == graphs
+
+
+def test_a_seed_gives_the_same_weights_on_the_gpu_as_on_the_cpu():
+    from allpaca_amd.parts import ParamSpec
+    from allpaca_amd.weights import random_tensors
+    specs = {"w": ParamSpec((1000, 333)), "n": ParamSpec((77,), store="float32")}
+    for dtype in (torch.float32, torch.bfloat16):
+        cpu = random_tensors(specs, 5, dtype, norm_std=0.1)
+        gpu = random_tensors(specs, 5, dtype, norm_std=0.1, device="cuda:0")
+        assert all(torch.equal(cpu[k], gpu[k].cpu()) for k in specs)

@@ -486,21 +486,24 @@ def test_product_for_q_k_v_that_rotates_declines_what_it_does_not_take():
                                   torch.zeros(17, dtype=torch.int32, device=DEV), bt, cache2, P_)
 
 
-def run_attention(H, Hk, d, P_, lens, rows_per_seg, window=0, seed=0, stale=0.0, loud=None, ranges=None):
+def run_attention(H, Hk, d, P_, lens, rows_per_seg, window=0, seed=0, stale=0.0, loud=None, ranges=None, relocate=None):
     """Sequences of `lens` keys in the cache; the last `rows_per_seg[s]` positions of sequence s are the step's rows.
     `ranges`: into how many ranges the kernel for tiles of 128 rows is expected to cut the keys of this step.
     `stale`: what lies in the slots beyond a sequence's last key and in the spare page; with a window, the pages that
     every row of the step has passed are marked as given back in the block table (the spare page stands in).
-    `loud`: (sequence, position, factor) of a key whose scores dwarf all others."""
+    `loud`: (sequence, position, factor) of a key whose scores dwarf all others.
+    `relocate`: (cache, block tables) -> the same pages at other places of another cache tensor."""
     from allpaca_amd.engine.batch import Entry, pack_step
     from allpaca_amd.kernels import ops as kernel_ops
     t = tuned()
     cache, bt, ks, vs = make_cache(lens, Hk, d, P_, BF, seed=seed, stale=stale, loud=loud)
+    if relocate is not None:
+        cache, bt = relocate(cache, bt)
     pos0 = [n - r for n, r in zip(lens, rows_per_seg)]
     entries = [Entry(i, [0] * r, []) for i, r in enumerate(rows_per_seg)]
     tables = [[list(bt[i, : -(-n // P_)].cpu().numpy()) for i, n in enumerate(lens)]]
     used = {int(p) for tb in tables[0] for p in tb}
-    spare = min(set(range(cache.shape[0])) - used)
+    spare = next(p for p in range(cache.shape[0]) if p not in used)
     if window:
         for tb, p0 in zip(tables[0], pos0):
             for b in range(max(0, p0 - window + 1) // P_):
