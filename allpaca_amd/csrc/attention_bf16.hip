@@ -555,7 +555,16 @@ struct KVRegs {
 //             faster at one block a compute unit and 8-15 % slower at two).
 // The order of additions for a row depends on its position, KW and the number of parts only.
 constexpr int NW = 4;  // waves of a block of the decode kernel
+constexpr int LAST_DIRECT = 8;  // up to so many blocks a pair the last one reads the others' results in one go
 enum { DEC_PARTS = 0, DEC_WHOLE = 1, DEC_LAST = 2 };
+// Keys a part of a row takes when the launch gives the number of parts and not their length (KW == 0): the row's
+// `span` keys in n_parts equal ranges, in whole steps of 32 keys and no fewer than 64.  Rows of different lengths in
+// one launch then all use every block of their pair, and a launch's shape (blocks a pair) does not change with the
+// rows' lengths, which is what a recorded graph needs.
+__device__ __forceinline__ int row_keys_per_part(int KW, int span, int n_parts) {
+  if (KW > 0) return KW;
+  return max(64, ((span + n_parts - 1) / n_parts + 31) / 32 * 32);
+}
 // Why the hand-over of DEC_LAST holds without a release/acquire pair.  Every access to a partial result, on either
 // side, is a relaxed atomic of agent scope: on this chip such a store goes through to memory past the block's own L2
 // (sc1) and such a load is served from memory, so neither a write-back of the writer's L2 nor an invalidation of the
@@ -591,9 +600,15 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(
   const int part = blockIdx.z * NW + wave;
   const int pos = positions[row];
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int seen0 = (first / 32) * 32;  // the first position that is loaded
+  // KW == 0: the row's own keys, from the first one it sees, in n_parts equal ranges (see row_keys_per_part); else
+  // ranges of KW keys counted from position 0
+  const int base = KW > 0 ? 0 : seen0;
+  KW = row_keys_per_part(KW, pos + 1 - seen0, n_parts);
   // nothing to see for this part: the wave leaves (DEC_PARTS), or stays with an empty result (DEC_LAST: the block's
   // waves meet)
-  const bool empty = !WHOLE && (part >= n_parts || max(part * KW, (first / 32) * 32) >= min((part + 1) * KW, pos + 1));
+  const bool empty =
+      !WHOLE && (part >= n_parts || max(base + part * KW, seen0) >= min(base + (part + 1) * KW, pos + 1));
   if (MODE == DEC_PARTS && empty) return;
   const int* bt = block_table + (size_t)row_seg[row] * max_blocks;
   const size_t page_stride = (size_t)2 * Hk * P * d;
@@ -725,11 +740,15 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(
   };
   if constexpr (WHOLE) {
     for (int r = wave; r * KW <= pos; r += NW) {
-      const int k_lo = max(r * KW, (first / 32) * 32), k_hi = min((r + 1) * KW, pos + 1);
+      const int k_lo = max(r * KW, seen0), k_hi = min((r + 1) * KW, pos + 1);
       if (k_lo < k_hi) run_range(k_lo, k_hi);
     }
   } else if (!empty) {
-    run_range(max(part * KW, (first / 32) * 32), min((part + 1) * KW, pos + 1));
+    // a part in pieces of no more keys than a wave keeps page ids for (one piece, but for rows far longer than the
+    // launch's parts were counted for)
+    const int k_lo = max(base + part * KW, seen0), k_hi = min(base + (part + 1) * KW, pos + 1);
+    const int piece = max(32, (62 * P) / 32 * 32);
+    for (int k = k_lo; k < k_hi; k += piece) run_range(k, min(k + piece, k_hi));
   }
 
   // this wave's result for the heads of the group (maxima are in base-2 units, as the merge expects)
@@ -809,8 +828,38 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(
     __syncthreads();
     if (!is_last) return;
     // the last block of the pair: the blocks' results of every head, in block order (only blocks with a visible key)
-    const int p_lo = ((first / 32) * 32) / KW, p_hi = min(pos / KW, n_parts - 1);
+    const int p_lo = (seen0 - base) / KW, p_hi = min((pos - base) / KW, n_parts - 1);
     const int z_lo = p_lo / NW, nzv = p_hi / NW - z_lo + 1;
+    if (nzv <= LAST_DIRECT) {
+      // few blocks: a thread asks for the maxima, sums and its element of all of them at once (one trip to memory
+      // where the general way below makes two with a barrier between); the same additions in the same order
+      for (int idx = threadIdx.x; idx < tile_heads * d; idx += NW * 64) {
+        const int hg = idx / d, e = idx % d;
+        const float* src = parts + (((size_t)ri * H + (kvh * G + gt * 16 + hg)) * nz + z_lo) * stride;
+        float pm[LAST_DIRECT], pl[LAST_DIRECT], po[LAST_DIRECT];
+#pragma unroll
+        for (int zz = 0; zz < LAST_DIRECT; ++zz) {
+          const float* sz = src + (size_t)min(zz, nzv - 1) * stride;
+          pm[zz] = ld_coh(sz + d);
+          pl[zz] = ld_coh(sz + d + 1);
+          po[zz] = ld_coh(sz + e);
+        }
+        float m = -INFINITY;
+#pragma unroll
+        for (int zz = 0; zz < LAST_DIRECT; ++zz)
+          if (zz < nzv) m = fmaxf(m, pm[zz]);
+        float l = 0.f, acc = 0.f;
+#pragma unroll
+        for (int zz = 0; zz < LAST_DIRECT; ++zz)
+          if (zz < nzv) {
+            const float wgt = pm[zz] == -INFINITY ? 0.f : exp2_neg(pm[zz] - m);
+            l += pl[zz] * wgt;
+            acc = fmaf(po[zz], wgt, acc);
+          }
+        out[(size_t)row * ldo + (size_t)(kvh * G + gt * 16 + hg) * d + e] = float_to_bf16(acc / l);
+      }
+      return;
+    }
     float* ml = meet;  // [heads of the tile][nzv][2]: maximum, sum (the waves' results are not needed any more)
     for (int idx = threadIdx.x; idx < tile_heads * nzv; idx += NW * 64) {
       const int hg = idx / nzv, zz = idx % nzv;
@@ -852,7 +901,9 @@ __global__ __launch_bounds__(MERGE_NT) void attn_merge_kernel(const float* __res
   const int row = rows ? rows[ri] : ri;
   const int pos = positions[row];
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int p_lo = ((first / 32) * 32) / KW, p_hi = min(pos / KW, n_parts - 1);  // parts with a visible key
+  const int seen0 = (first / 32) * 32, part_base = KW > 0 ? 0 : seen0;  // as attn_decode_kernel counts the parts
+  KW = row_keys_per_part(KW, pos + 1 - seen0, n_parts);
+  const int p_lo = (seen0 - part_base) / KW, p_hi = min((pos - part_base) / KW, n_parts - 1);  // parts with a visible key
   const int np = p_hi - p_lo + 1;
   const size_t stride = (size_t)d + 2;
   const float* base = parts + (((size_t)ri * H + h) * n_parts + p_lo) * stride;
@@ -965,6 +1016,9 @@ static bool last_fits(int G, int d, int n_parts) {
 //                                 (row, kv head tile) = n_rows * Hk * ceil(H / Hk / 16), zero before the first call
 //                                 (every call leaves them zero); `apc_attention_decode_last_fits` says whether it can;
 //   workspace, counters null      workspace: n_rows * H * n_parts * (d + 2) floats; a second kernel merges.
+// keys_per_part: the keys of a part (a multiple of 32; the parts are counted from position 0, and n_parts of them
+// must reach the longest row's position), or, with a workspace, 0: every row's own keys in n_parts equal ranges
+// (rows of any length).
 // Calls that share counters or a workspace must not overlap (one stream).
 APC_EXPORT int apc_attention_decode_bf16(const void* q, int ldq, int q_off, void* out, int ldo, int n_rows, int H,
                                          int Hk, int d, const void* cache, int page_tokens, const int* block_table,
@@ -974,7 +1028,8 @@ APC_EXPORT int apc_attention_decode_bf16(const void* q, int ldq, int q_off, void
   if (n_rows <= 0) return 0;
   int e = check_common(q, ldq, q_off, cache, H, Hk, d, page_tokens);
   if (e) return e;
-  if (keys_per_part <= 0 || keys_per_part % 32 || max_blocks <= 0 || window < 0 || !out) return APC_ERR_BAD_ARG;
+  if (keys_per_part < 0 || keys_per_part % 32 || max_blocks <= 0 || window < 0 || !out) return APC_ERR_BAD_ARG;
+  if (keys_per_part == 0 && !workspace) return APC_ERR_BAD_ARG;      // a block that takes a pair whole is told its ranges
   if (keys_per_part / page_tokens + 2 > 64) return APC_ERR_BAD_ARG;  // a wave keeps one page id per lane
   const int G = H / Hk, gtiles = (G + 15) / 16;
   if (Hk * gtiles > 65535 || H > 65535) return APC_ERR_BAD_ARG;

@@ -414,7 +414,9 @@ int attention_bf16(Program& P, const Buf& q, const Buf& out, const ApcLayer& L, 
     const int span = window ? std::min(s.max_decode_context, window) : s.max_decode_context;
     const int* rows = s.all_rows_decode ? nullptr : s.decode_rows;
     const long pairs = (long)n * Hk * cdiv(H / Hk, 16);
-    if (pairs >= P.tun.whole_min_pairs && apc_attention_decode_whole_fits(H, Hk, d)) {
+    const int n_parts = decode_parts(pairs, span);
+    // (rows so short that one block's waves take a pair's ranges need no partial results either)
+    if ((pairs >= P.tun.whole_min_pairs || n_parts <= WHOLE_WAVES) && apc_attention_decode_whole_fits(H, Hk, d)) {
       const int kw = keys_per_wave_whole(span, page);
       LAUNCH(P, "attention_decode_bf16 (whole)",
              apc_attention_decode_bf16(q.p, q.ld, 0, out.p, out.ld, n, H, Hk, d, E.kv, page, table, width,
@@ -422,8 +424,7 @@ int attention_bf16(Program& P, const Buf& q, const Buf& out, const ApcLayer& L, 
                                        P.stream));
       return 1;
     }
-    const int kw = keys_per_part(n, Hk, span, page);
-    const int n_parts = (int)cdiv(s.max_decode_context, kw);
+    const int kw = 0;  // every row's own keys in n_parts ranges
     if (P.tun.last_block_merges && pairs <= P.pair_capacity && apc_attention_decode_last_fits(H, Hk, d, n_parts)) {
       const int nz = (int)cdiv(n_parts, WHOLE_WAVES);
       float* ws = P.floats((size_t)n * H * nz * (d + 2));
@@ -701,8 +702,8 @@ APC_HOST_EXPORT const char* apc_host_timing_report(void* prog) {
 
 // ---- the rules, for tests that hold them against the Python wrappers' own
 APC_HOST_EXPORT int apc_host_rule_tiled_k_split(int M, int N, int K) { return apc_rules::tiled_k_split(M, N, K); }
-APC_HOST_EXPORT int apc_host_rule_keys_per_part(int n_rows, int n_kv_heads, int max_context, int page_tokens) {
-  return apc_rules::keys_per_part(n_rows, n_kv_heads, max_context, page_tokens);
+APC_HOST_EXPORT int apc_host_rule_decode_parts(long long pairs, int span) {
+  return apc_rules::decode_parts((long)pairs, span);
 }
 APC_HOST_EXPORT int apc_host_rule_keys_per_wave_whole(int max_context, int page_tokens) {
   return apc_rules::keys_per_wave_whole(max_context, page_tokens);

@@ -37,12 +37,10 @@ inline int tiled_k_split(int M, int N, int K) {
   return M <= MANY_ROWS_SPLIT_MAX ? k_split_many_rows(M, N, K) : 1;
 }
 
-inline int keys_per_part(int n_rows, int n_kv_heads, int max_context, int page_tokens) {
-  int kw = 64;
-  while (kw < 1024 && (long)n_rows * n_kv_heads * cdiv(max_context, kw * 2) >= 768 && (kw * 2) / page_tokens + 2 <= 64)
-    kw *= 2;
-  while (kw > 32 && kw / page_tokens + 2 > 64) kw /= 2;
-  return kw;
+// ranges that the decode kernel cuts every row's keys into (the kernel sizes them from the row's own length)
+inline int decode_parts(long pairs, int span) {
+  const long per_pair = std::max(1L, (long)CHIP_UNITS / std::max(1L, pairs));
+  return (int)std::max(1L, std::min((long)WHOLE_WAVES * per_pair, cdiv(span, 64)));
 }
 
 inline int keys_per_wave_whole(int max_context, int page_tokens) {

@@ -318,19 +318,21 @@ def swiglu_pre_bf16(raw: torch.Tensor, ss: torch.Tensor, eps: float, wg: PackedW
     return True
 
 
-def _keys_per_part(n_rows: int, n_kv_heads: int, max_context: int, page_tokens: int = 16) -> int:
-    """Keys one wave covers in the decode kernel.  A wave that walks through many keys overlaps its loads
-    with its work, so: the longest range that still leaves 768 waves on the chip (three per compute unit; measured
-    at 8B shapes with 1 to 24 rows over 2,048 to 32,768 keys: the best choice of 64 .. 512 keys in every case, where
-    a thousand waves chose half the range at 12 and 24 rows and lost 9 and 12 %), at least 64 keys, and no more pages
-    than a wave keeps ids for (one per lane)."""
-    kw = 64
-    while (kw < 1024 and n_rows * n_kv_heads * (-(-max_context // (kw * 2))) >= 768
-           and (kw * 2) // page_tokens + 2 <= 64):
-        kw *= 2
-    while kw > 32 and kw // page_tokens + 2 > 64:
-        kw //= 2
-    return kw
+def _decode_parts(pairs: int, span: int) -> int:
+    """Ranges that the decode kernel cuts the keys of every row into (four to a block, one per wave): as many blocks
+    a (row, kv head) pair as keep the launch at one block a compute unit or under, and no range under 64 keys.  The
+    kernel sizes a row's ranges from the row's own length, so the count depends on the step's shape alone.  Measured at
+    8B shapes (32 heads over 8, heads of 128), 1 to 16 rows over 512 to 8,192 keys, ranges of 64 to 512 keys: the
+    fastest choice was in every case the shortest range whose launch fits the chip once (8 rows over 2,063 keys: 256
+    blocks 18.9 us, 320 blocks 21.4 us, 192 blocks 20.6 us; over 8,192 keys: 256 blocks 53.3 us, 512 blocks 54.6 us,
+    1,024 blocks 56.5 us)."""
+    per_pair = max(1, CHIP_UNITS // max(1, pairs))
+    return max(1, min(WHOLE_WAVES * per_pair, -(-span // 64)))
+
+
+# Keys of a range of the decode kernel, the same for every row and counted from position 0, instead of the rule above
+# (0: the rule): for measurements and tests.
+KEYS_PER_PART = 0
 
 
 # From how many (row, kv head) pairs on a decode step's attention runs as one block per pair that finishes its heads
@@ -435,15 +437,17 @@ def attention_bf16(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int,
         span = min(step.max_decode_context, window) if window else step.max_decode_context
         rows = step.decode_rows.data_ptr() if step.decode_rows is not None else 0
         pairs = n * n_kv_heads * -(-(n_heads // n_kv_heads) // 16)
-        if pairs >= WHOLE_MIN_PAIRS and L.apc_attention_decode_whole_fits(n_heads, n_kv_heads, head_dim):
+        n_parts = -(-step.max_decode_context // KEYS_PER_PART) if KEYS_PER_PART else _decode_parts(pairs, span)
+        # (rows so short that one block's waves take a pair's ranges need no partial results either)
+        if ((pairs >= WHOLE_MIN_PAIRS or n_parts <= WHOLE_WAVES)
+                and L.apc_attention_decode_whole_fits(n_heads, n_kv_heads, head_dim)):
             kw = _keys_per_wave_whole(span, page_tokens)
             _lib.check(L.apc_attention_decode_bf16(
                 q.data_ptr(), ldq, q_off, out.data_ptr(), ldo, n, n_heads, n_kv_heads, head_dim, cache.data_ptr(),
                 page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
                 step.row_seg.data_ptr(), rows, int(window), sc, kw, 0, 0, 0, stream), "attention_decode_bf16 (whole)")
             return True
-        kw = _keys_per_part(n, n_kv_heads, span, page_tokens)
-        n_parts = -(-step.max_decode_context // kw)
+        kw = KEYS_PER_PART
         if LAST_BLOCK_MERGES and L.apc_attention_decode_last_fits(n_heads, n_kv_heads, head_dim, n_parts):
             # one partial result a block; the block of a (row, kv head) that finishes last adds them: one launch
             nz = -(-n_parts // WHOLE_WAVES)

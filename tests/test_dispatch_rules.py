@@ -71,16 +71,20 @@ def test_what_the_sampler_tells_the_kernels(monkeypatch, rules, want):
     assert (seen["any_top_k"], seen["any_top_p"], seen["few_after_top_k"]) == want
 
 
-def test_keys_a_wave_of_the_decode_attention_takes():
-    """The longest range of keys that leaves 768 waves on the chip, from 64 keys on; never more pages than a wave
-    keeps ids for."""
+def test_ranges_the_decode_attention_cuts_a_rows_keys_into():
+    """Four ranges a block, as many blocks a (row, kv head) pair as keep the launch within the chip's compute units,
+    and no range under 64 keys."""
     from allpaca_amd.kernels import tuned as t
-    got = {(n, ctx): t._keys_per_part(n, 8, ctx, 16) for n, ctx in
-           [(1, 2048), (4, 2048), (8, 2048), (12, 2048), (16, 2048), (24, 2048), (8, 8192), (16, 8192), (1, 32768)]}
-    assert got == {(1, 2048): 64, (4, 2048): 64, (8, 2048): 128, (12, 2048): 256, (16, 2048): 256, (24, 2048): 512,
-                   (8, 8192): 512, (16, 8192): 512, (1, 32768): 256}
-    assert t._keys_per_part(16, 8, 1 << 20, 16) // 16 + 2 <= 64 and t._keys_per_part(16, 8, 1 << 20, 128) == 1024
-    assert t._keys_per_part(1, 1, 10, 16) == 64
+    got = {(n, ctx): t._decode_parts(n * 8, ctx) for n, ctx in
+           [(1, 2048), (4, 2048), (8, 2048), (8, 2063), (12, 2048), (16, 2048), (24, 2048), (8, 8192), (16, 8192),
+            (1, 32768), (8, 512), (1, 10), (40, 2048)]}
+    assert got == {(1, 2048): 32, (4, 2048): 32, (8, 2048): 16, (8, 2063): 16, (12, 2048): 8, (16, 2048): 8,
+                   (24, 2048): 4, (8, 8192): 16, (16, 8192): 8, (1, 32768): 128, (8, 512): 8, (1, 10): 1, (40, 2048): 4}
+    for pairs in (1, 8, 64, 100, 255, 256, 1000):
+        for span in (1, 64, 65, 2048, 1 << 20):
+            parts = t._decode_parts(pairs, span)
+            blocks = pairs * -(-parts // t.WHOLE_WAVES)
+            assert parts >= 1 and (blocks <= max(pairs, t.CHIP_UNITS)) and (parts == 1 or span / parts >= 32)
 
 
 def test_the_executors_rules_are_the_wrappers_rules():
@@ -92,12 +96,9 @@ def test_the_executors_rules_are_the_wrappers_rules():
         for N in (192, 1000, 2048, 3072, 4096, 5120, 6144, 8192, 14336, 16384, 28672, 57344, 128256):
             for K in (120, 192, 512, 2048, 3072, 4096, 8192, 14336, 28672):
                 assert L.apc_host_rule_tiled_k_split(M, N, K) == tuned._tiled_k_split(M, N, K), (M, N, K)
-    for n in (1, 2, 3, 8, 12, 16, 24, 31, 64, 255):
-        for hk in (1, 2, 8):
-            for ctx in (1, 63, 64, 65, 2048, 2049, 8192, 32768, 131072):
-                for page in (8, 16, 24, 64, 128, 256):
-                    assert (L.apc_host_rule_keys_per_part(n, hk, ctx, page)
-                            == tuned._keys_per_part(n, hk, ctx, page)), (n, hk, ctx, page)
+    for pairs in (1, 2, 3, 8, 12, 16, 24, 31, 64, 100, 255, 256, 257, 2040):
+        for span in (1, 63, 64, 65, 2048, 2049, 8192, 32768, 131072):
+            assert L.apc_host_rule_decode_parts(pairs, span) == tuned._decode_parts(pairs, span), (pairs, span)
     for ctx in (1, 100, 256, 257, 2048, 2049, 5000, 131072):
         for page in (8, 16, 24, 64, 128, 256):
             assert L.apc_host_rule_keys_per_wave_whole(ctx, page) == tuned._keys_per_wave_whole(ctx, page), (ctx, page)

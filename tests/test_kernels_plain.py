@@ -379,6 +379,46 @@ def test_sample_rows_among_equal_values(values):
         assert alone.cpu().tolist() == outs["many blocks"], V
 
 
+@pytest.mark.parametrize("one_block", [False, True], ids=["many blocks a row", "one block a row"])
+def test_sample_rows_on_the_boundaries_between_candidates(one_block):
+    """Rows with more than 1,024 survivors (no cut, a wide top-k, top-p alone): the many-block kernels add integer
+    weights (exp in units of 2^-40), the one-block kernel walks in float32 as the reference does
+    (crates/allpaca-core/src/sampling.rs:55-67) and the plain sampler in float64, so a uniform number on the boundary
+    between two candidates may fall on either side.  The number is put on boundaries of the plain sampler's walk and
+    one float32 step to either side: the token is the plain sampler's or its neighbour in the walk, never a
+    candidate further away, on either way through the kernels; and away from the boundaries (the other sampler
+    tests) it is the plain sampler's."""
+    o = ops()
+    V = 5000
+    base = (gen(1, V, seed=77) * 2.5)[0]
+    cases, rows, temps, ks, ps, us = [], [], [], [], [], []
+    for temperature, top_k, top_p in ((1.0, 0, 1.0), (0.7, 2000, 1.0), (1.0, 0, 0.95), (1.3, 3000, 0.9)):
+        cand, draws = P.sample_candidates(base.numpy(), temperature, top_k, top_p)
+        assert draws and len(cand) > 1024
+        place = {i: n for n, (i, _) in enumerate(cand)}
+        edges = np.cumsum([p for _, p in cand])
+        for j in np.linspace(0, len(cand) - 2, 25).astype(int):
+            on = np.float32(edges[j])
+            for u in (np.nextafter(on, np.float32(0)), on, np.nextafter(on, np.float32(1))):
+                if 0.0 <= u < 1.0:
+                    cases.append((place, P.sample(base.numpy(), temperature, top_k, top_p, float(u))))
+                    rows.append(base)
+                    temps.append(temperature)
+                    ks.append(top_k)
+                    ps.append(top_p)
+                    us.append(u)
+    R = len(rows)
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    o.sample_rows(torch.stack(rows).to(DEV), torch.tensor(temps, device=DEV), torch.tensor(ks, dtype=torch.int32, device=DEV),
+                  torch.tensor(ps, device=DEV), torch.tensor(np.asarray(us, np.float32), device=DEV), out,
+                  one_block=one_block)
+    got = out.cpu().tolist()
+    far = [(r, got[r], want) for r, (place, want) in enumerate(cases)
+           if got[r] not in place or abs(place[got[r]] - place[want]) > 1]
+    assert not far, far[:5]
+    assert sum(got[r] == want for r, (_, want) in enumerate(cases)) > R // 2
+
+
 def test_sample_rows_frequencies():
     o = ops()
     V, n = 12, 4000

@@ -530,11 +530,16 @@ def run_attention(H, Hk, d, P_, lens, rows_per_seg, window=0, seed=0, stale=0.0,
         at += r
 
 
-@pytest.fixture(params=["last block merges", "merge kernel"])
+@pytest.fixture(params=["last block merges", "merge kernel", "ranges of 64 keys from position 0", "five ranges a row"])
 def decode_path(request, monkeypatch):
     """Single rows whose keys are split over blocks: the block that finishes last adds the blocks' results (the
-    default), or a second kernel does."""
-    monkeypatch.setattr(tuned(), "LAST_BLOCK_MERGES", request.param == "last block merges")
+    default), or a second kernel does; ranges of a given length for all rows instead of each row's own keys in equal
+    ranges; ranges so long that a wave takes them in pieces."""
+    monkeypatch.setattr(tuned(), "LAST_BLOCK_MERGES", request.param != "merge kernel")
+    if request.param == "ranges of 64 keys from position 0":
+        monkeypatch.setattr(tuned(), "KEYS_PER_PART", 64)
+    if request.param == "five ranges a row":
+        monkeypatch.setattr(tuned(), "_decode_parts", lambda pairs, span: 5)
     return request.param
 
 
@@ -732,6 +737,18 @@ def test_attention_finds_a_far_key_in_every_path(monkeypatch):
         for h in range(H):
             want = vs[0][key, h // 2].float()
             assert torch.allclose(out[-1, h * d:(h + 1) * d].float().cpu(), want, atol=2.0 ** -7 * 4)
+
+
+@pytest.mark.parametrize("parts", [4, 5, 6, 13, 32])
+@pytest.mark.parametrize("window", [0, 700])
+def test_attention_decode_with_rows_of_very_different_lengths(monkeypatch, parts, window, decode_path):
+    """Every row's own keys go into the launch's number of ranges: rows of 1 to 6,000 keys in one launch, with counts
+    of ranges that do not fill the last block, ranges far longer than a wave keeps page ids for (pages of 8), and a
+    window whose first key lies inside a range."""
+    if decode_path == "last block merges" or decode_path == "merge kernel":
+        monkeypatch.setattr(tuned(), "_decode_parts", lambda pairs, span: parts)
+    run_attention(H=8, Hk=2, d=64, P_=8, lens=[6000, 1, 63, 64, 65, 1500, 2063, 129], rows_per_seg=[1] * 8,
+                  window=window, seed=parts)
 
 
 def test_attention_decode_many_launches_leave_the_counters_at_zero():
