@@ -633,7 +633,8 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(
   float m_run = -INFINITY, l_run = 0.f;
   bf16_t* pw = Ps + wave * 16 * (32 + KPAD);
 
-  // Operands of 32 keys straight from the pages.  Nothing is loaded conditionally: a key beyond the row's own
+  // Operands of 32 keys straight from the pages, with loads that the caches do not keep (a decoded row reads its keys
+  // and values once).  Nothing is loaded conditionally: a key beyond the row's own
   // position is read from that position instead (its score is masked), an element beyond d from element 0 or
   // d - 1 (the query is zero there; such output columns are not stored), so the loads of the next 32 keys can be
   // in flight while these are used.
@@ -646,14 +647,14 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(
 #pragma unroll
       for (int ks = 0; ks < DP / 32; ++ks) {
         const int e = ks * 32 + lc * 8;
-        r.k[nt][ks] = load_frag(krow + (e < d ? e : 0));
+        r.k[nt][ks] = load_frag_once(krow + (e < d ? e : 0));
       }
     }
     const int tv = min(kb + lc * 8, (pos / 8) * 8);
     const int vpage = __shfl(my_page, tv / P - page0, WAVE);
     const bf16_t* vbase = cache + (size_t)vpage * page_stride + v_off + head_off + (tv % P);
 #pragma unroll
-    for (int dt = 0; dt < DP / 16; ++dt) r.v[dt] = load_frag(vbase + (size_t)min(dt * 16 + li, d - 1) * P);
+    for (int dt = 0; dt < DP / 16; ++dt) r.v[dt] = load_frag_once(vbase + (size_t)min(dt * 16 + li, d - 1) * P);
   };
 
   // lane holds keys kb + nt*16 + lc*4 + r (scores) and elements dt*16 + lc*4 + r (output) of head li of the group

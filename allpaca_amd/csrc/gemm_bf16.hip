@@ -45,7 +45,11 @@ struct TiledPre {
 };
 
 // EVEN_K: K is a multiple of 64, so no load needs a bound check.  BM: rows of the block tile, 64 or 128.
-template <int MODE, bool EVEN_K, int BM, bool PRE = false>
+// DEPTH (even): how many K steps the global loads run ahead of the MFMAs, one register set a step.  2 where two blocks
+// share a compute unit (many rows); 4 for the steps of up to 128 rows, whose blocks have a unit each and stream the
+// weights once: what they have in flight sets their pace (a block of 64 rows x 64 SwiGLU outputs with 2 steps in
+// flight took 0.8 us a step of 16 KiB of weights).
+template <int MODE, bool EVEN_K, int BM, bool PRE = false, int DEPTH = 2>
 __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda,
                                                         const bf16_t* __restrict__ W,
                                                         const bf16_t* __restrict__ W2, int chunks,
@@ -126,7 +130,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
     } else {
       const int p = j - AP;
       const bf16_t* src = (p < 2 ? wbase0 : wbase1) + (size_t)kt * 1024 + woff[p];
-      g.w[p] = (EVEN_K || kt * 2 + wkc < chunks) ? load_frag(src) : zero_frag();  // W is zero-padded to whole tiles
+      // W is zero-padded to whole tiles.  With up to 128 rows a weight is read once, by this block: a load that the
+      // caches do not keep, where the block walks all of K (SwiGLU of 64 rows at 8B shapes 45.2 -> 42.5 us; with K in
+      // slices the short runs of a slice were slower that way, o_proj of 64 rows 15.9 -> 17.9 us)
+      constexpr bool ONCE = DEPTH > 2 && MODE != G_PARTIAL;
+      g.w[p] = (EVEN_K || kt * 2 + wkc < chunks) ? (ONCE ? load_frag_once(src) : load_frag(src)) : zero_frag();
     }
   };
   auto store_piece = [&](const GemmRegs<BM>& g, int buf, int j) {
@@ -178,19 +186,22 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
   const int per_slice = MODE == G_PARTIAL ? ceil_div(all_tiles, k_split) : all_tiles;
   const int kt0 = slice * per_slice;
   const int ktiles = max(0, min(all_tiles, kt0 + per_slice) - kt0);
-  // K steps are loaded two ahead: while step t is multiplied out of one LDS buffer, step t+1 moves from registers
-  // into the other and the loads of step t+2 go out (register sets s0, s1 take turns).  The steady loop has no
-  // branch around a load, so the waits for one set never wait for the other.
+  // K steps are loaded DEPTH ahead: while step t is multiplied out of one LDS buffer, step t+1 moves from registers
+  // into the other and the loads of step t+DEPTH go out (register set t % DEPTH, whose step went into LDS a step
+  // ago).  The steady loop has no branch around a load, so the waits for one set never wait for another: near the end
+  // of K it loads the last step again instead.
+  static_assert(DEPTH >= 2 && DEPTH % 2 == 0, "the LDS buffer of a step is its register set's parity");
   if (ktiles > 0) {
-    GemmRegs<BM> s0, s1;
+    GemmRegs<BM> s[DEPTH];
+    const int last = kt0 + ktiles - 1;
 #pragma unroll
-    for (int j = 0; j < PIECES; ++j) load_piece(s0, kt0, j);
+    for (int j = 0; j < PIECES; ++j) load_piece(s[0], kt0, j);
 #pragma unroll
-    for (int j = 0; j < PIECES; ++j) store_piece(s0, 0, j);
-    if (ktiles > 1) {
+    for (int dd = 1; dd < DEPTH; ++dd)
 #pragma unroll
-      for (int j = 0; j < PIECES; ++j) load_piece(s1, kt0 + 1, j);
-    }
+      for (int j = 0; j < PIECES; ++j) load_piece(s[dd], min(kt0 + dd, last), j);
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) store_piece(s[0], 0, j);
     if constexpr (PRE) {  // behind the first loads of the tiles: one row a thread, its parts added in order, 8 loads
       if (tid < BM) {     // at a time; read after the barriers of the K loop
         const float* row = pre.ss + (size_t)min(m0 + tid, M - 1) * pre.parts;
@@ -207,26 +218,22 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
     }
     __syncthreads();
     int kt = 0;
-    while (kt + 3 < ktiles) {
-      step(yes, yes, 0, s0, kt0 + kt + 2, s1);
-      __syncthreads();
-      step(yes, yes, 1, s1, kt0 + kt + 3, s0);
-      __syncthreads();
-      kt += 2;
+    for (; kt + DEPTH < ktiles; kt += DEPTH) {  // whole rounds of the register sets with a step behind them
+#pragma unroll
+      for (int dd = 0; dd < DEPTH; ++dd) {
+        step(yes, yes, dd & 1, s[dd], min(kt0 + kt + dd + DEPTH, last), s[(dd + 1) % DEPTH]);
+        __syncthreads();
+      }
     }
-    const int rem = ktiles - kt;  // 1..3 steps left: step kt in LDS buffer 0, step kt+1 (if any) in s1
-    if (rem == 3) {
-      step(yes, yes, 0, s0, kt0 + kt + 2, s1);
-      __syncthreads();
-      step(no, yes, 1, s1, 0, s0);
-      __syncthreads();
-      step(no, no, 0, s0, 0, s1);
-    } else if (rem == 2) {
-      step(no, yes, 0, s0, 0, s1);
-      __syncthreads();
-      step(no, no, 1, s0, 0, s1);
-    } else {
-      step(no, no, 0, s0, 0, s1);
+    // 1..DEPTH steps left, all loaded: step kt in LDS buffer 0, the others in their sets
+#pragma unroll
+    for (int dd = 0; dd < DEPTH; ++dd) {
+      if (kt + dd + 1 < ktiles) {
+        step(no, yes, dd & 1, s[dd], 0, s[(dd + 1) % DEPTH]);
+        __syncthreads();
+      } else if (kt + dd < ktiles) {
+        step(no, no, dd & 1, s[dd], 0, s[dd]);
+      }
     }
   }
 
@@ -320,14 +327,23 @@ static int launch_gemm(const bf16_t* A, int lda, const bf16_t* W, const bf16_t* 
       N -= n_big;
     }
   }
-  const long blocks = 8L * ceil_div(ceil_div(N, NB), 8) * ceil_div(M, BM_ROWS);
+  // up to 128 rows (a decode step of many requests, a short portion): a block has a compute unit to itself and streams
+  // its weights once, so its loads run 4 steps ahead; up to 64 rows on tiles of 64 rows (half the loads of activations
+  // and half the MFMAs)
+  const int bm = M <= 64 ? 64 : BM_ROWS;
+  const long blocks = 8L * ceil_div(ceil_div(N, NB), 8) * ceil_div(M, bm);
   if (blocks > 0x7fffffffL) return APC_ERR_BAD_ARG;
-  if (K % BK == 0)
-    hipLaunchKernelGGL((gemm_bf16_kernel<MODE, true, BM_ROWS, PRE>), dim3((unsigned)blocks), dim3(256), 0, stream, A,
-                       lda, W, W2, ceil_div(K, 32), C, ldc, M, N, K, 1, pre);
-  else
-    hipLaunchKernelGGL((gemm_bf16_kernel<MODE, false, BM_ROWS, PRE>), dim3((unsigned)blocks), dim3(256), 0, stream, A,
-                       lda, W, W2, ceil_div(K, 32), C, ldc, M, N, K, 1, pre);
+#define TILED_LAUNCH(EVEN_, BM_, DEPTH_)                                                                              \
+  hipLaunchKernelGGL((gemm_bf16_kernel<MODE, EVEN_, BM_, PRE, DEPTH_>), dim3((unsigned)blocks), dim3(256), 0, stream, A, \
+                     lda, W, W2, ceil_div(K, 32), C, ldc, M, N, K, 1, pre)
+#define TILED_BY_K(BM_, DEPTH_)                     \
+  if (K % BK == 0) TILED_LAUNCH(true, BM_, DEPTH_); \
+  else TILED_LAUNCH(false, BM_, DEPTH_)
+  if (M <= 64) { TILED_BY_K(64, 4); }
+  else if (M <= 128) { TILED_BY_K(BM_ROWS, 4); }
+  else { TILED_BY_K(BM_ROWS, 2); }
+#undef TILED_BY_K
+#undef TILED_LAUNCH
   APC_LAUNCH_CHECK();
   return 0;
 }
@@ -402,16 +418,20 @@ static int launch_partials(const void* A, int lda, const void* W, const void* Wu
     if (e != APC_ERR_UNSUPPORTED) return e;
   }
   // up to 64 rows: tiles of 64 rows (half the loads of activations and half the MFMAs of a 128-row tile)
-#define PARTIAL_LAUNCH(EVEN_, BM_)                                                                                  \
-  hipLaunchKernelGGL((gemm_bf16_kernel<G_PARTIAL, EVEN_, BM_>), dim3(ceil_div(N, BN), ceil_div(M, BM_), k_split * n_mats), \
-                     dim3(256), 0, stream, (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)Wu, ceil_div(K, 32), \
-                     workspace, N, M, N, K, k_split, TiledPre{})
+#define PARTIAL_LAUNCH(EVEN_, BM_, DEPTH_)                                                                          \
+  hipLaunchKernelGGL((gemm_bf16_kernel<G_PARTIAL, EVEN_, BM_, false, DEPTH_>),                                      \
+                     dim3(ceil_div(N, BN), ceil_div(M, BM_), k_split * n_mats), dim3(256), 0, stream, (const bf16_t*)A, \
+                     lda, (const bf16_t*)W, (const bf16_t*)Wu, ceil_div(K, 32), workspace, N, M, N, K, k_split,      \
+                     TiledPre{})
   if (M <= 64) {
-    if (K % BK == 0) PARTIAL_LAUNCH(true, 64);
-    else PARTIAL_LAUNCH(false, 64);
+    if (K % BK == 0) PARTIAL_LAUNCH(true, 64, 4);
+    else PARTIAL_LAUNCH(false, 64, 4);
+  } else if (M <= 128) {
+    if (K % BK == 0) PARTIAL_LAUNCH(true, BM_ROWS, 4);
+    else PARTIAL_LAUNCH(false, BM_ROWS, 4);
   } else {
-    if (K % BK == 0) PARTIAL_LAUNCH(true, BM_ROWS);
-    else PARTIAL_LAUNCH(false, BM_ROWS);
+    if (K % BK == 0) PARTIAL_LAUNCH(true, BM_ROWS, 2);
+    else PARTIAL_LAUNCH(false, BM_ROWS, 2);
   }
 #undef PARTIAL_LAUNCH
   APC_LAUNCH_CHECK();

@@ -22,6 +22,13 @@ struct alignas(16) Frag {  // 8 bfloat16 as raw bits
 __device__ __forceinline__ bf16x8_t as_bf16x8(const Frag& f) { return __builtin_bit_cast(bf16x8_t, f); }
 
 __device__ __forceinline__ Frag load_frag(const bf16_t* p) { return *reinterpret_cast<const Frag*>(p); }
+// The same for bytes that are read once (weights of a step with few rows, keys and values of a decoded row): a
+// non-temporal load, which the caches do not keep.  A read of 8 GiB streams at 7.3 TB/s this way and at 6.2 TB/s with
+// ordinary loads (measured with blocks that walk their own share, 16 bytes a lane, 8 loads in flight a lane).
+__device__ __forceinline__ Frag load_frag_once(const bf16_t* p) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  return __builtin_bit_cast(Frag, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)));
+}
 __device__ __forceinline__ Frag zero_frag() { Frag f; f.w[0] = f.w[1] = f.w[2] = f.w[3] = 0u; return f; }
 
 // A buffer descriptor over global memory from `base` on (raw, no stride, no bound that matters): a load then takes the

@@ -6,8 +6,19 @@
 #include "mfma.h"
 
 // Every thread reads 16 bytes at a time, UNROLL loads in flight, the block walks through its own contiguous share of
-// the buffer; the sums keep the loads alive and go to out[block].
-template <int UNROLL>
+// the buffer; the sums keep the loads alive and go to out[block].  ONCE: with loads that the caches do not keep, which is
+// how the decode kernels read weights, keys and values (8 GiB: 7.3 TB/s against 6.2 TB/s with ordinary loads).
+typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
+template <bool ONCE>
+__device__ __forceinline__ uint4 probe_load(const uint4* p) {
+  if constexpr (ONCE) {
+    const probe_u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const probe_u32x4*>(p));
+    return uint4{v[0], v[1], v[2], v[3]};
+  } else {
+    return *p;
+  }
+}
+template <int UNROLL, bool ONCE>
 __global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict__ p, size_t n16, float* __restrict__ out) {
   const size_t per_block = (n16 + gridDim.x - 1) / gridDim.x;
   const size_t lo = (size_t)blockIdx.x * per_block, hi = lo + per_block < n16 ? lo + per_block : n16;
@@ -16,12 +27,12 @@ __global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict
   for (; i + (size_t)(UNROLL - 1) * 256 < hi; i += (size_t)UNROLL * 256) {
     uint4 v[UNROLL];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) v[u] = p[i + (size_t)u * 256];
+    for (int u = 0; u < UNROLL; ++u) v[u] = probe_load<ONCE>(p + i + (size_t)u * 256);
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) acc += v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
   }
   for (; i < hi; i += 256) {
-    const uint4 v = p[i];
+    const uint4 v = probe_load<ONCE>(p + i);
     acc += v.x ^ v.y ^ v.z ^ v.w;
   }
   __shared__ float part[4];
@@ -31,14 +42,22 @@ __global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict
   if (threadIdx.x == 0) out[blockIdx.x] = part[0] + part[1] + part[2] + part[3];
 }
 
-// Reads `bytes` (a multiple of 16) from p with `blocks` blocks of 256 threads; out: float [blocks].
-APC_EXPORT int apc_probe_read(const void* p, size_t bytes, float* out, int blocks, int unroll, hipStream_t stream) {
+// Reads `bytes` (a multiple of 16) from p with `blocks` blocks of 256 threads; out: float [blocks].  once: 1 for loads
+// that the caches do not keep.
+APC_EXPORT int apc_probe_read(const void* p, size_t bytes, float* out, int blocks, int unroll, int once,
+                              hipStream_t stream) {
   if (!p || !out || blocks <= 0 || bytes % 16 || ((uintptr_t)p & 15u)) return APC_ERR_BAD_ARG;
   const size_t n16 = bytes / 16;
-  if (unroll == 8) hipLaunchKernelGGL(probe_read_kernel<8>, dim3(blocks), dim3(256), 0, stream, (const uint4*)p, n16, out);
-  else if (unroll == 4) hipLaunchKernelGGL(probe_read_kernel<4>, dim3(blocks), dim3(256), 0, stream, (const uint4*)p, n16, out);
-  else if (unroll == 2) hipLaunchKernelGGL(probe_read_kernel<2>, dim3(blocks), dim3(256), 0, stream, (const uint4*)p, n16, out);
+#define PROBE_READ(U_, O_) \
+  hipLaunchKernelGGL((probe_read_kernel<U_, O_>), dim3(blocks), dim3(256), 0, stream, (const uint4*)p, n16, out)
+  if (unroll == 8 && once) PROBE_READ(8, true);
+  else if (unroll == 8) PROBE_READ(8, false);
+  else if (unroll == 4 && once) PROBE_READ(4, true);
+  else if (unroll == 4) PROBE_READ(4, false);
+  else if (unroll == 2 && once) PROBE_READ(2, true);
+  else if (unroll == 2) PROBE_READ(2, false);
   else return APC_ERR_BAD_ARG;
+#undef PROBE_READ
   APC_LAUNCH_CHECK();
   return 0;
 }

@@ -129,7 +129,7 @@ __global__ __launch_bounds__(WPB * 64, sk_blocks(MODE, WPB)) void skinny_gemm_ke
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
-      for (int b = 0; b < NB; ++b) r.w[b][u] = load_frag(wb[b] + (size_t)(ch + u) * TILE_ELEMS);
+      for (int b = 0; b < NB; ++b) r.w[b][u] = load_frag_once(wb[b] + (size_t)(ch + u) * TILE_ELEMS);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) r.a[mt][u] = load_frag(arow[mt] + (ch + u) * 32);
     }
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(WPB * 64, sk_blocks(MODE, WPB)) void skinny_gemm_ke
     for (int mt = 0; mt < MT; ++mt) {
       const Frag af = in ? load_frag(arow[mt] + ch * 32) : zero_frag();
 #pragma unroll
-      for (int b = 0; b < NB; ++b) acc[b][mt] = mfma16(load_frag(wb[b] + (size_t)ch * TILE_ELEMS), af, acc[b][mt]);
+      for (int b = 0; b < NB; ++b) acc[b][mt] = mfma16(load_frag_once(wb[b] + (size_t)ch * TILE_ELEMS), af, acc[b][mt]);
     }
   }
 

@@ -65,7 +65,7 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_attention_prefill_wide_takes": [I, I, I, I],
     },
     "bench": {
-        "apc_probe_read": [P, Z, P, I, I, P],
+        "apc_probe_read": [P, Z, P, I, I, I, P],
         "apc_probe_mfma": [I, P, I, P],
     },
 }

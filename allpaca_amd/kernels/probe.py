@@ -8,8 +8,9 @@ from . import lib as _lib
 from . import ops as _ops
 
 
-def read_bandwidth(gib: float = 8.0, blocks: int = 256 * 8, unroll: int = 8, repeats: int = 3) -> float:
-    """GB/s of reading `gib` GiB of device memory once with 16-byte loads (best of `repeats`)."""
+def read_bandwidth(gib: float = 8.0, blocks: int = 256 * 8, unroll: int = 8, repeats: int = 3, once: bool = True) -> float:
+    """GB/s of reading `gib` GiB of device memory once with 16-byte loads (best of `repeats`); `once`: with loads that
+    the caches do not keep, as the decode kernels read weights, keys and values."""
     L = _lib.load("bench")
     n = int(gib * 2 ** 30) // 16 * 16
     buf = torch.empty(n, dtype=torch.uint8, device="cuda")
@@ -19,7 +20,7 @@ def read_bandwidth(gib: float = 8.0, blocks: int = 256 * 8, unroll: int = 8, rep
     for _ in range(repeats + 1):
         t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0.record()
-        _lib.check(L.apc_probe_read(buf.data_ptr(), n, out.data_ptr(), blocks, unroll, _ops._stream()), "probe_read")
+        _lib.check(L.apc_probe_read(buf.data_ptr(), n, out.data_ptr(), blocks, unroll, int(once), _ops._stream()), "probe_read")
         t1.record()
         t1.synchronize()
         best = max(best, n / (t0.elapsed_time(t1) * 1e-3) / 1e9)
