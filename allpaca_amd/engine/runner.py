@@ -264,7 +264,7 @@ class ModelRunner:
     # ---- decode-only steps as HIP graphs -----------------------------------------------
     def graph_step(self, entries: Sequence[Entry]) -> torch.Tensor:
         """A step in which every request brings one token and wants its logits: the launches of the whole
-        model are replayed from a graph captured for (rows rounded up to a power of two, context rounded
+        model are replayed from a graph captured for (rows rounded up, see `_row_bucket`, context rounded
         up to a power of two); only the batch description is copied in."""
         seqs = [e.seq for e in entries]
         g = self._graph_for(seqs)
@@ -273,10 +273,20 @@ class ModelRunner:
 
     def _bucket(self, n: int, longest: int) -> tuple:
         """(rows, span) of the graph for n requests of which the longest will hold `longest` tokens."""
-        rows = 1 << max(0, (n - 1).bit_length())
+        rows = self._row_bucket(n)
         span = max(256, 1 << (longest - 1).bit_length())
         span = min(span, -(-self.rt.max_positions // self.cache.page_tokens) * self.cache.page_tokens)
         return rows, max(span, longest)
+
+    @staticmethod
+    def _row_bucket(n: int) -> int:
+        """Rows of the graph that takes n requests: the next power of two, but every even number from 8 to 16: there the
+        products stream the weights through one 16-row MFMA tile and read, beside every weight tile, the activations of
+        the rows that exist (padding rows are rows of their own), so a step of 9 rows in a graph of 16 took 4.36 ms at
+        8B shapes where 10 rows take about what 8 do (3.6 ms)."""
+        if 8 < n <= 16:
+            return (n + 1) // 2 * 2
+        return 1 << max(0, (n - 1).bit_length())
 
     def _graph_for(self, seqs: Sequence[Hashable]) -> "DecodeGraph":
         key = self._bucket(len(seqs), max(self.cache.length(s) for s in seqs) + 1)
@@ -293,17 +303,13 @@ class ModelRunner:
             return 0
         top = min(max_context or self.rt.max_positions, self.rt.max_positions)
         keys = set()
-        n = 1
-        while True:
+        for n in sorted({self._row_bucket(k) for k in range(1, max_rows + 1)}):
             longest = 1
             while True:
                 keys.add(self._bucket(min(n, max_rows), min(longest, top)))
                 if longest >= top:
                     break
                 longest *= 2
-            if n >= max_rows:
-                break
-            n *= 2
         made = 0
         for key in sorted(keys):
             if key not in self.graphs:
