@@ -301,6 +301,46 @@ def test_graph_replays_equal_eager_steps(dtype):
     H.assert_close(got, H.oracle_logits(folder, toks1[:upto])[want_rows], dtype, "graph decode", noise)
 
 
+def test_graphs_of_nine_to_sixteen_rows():
+    """Decode steps of 9 to 16 requests are replayed from a graph of the next even number of rows (a padding row costs
+    the streaming products what a live one does): 11 requests, then 9 when two have left, against eager steps and
+    against the plain implementation; and the buckets that `capture_decode_graphs` makes for up to 13 requests."""
+    from allpaca_amd.engine.batch import Entry
+    from allpaca_amd.engine.runner import ModelRunner
+    from allpaca_amd.models import load_model
+    assert [ModelRunner._row_bucket(n) for n in (1, 2, 3, 5, 8, 9, 10, 11, 15, 16, 17, 33)] == \
+        [1, 2, 4, 8, 8, 10, 10, 12, 16, 16, 32, 64]
+    folder = H.model_folder("B", "float32", True)
+    cfg, model = load_model(folder, torch.float32, "cuda:0")
+    runs = {}
+    for graphs in (False, True):
+        runner = ModelRunner(model, 16, 96, 16, use_graphs=graphs)
+        toks = {i: H.random_tokens(1000, 40, seed=500 + i) for i in range(11)}
+        at = {}
+        for i in range(11):
+            runner.admit(i)
+            runner.step([Entry(i, toks[i][:3 + i], [])])
+            at[i] = 3 + i
+        out = []
+        for s in range(12):
+            if s == 6:
+                for i in (2, 7):
+                    runner.release(i)
+                    del at[i]
+            out.append(runner.step([Entry(i, [toks[i][p]], [0]) for i, p in sorted(at.items())]).float().cpu().numpy())
+            for i in at:
+                at[i] += 1
+        runs[graphs] = out
+        if graphs:
+            assert runner.graph_replays == 12 and {k[0] for k in runner.graphs} == {12, 10}
+            assert runner.capture_decode_graphs(13, 64) > 0
+            assert {k[0] for k in runner.graphs} == {1, 2, 4, 8, 10, 12, 14}
+    for a, b in zip(runs[False], runs[True]):
+        assert np.array_equal(a, b)
+    got = np.concatenate([r[-1][None] for r in runs[True]])          # request 10: its tokens 13 .. 24
+    H.assert_close(got, H.oracle_logits(folder, H.random_tokens(1000, 40, seed=510)[:25])[13:25], "float32", "graphs of 12 and 10 rows")
+
+
 def test_generation_with_graphs_equals_the_plain_implementation():
     folder = H.model_folder("A", "float32", True)
     cfg, w = H.oracle(folder)
