@@ -185,7 +185,8 @@ def test_product_of_the_normalised_row_from_what_was_left(M, N, K):
     assert np.abs(f64(out) - exact).max() <= 2.0 ** -8 * np.abs(x * rstd * g).max() * np.abs(f64(w)).sum(axis=1).max()
 
 
-@pytest.mark.parametrize("M,F,K", [(1, 24, 64), (8, 176, 512), (16, 200, 112), (4, 14336 // 8, 1024)])
+@pytest.mark.parametrize("M,F,K", [(1, 24, 64), (8, 176, 512), (16, 200, 112), (4, 14336 // 8, 1024), (8, 14336, 512),
+                                   (11, 9000, 256)])
 def test_swiglu_of_the_normalised_row_from_what_was_left(M, F, K):
     t = tuned()
     x = f64(gen(M, K, seed=1, scale=2.0))
@@ -350,7 +351,10 @@ def test_embedding_from_the_tiled_table():
                                    # weights straight into registers (K a multiple of 128): 2, 3 and 4 gate bands a
                                    # wave, a last band of 8 columns, a last row tile of 76 rows
                                    (1024, 136, 128), (1100, 13208, 256), (2048, 3072, 384), (2048, 14336 // 2, 128),
-                                   (2048, 14336, 128)])
+                                   (2048, 14336, 128),
+                                   # few rows and more than 512 bands of outputs: two gate bands and their up bands a
+                                   # block of the streaming kernel (an odd number of bands; a last band of 8 columns)
+                                   (8, 14336, 256), (16, 9000, 64), (3, 8200, 520)])
 def test_swiglu_bf16(M, F, K):
     t = tuned()
     h = gen(M, K, seed=1, dtype=BF).to(DEV)
