@@ -8,9 +8,10 @@
 // loads (no registers in between), already in fragment order (a 16 x 32 fragment = one load instruction = 1 KiB
 // that a later ds_read_b128 returns lane by lane, free of bank conflicts), in four stages of 64 columns.
 // Per 64 columns a block moves 16 KiB of A and 8 NF KiB of W through the load path and reads 64 KiB from LDS, where
-// the 128 x 128 tile of gemm_bf16.hip moves 32 KiB and 96 KiB for half as many MFMAs (NF = 8).  What bounds it at
-// the shapes of a 2,048-row step is the L2: every block streams (128 + 64 NF) K 2 bytes through it, the counters
-// show the L2 busy three quarters of the time, and the vendor library's products sit at the same bound.
+// the 128 x 128 tile of gemm_bf16.hip moves 32 KiB and 96 KiB for half as many MFMAs (NF = 8).  At the shapes of a
+// 2,048-row step it waits for its loads: every block streams (128 + 64 NF) K 2 bytes through the L2, which the
+// counters show busy three quarters of the time or more; 60 % fewer requests to the L2 (four waves made to load
+// the same bands, timing only) bought 13 %, and the vendor library's products take about the same time.
 //
 // The accumulators (8 row groups x NF bands x 4 registers) live in the accumulation registers; the MFMA is written as
 // an instruction with that register class, because left to itself the compiler moved accumulators between the two
