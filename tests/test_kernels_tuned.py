@@ -368,7 +368,11 @@ def test_swiglu_bf16(M, F, K):
 
 @pytest.mark.parametrize("H,Hk,d,rot,P_,with_cache", [(32, 8, 128, 128, 16, True), (5, 1, 64, 32, 8, True),
                                                       (6, 2, 80, 0, 16, True), (4, 4, 256, 256, 32, False),
-                                                      (3, 3, 48, 48, 24, True)])
+                                                      (3, 3, 48, 48, 24, True),
+                                                      # pages whose columns do not start on 16 bytes: values slot by slot
+                                                      (4, 2, 64, 64, 12, True),
+                                                      # more columns of values than a block has in LDS at a time
+                                                      (8, 8, 128, 128, 16, True)])
 def test_rotation_and_cache_write_16_bytes_a_lane_equals_the_plain_kernel(H, Hk, d, rot, P_, with_cache):
     """`ops.rope_kv_write` on bfloat16 rows takes the kernel of the MFMA library; the plain kernel on the same input
     gives the same rows and the same cache (the same float32 formula; a rounding may fall the other way where the
