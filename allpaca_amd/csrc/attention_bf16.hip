@@ -548,7 +548,9 @@ struct KVRegs {
 //             partial results go through memory with stores and loads that are coherent across the chip's eight L2
 //             caches one by one (sc1), not with a fence: a device-wide fence writes back and invalidates a whole L2
 //             and cost ten times what the second launch did.
-//  DEC_WHOLE  the block's 4 waves take all ranges of KW keys of the pair in turn (wave w the ranges w, w + 4, ..),
+//  DEC_WHOLE  the block's 4 waves take all ranges of KW keys of the pair in turn (wave w the ranges w, w + 4, ..; with
+//             KW == 0 the row's own keys in 4 equal ranges, one a wave, so that a short row beside a long one still
+//             has work for every wave: 32 rows of 328 to 4,296 keys 69.1 -> 66.7 us, equal rows as before),
 //             meet in LDS and the block writes the finished heads itself: no partial result goes through memory,
 //             which pays once the pairs alone fill the chip (8B shapes, 2,048 keys a row: 32 rows 52.9 -> 49.1 us, 64
 //             rows 98.2 -> 91.6 us, 128 rows 196 -> 181 us; with 16 rows 30.2 -> 34.7 us.  Blocks of 8 waves were 2 %
@@ -739,16 +741,17 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(
       step(ra, kb);
     }
   };
+  // a range in pieces of no more keys than a wave keeps page ids for (one piece, but for rows far longer than the
+  // launch's parts were counted for, and for the one range a wave of DEC_WHOLE has of a long row)
+  const int piece = max(32, (62 * P) / 32 * 32);
   if constexpr (WHOLE) {
-    for (int r = wave; r * KW <= pos; r += NW) {
-      const int k_lo = max(r * KW, seen0), k_hi = min((r + 1) * KW, pos + 1);
-      if (k_lo < k_hi) run_range(k_lo, k_hi);
+    // ranges wave, wave + NW, ..: with the row's own ranges (the launch gave no length) that is one range a wave
+    for (int r = wave; base + r * KW <= pos; r += NW) {
+      const int k_lo = max(base + r * KW, seen0), k_hi = min(base + (r + 1) * KW, pos + 1);
+      for (int k = k_lo; k < k_hi; k += piece) run_range(k, min(k + piece, k_hi));
     }
   } else if (!empty) {
-    // a part in pieces of no more keys than a wave keeps page ids for (one piece, but for rows far longer than the
-    // launch's parts were counted for)
     const int k_lo = max(base + part * KW, seen0), k_hi = min(base + (part + 1) * KW, pos + 1);
-    const int piece = max(32, (62 * P) / 32 * 32);
     for (int k = k_lo; k < k_hi; k += piece) run_range(k, min(k + piece, k_hi));
   }
 
@@ -1018,8 +1021,8 @@ static bool last_fits(int G, int d, int n_parts) {
 //                                 (every call leaves them zero); `apc_attention_decode_last_fits` says whether it can;
 //   workspace, counters null      workspace: n_rows * H * n_parts * (d + 2) floats; a second kernel merges.
 // keys_per_part: the keys of a part (a multiple of 32; the parts are counted from position 0, and n_parts of them
-// must reach the longest row's position), or, with a workspace, 0: every row's own keys in n_parts equal ranges
-// (rows of any length).
+// must reach the longest row's position), or 0: every row's own keys in n_parts equal ranges (rows of any length;
+// without a workspace in 4, one a wave of the pair's block).
 // Calls that share counters or a workspace must not overlap (one stream).
 APC_EXPORT int apc_attention_decode_bf16(const void* q, int ldq, int q_off, void* out, int ldo, int n_rows, int H,
                                          int Hk, int d, const void* cache, int page_tokens, const int* block_table,
@@ -1030,7 +1033,6 @@ APC_EXPORT int apc_attention_decode_bf16(const void* q, int ldq, int q_off, void
   int e = check_common(q, ldq, q_off, cache, H, Hk, d, page_tokens);
   if (e) return e;
   if (keys_per_part < 0 || keys_per_part % 32 || max_blocks <= 0 || window < 0 || !out) return APC_ERR_BAD_ARG;
-  if (keys_per_part == 0 && !workspace) return APC_ERR_BAD_ARG;      // a block that takes a pair whole is told its ranges
   if (keys_per_part / page_tokens + 2 > 64) return APC_ERR_BAD_ARG;  // a wave keeps one page id per lane
   const int G = H / Hk, gtiles = (G + 15) / 16;
   if (Hk * gtiles > 65535 || H > 65535) return APC_ERR_BAD_ARG;
@@ -1049,7 +1051,8 @@ APC_EXPORT int apc_attention_decode_bf16(const void* q, int ldq, int q_off, void
   if (!workspace) {
     if (!whole_fits(G, d)) return APC_ERR_UNSUPPORTED;
     dim3 grid(n_rows, Hk * gtiles, 1);
-    DEC_BY_HEAD(DEC_WHOLE, grid, lds, 0, (float*)nullptr, (int*)nullptr);
+    // without a length of the ranges every row's own keys go in NW equal ranges, one a wave
+    DEC_BY_HEAD(DEC_WHOLE, grid, lds, NW, (float*)nullptr, (int*)nullptr);
     APC_LAUNCH_CHECK();
     return 0;
   }

@@ -417,10 +417,10 @@ int attention_bf16(Program& P, const Buf& q, const Buf& out, const ApcLayer& L, 
     const int n_parts = decode_parts(pairs, span);
     // (rows so short that one block's waves take a pair's ranges need no partial results either)
     if ((pairs >= P.tun.whole_min_pairs || n_parts <= WHOLE_WAVES) && apc_attention_decode_whole_fits(H, Hk, d)) {
-      const int kw = keys_per_wave_whole(span, page);
+      // no length of the ranges: every row's own keys, one range a wave of its block
       LAUNCH(P, "attention_decode_bf16 (whole)",
              apc_attention_decode_bf16(q.p, q.ld, 0, out.p, out.ld, n, H, Hk, d, E.kv, page, table, width,
-                                       s.positions, s.row_seg, rows, window, sc, kw, 0, nullptr, nullptr,
+                                       s.positions, s.row_seg, rows, window, sc, 0, 0, nullptr, nullptr,
                                        P.stream));
       return 1;
     }
@@ -704,9 +704,6 @@ APC_HOST_EXPORT const char* apc_host_timing_report(void* prog) {
 APC_HOST_EXPORT int apc_host_rule_tiled_k_split(int M, int N, int K) { return apc_rules::tiled_k_split(M, N, K); }
 APC_HOST_EXPORT int apc_host_rule_decode_parts(long long pairs, int span) {
   return apc_rules::decode_parts((long)pairs, span);
-}
-APC_HOST_EXPORT int apc_host_rule_keys_per_wave_whole(int max_context, int page_tokens) {
-  return apc_rules::keys_per_wave_whole(max_context, page_tokens);
 }
 APC_HOST_EXPORT int apc_host_rule_key_splits(int n_tiles, int n_heads, int keys, int window, int splits_max,
                                              int range_min) {

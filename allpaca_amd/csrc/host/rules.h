@@ -43,13 +43,6 @@ inline int decode_parts(long pairs, int span) {
   return (int)std::max(1L, std::min((long)WHOLE_WAVES * per_pair, cdiv(span, 64)));
 }
 
-inline int keys_per_wave_whole(int max_context, int page_tokens) {
-  int kw = (int)cdiv(max_context, WHOLE_WAVES);
-  kw = std::min(512, std::max(64, (int)cdiv(kw, 32) * 32));
-  while (kw > 32 && kw / page_tokens + 2 > 64) kw -= 32;
-  return kw;
-}
-
 // ranges of keys that the 128-row attention kernel cuts every tile of a step into; `keys`: of the longest prompt
 inline int key_splits(int n_tiles, int n_heads, int keys, int window, int splits_max, int range_min) {
   const long blocks = (long)n_tiles * n_heads;

@@ -69,7 +69,6 @@ _lib.SIGNATURES["host"].update({
     "apc_host_timing_report": [P],
     "apc_host_rule_tiled_k_split": [I, I, I],
     "apc_host_rule_decode_parts": [c_longlong, I],
-    "apc_host_rule_keys_per_wave_whole": [I, I],
     "apc_host_rule_key_splits": [I, I, I, I, I, I],
     # ---- the cache manager's books
     "apc_pool_new": [I], "apc_pool_free": [P], "apc_pool_alloc": [P], "apc_pool_give_back": [P, I],

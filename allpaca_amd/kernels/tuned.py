@@ -385,16 +385,6 @@ def _pair_counters(device: torch.device, pairs: int) -> torch.Tensor:
     return have[-1]
 
 
-def _keys_per_wave_whole(max_context: int, page_tokens: int) -> int:
-    """Keys of a range in the kernel that takes a (row, kv head) whole: the context spread over the block's waves,
-    64 to 512 keys, and no more pages than a wave keeps ids for (one per lane)."""
-    kw = -(-max_context // WHOLE_WAVES)
-    kw = min(512, max(64, -(-kw // 32) * 32))
-    while kw > 32 and kw // page_tokens + 2 > 64:
-        kw -= 32
-    return kw
-
-
 def attention_bf16(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
                    cache: torch.Tensor, page_tokens: int, block_table: torch.Tensor, step, window: int = 0,
                    scale: Optional[float] = None) -> bool:
@@ -441,11 +431,10 @@ def attention_bf16(q: torch.Tensor, q_off: int, out: torch.Tensor, n_heads: int,
         # (rows so short that one block's waves take a pair's ranges need no partial results either)
         if ((pairs >= WHOLE_MIN_PAIRS or n_parts <= WHOLE_WAVES)
                 and L.apc_attention_decode_whole_fits(n_heads, n_kv_heads, head_dim)):
-            kw = _keys_per_wave_whole(span, page_tokens)
             _lib.check(L.apc_attention_decode_bf16(
                 q.data_ptr(), ldq, q_off, out.data_ptr(), ldo, n, n_heads, n_kv_heads, head_dim, cache.data_ptr(),
                 page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
-                step.row_seg.data_ptr(), rows, int(window), sc, kw, 0, 0, 0, stream), "attention_decode_bf16 (whole)")
+                step.row_seg.data_ptr(), rows, int(window), sc, 0, 0, 0, 0, stream), "attention_decode_bf16 (whole)")
             return True
         kw = KEYS_PER_PART
         if LAST_BLOCK_MERGES and L.apc_attention_decode_last_fits(n_heads, n_kv_heads, head_dim, n_parts):

@@ -99,9 +99,6 @@ def test_the_executors_rules_are_the_wrappers_rules():
     for pairs in (1, 2, 3, 8, 12, 16, 24, 31, 64, 100, 255, 256, 257, 2040):
         for span in (1, 63, 64, 65, 2048, 2049, 8192, 32768, 131072):
             assert L.apc_host_rule_decode_parts(pairs, span) == tuned._decode_parts(pairs, span), (pairs, span)
-    for ctx in (1, 100, 256, 257, 2048, 2049, 5000, 131072):
-        for page in (8, 16, 24, 64, 128, 256):
-            assert L.apc_host_rule_keys_per_wave_whole(ctx, page) == tuned._keys_per_wave_whole(ctx, page), (ctx, page)
     for rows in (2, 100, 128, 129, 256, 512, 1024, 2048):
         for pos0 in (0, 500, 1920, 3584, 8000, 32640, 130000):
             for heads in (4, 8, 24, 32, 64):

@@ -709,6 +709,8 @@ def test_attention_long_context_decode_and_portion_over_history(decode_path):
     (16, 1, 256, 32, [500, 90], [1, 1], 0),                            # the meeting place does not fit: parts and merge
     (4, 2, 32, 16, [300, 200, 90, 2500], [1, 1, 1, 1], 100),
     (4, 4, 16, 16, [300, 200, 90, 1200], [1, 1, 1, 1], 1000),
+    (4, 2, 64, 8, [4000, 70, 1500, 1], [1, 1, 1, 1], 0),               # a wave's range in several pieces (pages of 8)
+    (4, 2, 32, 8, [4000, 300], [1, 1], 3000),
     (8, 2, 128, 16, [900, 133, 400], [1, 40, 1], 5),                    # decode rows beside a portion
 ])
 def test_attention_decode_by_one_block_a_row_and_kv_head(monkeypatch, H, Hk, d, P_, lens, rows, window):
